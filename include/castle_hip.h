@@ -1,0 +1,105 @@
+/* C ABI of libcastle_hip.so: the CASTLE (causal attention with lookahead keys) hot path
+ * for AMD MI355X (gfx950).  Plain pointers and sizes only; every tensor pointer is DEVICE
+ * memory, every call enqueues work on the HIP stream handed in (a hipStream_t passed as
+ * void*; NULL = the default stream) and returns without synchronising.
+ *
+ * Return value of the int entry points: 0 on success, negative on error
+ * (castle_error_string() gives the text).  Inputs are never modified.
+ *
+ * Reference interfaces replaced (paths inside lucidrains/lookahead-keys-attention):
+ *   castle_fwd          lookahead_keys_attention_triton.py:417-506  CastleAttentionFunction.forward
+ *                       (= castle_attention_triton, :605, called at lookahead_keys_attention.py:122);
+ *                       math of lookahead_keys_attention.py:132-164
+ *   castle_bwd          lookahead_keys_attention_triton.py:508-602  CastleAttentionFunction.backward
+ *   castle_decode_step  lookahead_keys_attention.py:166-203         the seq_len == 1 branch of Castle.forward
+ */
+#ifndef CASTLE_HIP_H_
+#define CASTLE_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CASTLE_ABI_VERSION 1
+
+/* element types of the tensors (accumulation is always fp32) */
+#define CASTLE_F32 0
+#define CASTLE_BF16 1
+#define CASTLE_F16 2
+
+/* error codes */
+#define CASTLE_OK 0
+#define CASTLE_ERR_DTYPE (-1)      /* unknown element type */
+#define CASTLE_ERR_SHAPE (-2)      /* unsupported head dim / size, or (dtype, d) does not fit the LDS */
+#define CASTLE_ERR_LAUNCH (-3)     /* HIP reported a launch / configuration error */
+#define CASTLE_ERR_WORKSPACE (-4)  /* workspace NULL, misaligned or too small */
+#define CASTLE_ERR_ARG (-5)        /* NULL pointer, misaligned pointer or stride */
+
+/* A (B, H, L, d) tensor view: element strides for b, h and l; the d axis has stride 1.
+ * ptr must be 16-byte aligned and every stride a multiple of 16 bytes / sizeof(element). */
+typedef struct castle_view4 {
+  void* ptr;
+  int64_t stride_b;
+  int64_t stride_h;
+  int64_t stride_l;
+} castle_view4;
+
+int castle_abi_version(void);
+const char* castle_error_string(int code);
+
+/* Bytes of device workspace castle_fwd needs.  The forward pass leaves there what the
+ * backward pass reads again (per-block T tiles, forward state snapshots, log-sum-exp);
+ * keep the buffer alive and unmodified until castle_bwd has run.  < 0 on error. */
+int64_t castle_fwd_workspace_bytes(int B, int H, int L, int d, int dtype);
+
+/* Parallel forward.  qc,kc,vc,qu,ku,vu: (B,H,L,d), unscaled, as handed to
+ * castle_attention_triton (lookahead_keys_attention.py:122).  out: (B,H,L,d) view that is
+ * written (any strides, e.g. those of a (B,L,H,d) buffer).  U: optional (NULL, or a view
+ * with ptr == NULL, to skip) final lookahead keys for the decode cache
+ * (lookahead_keys_attention.py:161-164).  d in {16,32,64,128}; fp32 needs d <= 64. */
+int castle_fwd(const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
+               const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
+               int B, int H, int L, int d, int dtype, float scale,
+               const castle_view4* out, const castle_view4* U,
+               void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Bytes of extra device workspace castle_bwd needs (reverse state snapshots, delta). */
+int64_t castle_bwd_workspace_bytes(int B, int H, int L, int d, int dtype);
+
+/* Parallel backward.  Same operands as castle_fwd plus the forward output `out`, the
+ * upstream gradient `dout` and the forward workspace as castle_fwd left it.  Writes the six
+ * gradients (all (B,H,L,d) views; every element is written, nothing is accumulated).
+ * U carries no gradient (lookahead_keys_attention_triton.py:513-515). */
+int castle_bwd(const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
+               const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
+               const castle_view4* out, const castle_view4* dout,
+               int B, int H, int L, int d, int dtype, float scale,
+               const castle_view4* dqc, const castle_view4* dkc, const castle_view4* dvc,
+               const castle_view4* dqu, const castle_view4* dku, const castle_view4* dvu,
+               const void* fwd_workspace, int64_t fwd_workspace_bytes,
+               void* bwd_workspace, int64_t bwd_workspace_bytes, void* stream);
+
+/* Bytes of device workspace castle_decode_step needs for a cache of up to t_max rows. */
+int64_t castle_decode_workspace_bytes(int B, int H, int d, int t_max);
+
+/* One cached decode step (lookahead_keys_attention.py:166-203), in place.
+ * U, qu_cache, kc_cache, vc_cache: (B,H,capacity,d) buffers holding t valid rows,
+ * capacity > t.  The call updates U rows 0..t-1 in place (U_k += sigmoid(s qu_k.ku) vu),
+ * writes row t of all four (U_t = 0, qu, kc, vc of the new token) and writes
+ * out (B,H,1,d) = softmax_k(s qc.kc_k - silu(s qc.U_k)) vc_k over k = 0..t.
+ * qc..vu: the new token's (B,H,1,d) operands (stride_l unused).  After the call the cache
+ * holds t+1 rows.  d in {16,32,64,128}. */
+int castle_decode_step(const castle_view4* U, const castle_view4* qu_cache,
+                       const castle_view4* kc_cache, const castle_view4* vc_cache, int t,
+                       const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
+                       const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
+                       int B, int H, int d, int dtype, float scale,
+                       const castle_view4* out,
+                       void* workspace, int64_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CASTLE_HIP_H_ */

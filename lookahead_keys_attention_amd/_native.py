@@ -1,0 +1,124 @@
+"""ctypes binding of libcastle_hip.so (C ABI in include/castle_hip.h).
+
+The library is looked up next to this file only.  Nothing here falls back to another
+implementation: if the library is missing or a call fails, a RuntimeError is raised.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libcastle_hip.so")
+
+ABI_VERSION = 1
+DTYPE_CODES = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
+SUPPORTED_HEAD_DIMS = (16, 32, 64, 128)
+
+EXPORTED_SYMBOLS = (
+    "castle_abi_version",
+    "castle_error_string",
+    "castle_fwd_workspace_bytes",
+    "castle_fwd",
+    "castle_bwd_workspace_bytes",
+    "castle_bwd",
+    "castle_decode_workspace_bytes",
+    "castle_decode_step",
+)
+
+
+class View4(ctypes.Structure):
+    """struct castle_view4"""
+
+    _fields_ = [
+        ("ptr", ctypes.c_void_p),
+        ("stride_b", ctypes.c_int64),
+        ("stride_h", ctypes.c_int64),
+        ("stride_l", ctypes.c_int64),
+    ]
+
+
+_VP = ctypes.POINTER(View4)
+_lib = None
+_lock = threading.Lock()
+
+
+def _declare(lib):
+    i, i64, f, vp = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
+    lib.castle_abi_version.restype = i
+    lib.castle_abi_version.argtypes = []
+    lib.castle_error_string.restype = ctypes.c_char_p
+    lib.castle_error_string.argtypes = [i]
+    lib.castle_fwd_workspace_bytes.restype = i64
+    lib.castle_fwd_workspace_bytes.argtypes = [i, i, i, i, i]
+    lib.castle_bwd_workspace_bytes.restype = i64
+    lib.castle_bwd_workspace_bytes.argtypes = [i, i, i, i, i]
+    lib.castle_decode_workspace_bytes.restype = i64
+    lib.castle_decode_workspace_bytes.argtypes = [i, i, i, i]
+    lib.castle_fwd.restype = i
+    lib.castle_fwd.argtypes = [_VP] * 6 + [i, i, i, i, i, f, _VP, _VP, vp, i64, vp]
+    lib.castle_bwd.restype = i
+    lib.castle_bwd.argtypes = [_VP] * 8 + [i, i, i, i, i, f] + [_VP] * 6 + [vp, i64, vp, i64, vp]
+    lib.castle_decode_step.restype = i
+    lib.castle_decode_step.argtypes = [_VP] * 4 + [i] + [_VP] * 6 + [i, i, i, i, f, _VP, vp, i64, vp]
+
+
+def lib():
+    """The loaded library (loads it on first use; raises if it has not been built)."""
+    global _lib
+    if _lib is None:
+        with _lock:
+            if _lib is None:
+                if not os.path.exists(LIB_PATH):
+                    raise RuntimeError(
+                        f"{LIB_PATH} not found: build the HIP kernels first "
+                        "(python -m lookahead_keys_attention_amd.build)"
+                    )
+                handle = ctypes.CDLL(LIB_PATH)
+                _declare(handle)
+                got = handle.castle_abi_version()
+                if got != ABI_VERSION:
+                    raise RuntimeError(f"libcastle_hip.so has ABI {got}, this package needs {ABI_VERSION}")
+                _lib = handle
+    return _lib
+
+
+def is_built() -> bool:
+    return os.path.exists(LIB_PATH)
+
+
+def check(code: int, what: str):
+    if code < 0:
+        msg = lib().castle_error_string(int(code)).decode()
+        raise RuntimeError(f"{what} failed: {msg} (code {code})")
+    return code
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return DTYPE_CODES[dtype]
+    except KeyError:
+        raise TypeError(f"castle HIP kernels support float32, bfloat16 and float16, not {dtype}") from None
+
+
+def view4(t: torch.Tensor) -> View4:
+    """castle_view4 of a (B, H, L, d) tensor with unit stride along d."""
+    assert t.dim() == 4 and (t.stride(3) == 1 or t.shape[3] == 1)
+    return View4(t.data_ptr(), t.stride(0), t.stride(1), t.stride(2))
+
+
+def vector_ok(t: torch.Tensor) -> bool:
+    """True if the kernels can read `t` in place: unit stride along d, 16-byte aligned rows."""
+    q = 16 // t.element_size()
+    return (
+        t.stride(3) == 1
+        and t.data_ptr() % 16 == 0
+        and all(t.stride(i) % q == 0 for i in range(3))
+    )
+
+
+def stream_ptr(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream

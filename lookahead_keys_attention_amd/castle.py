@@ -1,0 +1,225 @@
+"""`Castle`: causal attention with lookahead keys, host side of the MI355X kernels.
+
+Same constructor, forward signature, state_dict keys and cache layout as the reference
+module (lookahead_keys_attention.py:41-214), so it can replace it where the reference's
+`use_triton` path is used:
+
+    Castle(dim, heads=8, dim_head=64, use_triton=None, rotary_emb=False, prenorm=False)
+    forward(x, cache=None, return_next_cache=None) -> out | (out, Cache)
+
+`use_triton` keeps its name for drop-in compatibility and selects the native kernels:
+  None  -> native HIP kernels when a GPU is present (reference: lookahead_keys_attention.py:58)
+  True  -> native HIP kernels; anything that prevents them raises
+  False -> the dense PyTorch formulation (the reference's own non-Triton path), any device
+On the native path both the parallel pass (seq_len > 1) and the cached single-token step
+run in HIP; nothing silently falls back.
+
+Decode cache.  `Cache(U, qu_cache, kc_cache, vc_cache)` holds four (B, H, n, d) tensors as in
+the reference (lookahead_keys_attention.py:26).  Caches made by the native path are views into
+preallocated capacity buffers and the step updates them IN PLACE (U rows are advanced, one row
+is appended); a cache handed to a native decode step is consumed by it and must not be reused.
+Plain 4-tuples of tensors are accepted too (they are copied into a fresh buffer first).
+"""
+from __future__ import annotations
+
+from collections import namedtuple
+
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+from . import ops
+from . import _native
+
+_CacheFields = namedtuple("Cache", ("U", "qu_cache", "kc_cache", "vc_cache"))
+
+
+class Cache(_CacheFields):
+    """Four (B, H, n, d) tensors; field names as in the reference (lookahead_keys_attention.py:26)."""
+
+    _store = None   # set on caches that live in a native capacity buffer
+
+
+class _CacheStore:
+    """Capacity buffers behind a native cache: four (B, H, capacity, d) tensors and a row count."""
+
+    def __init__(self, B, H, d, capacity, dtype, device):
+        self.buffers = tuple(torch.empty((B, H, capacity, d), dtype=dtype, device=device) for _ in range(4))
+        self.capacity = capacity
+        self.length = 0
+        self.workspace = ops.decode_workspace(B, H, d, device)
+
+    def as_cache(self) -> Cache:
+        n = self.length
+        cache = Cache(*(buf[:, :, :n] for buf in self.buffers))
+        cache._store = self
+        return cache
+
+    def grown(self, min_capacity):
+        B, H, _, d = self.buffers[0].shape
+        new = _CacheStore(B, H, d, max(min_capacity, 2 * self.capacity), self.buffers[0].dtype, self.buffers[0].device)
+        for dst, src in zip(new.buffers, self.buffers):
+            dst[:, :, : self.length].copy_(src[:, :, : self.length])
+        new.length = self.length
+        return new
+
+
+def _reserve_rows(n: int) -> int:
+    """Capacity for a cache that currently needs n rows: room for max(n/2, 1024) more steps."""
+    return n + max(n // 2, 1024)
+
+
+def rotate_half_pairs(t, positions, theta=10000.0):
+    """Rotary position embedding over interleaved pairs (x0,x1),(x2,x3),.. of the last axis.
+
+    t: (..., n, d); positions: (n,) absolute positions.  Frequencies theta^(-2i/d), the usual
+    RoPE.  The reference delegates this to a third-party package (lookahead_keys_attention.py:73,112)
+    that is not available for comparison, so exact agreement with it is unverified; the
+    properties the reference tests (parallel == cached sequential, causality) hold."""
+    d = t.shape[-1]
+    inv = theta ** (-torch.arange(0, d, 2, device=t.device, dtype=torch.float32) / d)
+    ang = positions.to(torch.float32)[:, None] * inv[None, :]
+    cos, sin = ang.cos().repeat_interleave(2, -1), ang.sin().repeat_interleave(2, -1)
+    x = t.float()
+    pairs = x.unflatten(-1, (d // 2, 2))
+    rot = torch.stack((-pairs[..., 1], pairs[..., 0]), dim=-1).flatten(-2)
+    return (x * cos + rot * sin).to(t.dtype)
+
+
+class Castle(nn.Module):
+    def __init__(self, dim, heads=8, dim_head=64, use_triton=None, rotary_emb=False, prenorm=False):
+        super().__init__()
+        self.dim, self.heads, self.dim_head = dim, heads, dim_head
+        if use_triton is None:
+            use_triton = torch.cuda.is_available()
+        if use_triton and not _native.is_built():
+            raise AssertionError(
+                "native kernels requested but libcastle_hip.so is not built "
+                "(python -m lookahead_keys_attention_amd.build), or pass use_triton=False"
+            )
+        self.use_triton = bool(use_triton)
+        self.scale = dim_head ** -0.5
+        self.norm = nn.RMSNorm(dim) if prenorm else nn.Identity()
+        self.rotary_emb = bool(rotary_emb)
+        inner = heads * dim_head
+        self.to_all_qkv = nn.Linear(dim, inner * 6, bias=False)
+        self.combine_heads = nn.Linear(inner, dim, bias=False)
+
+    # -- helpers ------------------------------------------------------------
+    def _split(self, proj):
+        B, n, _ = proj.shape
+        six = proj.view(B, n, 6, self.heads, self.dim_head).permute(2, 0, 3, 1, 4)
+        return six.unbind(0)   # qu, ku, vu, qc, kc, vc : (B, H, n, d) views
+
+    def _rotate(self, tensors, offset, n, device):
+        pos = torch.arange(offset, offset + n, device=device)
+        return tuple(rotate_half_pairs(t, pos) for t in tensors)
+
+    # -- forward ------------------------------------------------------------
+    def forward(self, x, cache=None, return_next_cache=None):
+        n = x.shape[1]
+        single = n == 1
+        if return_next_cache is None:
+            return_next_cache = single
+        proj = self.to_all_qkv(self.norm(x))
+        native = self.use_triton
+        if native and not x.is_cuda:
+            raise RuntimeError("Castle(use_triton=True) runs HIP kernels and needs GPU tensors; "
+                               "construct with use_triton=False for the PyTorch formulation")
+        if not single:
+            assert cache is None, "must be inferencing single tokens if receiving cache"
+            merged, next_cache = (self._parallel_native if native else self._parallel_dense)(proj, return_next_cache)
+        else:
+            merged, next_cache = (self._step_native if native else self._step_dense)(proj, cache)
+        y = self.combine_heads(merged)
+        return (y, next_cache) if return_next_cache else y
+
+    # -- native HIP paths ---------------------------------------------------
+    def _parallel_native(self, proj, want_cache):
+        B, n, _ = proj.shape
+        H, d = self.heads, self.dim_head
+        store = None
+        if want_cache:
+            store = _CacheStore(B, H, d, _reserve_rows(n), proj.dtype, proj.device)
+        if not self.rotary_emb:
+            U_view = store.buffers[0][:, :, :n] if want_cache else None
+            res = ops.castle_attention_packed(proj, H, self.scale, want_cache, U_view)
+            merged = res[0] if want_cache else res
+            qu, _, _, _, kc, vc = self._split(proj)
+        else:
+            qu, ku, vu, qc, kc, vc = self._split(proj)
+            qc, kc, qu, ku, vu = self._rotate((qc, kc, qu, ku, vu), 0, n, proj.device)
+            res = ops.castle_attention_hip(qc, kc, vc, qu, ku, vu, self.scale, want_cache)
+            o = res[0] if want_cache else res
+            merged = o.permute(0, 2, 1, 3).reshape(B, n, H * d)
+            if want_cache:
+                store.buffers[0][:, :, :n].copy_(res[1])
+        if not want_cache:
+            return merged, None
+        with torch.no_grad():
+            for buf, src in zip(store.buffers[1:], (qu, kc, vc)):
+                buf[:, :, :n].copy_(src)
+        store.length = n
+        return merged, store.as_cache()
+
+    def _step_native(self, proj, cache):
+        B = proj.shape[0]
+        H, d = self.heads, self.dim_head
+        qu, ku, vu, qc, kc, vc = self._split(proj)
+        store = getattr(cache, "_store", None) if cache is not None else None
+        if cache is None:
+            store = _CacheStore(B, H, d, _reserve_rows(1), proj.dtype, proj.device)
+        elif store is None:
+            t = cache[0].shape[-2]
+            store = _CacheStore(B, H, d, _reserve_rows(t + 1), proj.dtype, proj.device)
+            for buf, src in zip(store.buffers, cache):
+                buf[:, :, :t].copy_(src)
+            store.length = t
+        elif store.length != cache[0].shape[-2]:
+            raise RuntimeError("this cache was already advanced by a later decode step; the native "
+                               "decode updates its cache in place, so a cache can be used once")
+        t = store.length
+        if self.rotary_emb:
+            qc, kc, qu, ku, vu = self._rotate((qc, kc, qu, ku, vu), t, 1, proj.device)
+        if t + 1 > store.capacity:
+            store = store.grown(_reserve_rows(t + 1))
+        out = torch.empty((B, 1, H, d), dtype=proj.dtype, device=proj.device)
+        ops.castle_decode_step_hip(*store.buffers, t, qc, kc, vc, qu, ku, vu, self.scale,
+                                   out.permute(0, 2, 1, 3), store.workspace)
+        store.length = t + 1
+        return out.view(B, 1, H * d), store.as_cache()
+
+    # -- dense PyTorch formulation (use_triton=False) -------------------------
+    def _parallel_dense(self, proj, want_cache):
+        B, n, _ = proj.shape
+        qu, ku, vu, qc, kc, vc = self._split(proj)
+        if self.rotary_emb:
+            qc, kc, qu, ku, vu = self._rotate((qc, kc, qu, ku, vu), 0, n, proj.device)
+        s = self.scale
+        future = torch.ones(n, n, dtype=torch.bool, device=proj.device).triu(1)
+        T = ((qc * s) @ vu.mT).masked_fill(future, 0.0)
+        A = torch.sigmoid((qu * s) @ ku.mT).masked_fill(~future, 0.0)
+        S = (qc * s) @ kc.mT - F.silu(T @ A.mT)
+        P = S.masked_fill(future, -torch.finfo(S.dtype).max).softmax(dim=-1)
+        o = P @ vc
+        merged = o.permute(0, 2, 1, 3).reshape(B, n, -1)
+        return merged, (Cache(A @ vu, qu, kc, vc) if want_cache else None)
+
+    def _step_dense(self, proj, cache):
+        B = proj.shape[0]
+        qu, ku, vu, qc, kc, vc = self._split(proj)
+        if cache is None:
+            empty = qu[..., :0, :]
+            cache = (empty,) * 4
+        U, qu_hist, kc_hist, vc_hist = cache
+        t = kc_hist.shape[-2]
+        if self.rotary_emb:
+            qc, kc, qu, ku, vu = self._rotate((qc, kc, qu, ku, vu), t, 1, proj.device)
+        s = self.scale
+        gate = torch.sigmoid((qu_hist * s) @ ku.mT)
+        U = torch.cat((U + gate * vu, torch.zeros_like(qu)), dim=-2)
+        kc_all, vc_all = torch.cat((kc_hist, kc), dim=-2), torch.cat((vc_hist, vc), dim=-2)
+        q = qc * s
+        P = (q @ kc_all.mT - F.silu(q @ U.mT)).softmax(dim=-1)
+        merged = (P @ vc_all).permute(0, 2, 1, 3).reshape(B, 1, -1)
+        return merged, Cache(U, torch.cat((qu_hist, qu), dim=-2), kc_all, vc_all)

@@ -1,0 +1,222 @@
+// extern "C" surface of libcastle_hip.so (declared in include/castle_hip.h): argument
+// validation, workspace carving and dispatch to the kernel launchers.  No torch types.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/castle_hip.h"
+#include "castle_params.h"
+#include "castle_tiles.h"
+
+namespace castle {
+int launch_fwd(const FwdArgs& a, int dtype, hipStream_t stream);
+int launch_bwd(const BwdArgs& a, int dtype, hipStream_t stream);
+int launch_decode(const DecodeArgs& a, int dtype, hipStream_t stream);
+int decode_pick_splits(int BH, int t);
+}  // namespace castle
+
+namespace {
+
+using castle::kNB;
+
+int elem_size(int dtype) {
+  switch (dtype) {
+    case CASTLE_F32: return 4;
+    case CASTLE_BF16:
+    case CASTLE_F16: return 2;
+    default: return 0;
+  }
+}
+
+bool head_dim_ok(int d) { return d == 16 || d == 32 || d == 64 || d == 128; }
+
+int64_t align_up(int64_t x, int64_t a) { return (x + a - 1) / a * a; }
+
+struct Geometry {
+  int Lp, nblk;
+  int64_t lse_bytes, tblk_bytes, snap_bytes;
+  int64_t off_lse, off_t, off_tt, off_snap, total;
+};
+
+Geometry geometry(int B, int H, int L, int d, int es) {
+  Geometry g;
+  g.Lp = (int)align_up(L, 128);
+  g.nblk = g.Lp / kNB;
+  const int64_t BH = (int64_t)B * H;
+  g.lse_bytes = align_up(BH * g.Lp * 4, 256);
+  g.tblk_bytes = align_up(BH * g.Lp * kNB * es, 256);
+  g.snap_bytes = align_up(BH * castle::snap_rows(g.nblk) * d * es, 256);
+  g.off_lse = 0;
+  g.off_t = g.off_lse + g.lse_bytes;
+  g.off_tt = g.off_t + g.tblk_bytes;
+  g.off_snap = g.off_tt + g.tblk_bytes;
+  g.total = g.off_snap + g.snap_bytes;
+  return g;
+}
+
+// pointer and strides must allow 16-byte vector access along d
+bool view_ok(const castle_view4* v, int es, bool need_l) {
+  if (v == nullptr || v->ptr == nullptr) return false;
+  const int64_t q = 16 / es;
+  if (reinterpret_cast<uintptr_t>(v->ptr) % 16 != 0) return false;
+  if (v->stride_b % q != 0 || v->stride_h % q != 0) return false;
+  if (need_l && v->stride_l % q != 0) return false;
+  return true;
+}
+
+castle::View4 to_view(const castle_view4* v) {
+  castle::View4 r;
+  if (v == nullptr) {
+    r.ptr = nullptr; r.sb = r.sh = r.sl = 0;
+  } else {
+    r.ptr = v->ptr; r.sb = v->stride_b; r.sh = v->stride_h; r.sl = v->stride_l;
+  }
+  return r;
+}
+
+int check_core(int B, int H, int L, int d, int dtype) {
+  if (elem_size(dtype) == 0) return CASTLE_ERR_DTYPE;
+  if (B <= 0 || H <= 0 || L <= 0 || !head_dim_ok(d)) return CASTLE_ERR_SHAPE;
+  if ((int64_t)B * H > 65535) return CASTLE_ERR_SHAPE;   // grid.y
+  if (dtype == CASTLE_F32 && d > 64) return CASTLE_ERR_SHAPE;
+  return CASTLE_OK;
+}
+
+castle::FwdWorkspace carve(void* base, const Geometry& g) {
+  char* p = static_cast<char*>(base);
+  castle::FwdWorkspace w;
+  w.lse = reinterpret_cast<float*>(p + g.off_lse);
+  w.t_blk = p + g.off_t;
+  w.tt_blk = p + g.off_tt;
+  w.usnap = p + g.off_snap;
+  return w;
+}
+
+}  // namespace
+
+extern "C" {
+
+int castle_abi_version(void) { return CASTLE_ABI_VERSION; }
+
+const char* castle_error_string(int code) {
+  switch (code) {
+    case CASTLE_OK: return "ok";
+    case CASTLE_ERR_DTYPE: return "unknown element type";
+    case CASTLE_ERR_SHAPE: return "unsupported shape (head dim must be 16/32/64/128, fp32 needs d <= 64, B*H <= 65535)";
+    case CASTLE_ERR_LAUNCH: return "HIP launch or configuration error";
+    case CASTLE_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
+    case CASTLE_ERR_ARG: return "NULL or misaligned tensor view";
+    default: return "unknown error";
+  }
+}
+
+int64_t castle_fwd_workspace_bytes(int B, int H, int L, int d, int dtype) {
+  const int rc = check_core(B, H, L, d, dtype);
+  if (rc != CASTLE_OK) return rc;
+  return geometry(B, H, L, d, elem_size(dtype)).total;
+}
+
+int castle_fwd(const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
+               const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
+               int B, int H, int L, int d, int dtype, float scale,
+               const castle_view4* out, const castle_view4* U,
+               void* workspace, int64_t workspace_bytes, void* stream) {
+  int rc = check_core(B, H, L, d, dtype);
+  if (rc != CASTLE_OK) return rc;
+  const int es = elem_size(dtype);
+  const castle_view4* in[] = {qc, kc, vc, qu, ku, vu, out};
+  for (const castle_view4* v : in)
+    if (!view_ok(v, es, true)) return CASTLE_ERR_ARG;
+  const bool want_U = U != nullptr && U->ptr != nullptr;
+  if (want_U && !view_ok(U, es, true)) return CASTLE_ERR_ARG;
+  const Geometry g = geometry(B, H, L, d, es);
+  if (workspace == nullptr || reinterpret_cast<uintptr_t>(workspace) % 256 != 0 || workspace_bytes < g.total)
+    return CASTLE_ERR_WORKSPACE;
+
+  castle::FwdArgs a;
+  a.s.B = B; a.s.H = H; a.s.L = L; a.s.d = d; a.s.Lp = g.Lp; a.s.nblk = g.nblk; a.s.scale = scale;
+  a.qc = to_view(qc); a.kc = to_view(kc); a.vc = to_view(vc);
+  a.qu = to_view(qu); a.ku = to_view(ku); a.vu = to_view(vu);
+  a.out = to_view(out);
+  a.U = to_view(want_U ? U : nullptr);
+  a.ws = carve(workspace, g);
+  return castle::launch_fwd(a, dtype, static_cast<hipStream_t>(stream));
+}
+
+int64_t castle_bwd_workspace_bytes(int B, int H, int L, int d, int dtype) {
+  const int rc = check_core(B, H, L, d, dtype);
+  if (rc != CASTLE_OK) return rc;
+  const Geometry g = geometry(B, H, L, d, elem_size(dtype));
+  return g.snap_bytes + g.lse_bytes;   // reverse-state snapshots + delta
+}
+
+int castle_bwd(const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
+               const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
+               const castle_view4* out, const castle_view4* dout,
+               int B, int H, int L, int d, int dtype, float scale,
+               const castle_view4* dqc, const castle_view4* dkc, const castle_view4* dvc,
+               const castle_view4* dqu, const castle_view4* dku, const castle_view4* dvu,
+               const void* fwd_workspace, int64_t fwd_workspace_bytes,
+               void* bwd_workspace, int64_t bwd_workspace_bytes, void* stream) {
+  int rc = check_core(B, H, L, d, dtype);
+  if (rc != CASTLE_OK) return rc;
+  const int es = elem_size(dtype);
+  const castle_view4* in[] = {qc, kc, vc, qu, ku, vu, out, dout, dqc, dkc, dvc, dqu, dku, dvu};
+  for (const castle_view4* v : in)
+    if (!view_ok(v, es, true)) return CASTLE_ERR_ARG;
+  const Geometry g = geometry(B, H, L, d, es);
+  if (fwd_workspace == nullptr || reinterpret_cast<uintptr_t>(fwd_workspace) % 256 != 0 || fwd_workspace_bytes < g.total)
+    return CASTLE_ERR_WORKSPACE;
+  if (bwd_workspace == nullptr || reinterpret_cast<uintptr_t>(bwd_workspace) % 256 != 0 ||
+      bwd_workspace_bytes < g.snap_bytes + g.lse_bytes)
+    return CASTLE_ERR_WORKSPACE;
+
+  castle::BwdArgs a;
+  a.s.B = B; a.s.H = H; a.s.L = L; a.s.d = d; a.s.Lp = g.Lp; a.s.nblk = g.nblk; a.s.scale = scale;
+  a.qc = to_view(qc); a.kc = to_view(kc); a.vc = to_view(vc);
+  a.qu = to_view(qu); a.ku = to_view(ku); a.vu = to_view(vu);
+  a.out = to_view(out); a.dout = to_view(dout);
+  a.dqc = to_view(dqc); a.dkc = to_view(dkc); a.dvc = to_view(dvc);
+  a.dqu = to_view(dqu); a.dku = to_view(dku); a.dvu = to_view(dvu);
+  a.ws = carve(const_cast<void*>(fwd_workspace), g);
+  a.gsnap = bwd_workspace;
+  a.delta = reinterpret_cast<float*>(static_cast<char*>(bwd_workspace) + g.snap_bytes);
+  return castle::launch_bwd(a, dtype, static_cast<hipStream_t>(stream));
+}
+
+int64_t castle_decode_workspace_bytes(int B, int H, int d, int t_max) {
+  if (B <= 0 || H <= 0 || !head_dim_ok(d) || t_max < 0) return CASTLE_ERR_SHAPE;
+  return align_up((int64_t)B * H * 64 * (d + 2) * 4, 256);
+}
+
+int castle_decode_step(const castle_view4* U, const castle_view4* qu_cache,
+                       const castle_view4* kc_cache, const castle_view4* vc_cache, int t,
+                       const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
+                       const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
+                       int B, int H, int d, int dtype, float scale,
+                       const castle_view4* out,
+                       void* workspace, int64_t workspace_bytes, void* stream) {
+  const int es = elem_size(dtype);
+  if (es == 0) return CASTLE_ERR_DTYPE;
+  if (B <= 0 || H <= 0 || t < 0 || !head_dim_ok(d) || (int64_t)B * H > 65535) return CASTLE_ERR_SHAPE;
+  const castle_view4* caches[] = {U, qu_cache, kc_cache, vc_cache};
+  for (const castle_view4* v : caches)
+    if (!view_ok(v, es, true)) return CASTLE_ERR_ARG;
+  const castle_view4* tok[] = {qc, kc, vc, qu, ku, vu, out};
+  for (const castle_view4* v : tok)
+    if (!view_ok(v, es, false)) return CASTLE_ERR_ARG;
+  if (workspace == nullptr || reinterpret_cast<uintptr_t>(workspace) % 256 != 0 ||
+      workspace_bytes < castle_decode_workspace_bytes(B, H, d, t))
+    return CASTLE_ERR_WORKSPACE;
+
+  castle::DecodeArgs a;
+  a.B = B; a.H = H; a.d = d; a.t = t; a.scale = scale;
+  a.splits = castle::decode_pick_splits(B * H, t);
+  a.U = to_view(U); a.qu_cache = to_view(qu_cache); a.kc_cache = to_view(kc_cache); a.vc_cache = to_view(vc_cache);
+  a.qc = to_view(qc); a.kc = to_view(kc); a.vc = to_view(vc);
+  a.qu = to_view(qu); a.ku = to_view(ku); a.vu = to_view(vu);
+  a.out = to_view(out);
+  a.part = static_cast<float*>(workspace);
+  return castle::launch_decode(a, dtype, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,218 @@
+// CASTLE cached decode step for gfx950: one streaming pass over the cache.
+//
+// Reference semantics: lookahead_keys_attention.py:166-203.  For every cached row k < t
+//     a_k  = sigmoid(s qu_k . ku_t)            U_k <- U_k + a_k vu_t      (in place)
+//     x_k  = s qc_t . kc_k - silu(s qc_t . U_k)
+// and for the appended row t:  U_t = 0,  x_t = s qc_t . kc_t;  out = softmax(x) V.
+// The pass is bandwidth bound: each cached element of qu, U, kc, vc is read once and U is
+// written once (5 * t * d elements per head and step).  The t rows of one (b, h) are split
+// over `splits` workgroups that each keep an online-softmax partial (acc, m, l) in fp32;
+// decode_finish_kernel merges the partials, folds in row t and appends the new rows.
+#include "castle_tiles.h"
+#include "castle_params.h"
+
+namespace castle {
+
+template <typename T> __device__ __forceinline__ T* view_row(const View4& v, int b, int h, int64_t row) {
+  return reinterpret_cast<T*>(v.ptr) + (int64_t)b * v.sb + (int64_t)h * v.sh + row * v.sl;
+}
+
+template <typename T, int N> __device__ __forceinline__ void load_f32(const T* p, float (&dst)[N]) {
+  typedef vec<T, N> vt;
+  vt x = *reinterpret_cast<const vt*>(p);
+#pragma unroll
+  for (int e = 0; e < N; ++e) dst[e] = (float)x[e];
+}
+
+template <int LPR> __device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+  for (int o = 1; o < LPR; o <<= 1) v += __shfl_xor(v, o);
+  return v;
+}
+
+// One workgroup = 4 waves; a group of LPR = d / V lanes owns one cache row per iteration.
+template <typename T, int HD>
+__global__ __launch_bounds__(kThreads) void decode_stream_kernel(DecodeArgs a) {
+  constexpr int V = elem_traits<T>::vec16;   // elements per 16-byte lane load
+  constexpr int LPR = HD / V;                // lanes per row
+  constexpr int RPI = kThreads / LPR;        // rows per workgroup iteration
+  typedef vec<T, V> vt;
+  __shared__ float s_acc[kThreads / LPR][HD + 2];
+
+  const int split = blockIdx.x, bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
+  const int tid = threadIdx.x;
+  const int grp = tid / LPR, sub = tid % LPR;
+  const float c0 = a.scale, c1 = a.scale * kLog2e;
+
+  // rows of this workgroup: [r0, r1), whole iterations of RPI rows
+  const int per = ((a.t + a.splits - 1) / a.splits + RPI - 1) / RPI * RPI;
+  const int r0 = split * per;
+  const int r1 = min(a.t, r0 + per);
+
+  float ku[V], vu[V], qc[V];
+  load_f32<T, V>(view_row<T>(a.ku, b, h, 0) + sub * V, ku);
+  load_f32<T, V>(view_row<T>(a.vu, b, h, 0) + sub * V, vu);
+  load_f32<T, V>(view_row<T>(a.qc, b, h, 0) + sub * V, qc);
+
+  float acc[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) acc[e] = 0.f;
+  float m = -INFINITY, l = 0.f;
+
+  for (int base = r0; base < r1; base += RPI) {
+    const int k = base + grp;
+    if (k < r1) {
+      float quk[V], uk[V], kck[V], vck[V];
+      T* urow = view_row<T>(a.U, b, h, k) + sub * V;
+      load_f32<T, V>(view_row<T>(a.qu_cache, b, h, k) + sub * V, quk);
+      load_f32<T, V>(urow, uk);
+      load_f32<T, V>(view_row<T>(a.kc_cache, b, h, k) + sub * V, kck);
+      load_f32<T, V>(view_row<T>(a.vc_cache, b, h, k) + sub * V, vck);
+      float dg = 0.f;
+#pragma unroll
+      for (int e = 0; e < V; ++e) dg = __builtin_fmaf(quk[e], ku[e], dg);
+      dg = group_sum<LPR>(dg);
+      const float gate = sigmoid_l2(dg * c1);
+      vt unew;
+#pragma unroll
+      for (int e = 0; e < V; ++e) unew[e] = (T)__builtin_fmaf(gate, vu[e], uk[e]);
+      *reinterpret_cast<vt*>(urow) = unew;
+      float dsu = 0.f, dsc = 0.f;
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        dsu = __builtin_fmaf(qc[e], (float)unew[e], dsu);   // the stored (rounded) lookahead key
+        dsc = __builtin_fmaf(qc[e], kck[e], dsc);
+      }
+      dsu = group_sum<LPR>(dsu);
+      dsc = group_sum<LPR>(dsc);
+      const float x = (dsc - dsu * sigmoid_l2(dsu * c1)) * c1;   // score in log2 units
+      const float mn = fmaxf(m, x);
+      const float al = fast_exp2(m - mn), p = fast_exp2(x - mn);
+      l = l * al + p;
+#pragma unroll
+      for (int e = 0; e < V; ++e) acc[e] = __builtin_fmaf(p, vck[e], acc[e] * al);
+      m = mn;
+    }
+  }
+  (void)c0;
+  // merge the row groups of the workgroup
+#pragma unroll
+  for (int e = 0; e < V; ++e) s_acc[grp][sub * V + e] = acc[e];
+  if (sub == 0) { s_acc[grp][HD] = m; s_acc[grp][HD + 1] = l; }
+  __syncthreads();
+  float* part = a.part + ((int64_t)bh * a.splits + split) * (HD + 2);
+  if (tid < HD) {
+    float M = -INFINITY;
+    for (int r = 0; r < RPI; ++r) M = fmaxf(M, s_acc[r][HD]);
+    float out = 0.f, lsum = 0.f;
+    for (int r = 0; r < RPI; ++r) {
+      const float w = (s_acc[r][HD] == -INFINITY) ? 0.f : fast_exp2(s_acc[r][HD] - M);
+      out = __builtin_fmaf(w, s_acc[r][tid], out);
+      lsum = __builtin_fmaf(w, s_acc[r][HD + 1], lsum);
+    }
+    part[tid] = out;
+    if (tid == 0) { part[HD] = M; part[HD + 1] = lsum; }
+  }
+}
+
+// One wave per (b, h): merge the split partials, add row t, normalise, append the new rows.
+template <typename T, int HD>
+__global__ __launch_bounds__(64) void decode_finish_kernel(DecodeArgs a) {
+  constexpr int EPL = (HD + 63) / 64;   // elements per lane
+  const int bh = blockIdx.x, b = bh / a.H, h = bh % a.H;
+  const int lane = threadIdx.x;
+  const float c1 = a.scale * kLog2e;
+  const float* part = a.part + (int64_t)bh * a.splits * (HD + 2);
+  const T* qc = view_row<T>(a.qc, b, h, 0);
+  const T* kc = view_row<T>(a.kc, b, h, 0);
+  const T* vc = view_row<T>(a.vc, b, h, 0);
+  const T* qu = view_row<T>(a.qu, b, h, 0);
+
+  float dot = 0.f;
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) {
+    const int n = lane + 64 * e;
+    if (n < HD) dot = __builtin_fmaf((float)qc[n], (float)kc[n], dot);
+  }
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) dot += __shfl_xor(dot, o);
+  const float xt = dot * c1;            // row t: U_t = 0, so the lookahead term is silu(0) = 0
+
+  float M = xt;
+  const int nsplit = a.t > 0 ? a.splits : 0;
+  for (int s = 0; s < nsplit; ++s) M = fmaxf(M, part[s * (HD + 2) + HD]);
+  const float pt = fast_exp2(xt - M);
+  float lsum = pt;
+  float o[EPL];
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) {
+    const int n = lane + 64 * e;
+    o[e] = n < HD ? pt * (float)vc[n] : 0.f;
+  }
+  for (int s = 0; s < nsplit; ++s) {
+    const float ms = part[s * (HD + 2) + HD];
+    const float w = (ms == -INFINITY) ? 0.f : fast_exp2(ms - M);
+    lsum = __builtin_fmaf(w, part[s * (HD + 2) + HD + 1], lsum);
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) {
+      const int n = lane + 64 * e;
+      if (n < HD) o[e] = __builtin_fmaf(w, part[s * (HD + 2) + n], o[e]);
+    }
+  }
+  const float inv = 1.f / lsum;
+  T* out = view_row<T>(a.out, b, h, 0);
+  T* Ut = view_row<T>(a.U, b, h, a.t);
+  T* qut = view_row<T>(a.qu_cache, b, h, a.t);
+  T* kct = view_row<T>(a.kc_cache, b, h, a.t);
+  T* vct = view_row<T>(a.vc_cache, b, h, a.t);
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) {
+    const int n = lane + 64 * e;
+    if (n < HD) {
+      out[n] = (T)(o[e] * inv);
+      Ut[n] = (T)0.f;
+      qut[n] = qu[n];
+      kct[n] = kc[n];
+      vct[n] = vc[n];
+    }
+  }
+}
+
+template <typename T, int HD> static int launch_decode_t(const DecodeArgs& a, hipStream_t stream) {
+  const int BH = a.B * a.H;
+  if (a.t > 0) hipLaunchKernelGGL((decode_stream_kernel<T, HD>), dim3(a.splits, BH), dim3(kThreads), 0, stream, a);
+  hipLaunchKernelGGL((decode_finish_kernel<T, HD>), dim3(BH), dim3(64), 0, stream, a);
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+template <typename T> static int launch_decode_d(const DecodeArgs& a, hipStream_t stream) {
+  switch (a.d) {
+    case 16: return launch_decode_t<T, 16>(a, stream);
+    case 32: return launch_decode_t<T, 32>(a, stream);
+    case 64: return launch_decode_t<T, 64>(a, stream);
+    case 128: return launch_decode_t<T, 128>(a, stream);
+    default: return -2;
+  }
+}
+
+int launch_decode(const DecodeArgs& a, int dtype, hipStream_t stream) {
+  switch (dtype) {
+    case 0: return launch_decode_d<float>(a, stream);
+    case 1: return launch_decode_d<bf16_t>(a, stream);
+    case 2: return launch_decode_d<fp16_t>(a, stream);
+    default: return -1;
+  }
+}
+
+// rows of one (b, h) handled per workgroup iteration, needed by the host to size `splits`
+int decode_pick_splits(int BH, int t) {
+  if (t <= 0) return 1;
+  int want = (2048 + BH - 1) / BH;          // aim at >= 2048 workgroups (256 CUs x 8)
+  int max_by_rows = (t + 63) / 64;          // at least 64 rows per workgroup
+  int s = want < max_by_rows ? want : max_by_rows;
+  if (s < 1) s = 1;
+  if (s > 64) s = 64;
+  return s;
+}
+
+}  // namespace castle

@@ -1,0 +1,346 @@
+// CASTLE parallel forward for gfx950: O(L^2 d) state form in three kernels.
+//
+//   tqv_kernel   per 64-row block I:  T_II = tril(Qc_I Vu_I^T)  (and its transpose)
+//   scan_kernel  key-stationary: for a group of 128 keys sweep the source blocks I,
+//                A_KI = sigmoid(s Qu_K Ku_I^T) (strictly j>k), state += A_KI Vu_I.
+//                The state as of the start of block I is stored as snapshot
+//                usnap[I][k]; the final state is the cache tensor U.
+//   attn_kernel  query-stationary: 128 queries per workgroup (two 64-row blocks),
+//                keys streamed in chunks of 64:
+//                  Su = Qc_I usnap[I][K]^T + T_II A_KI^T,  S = s(Sc - Su sigmoid(s Su)),
+//                online softmax over keys, O = P Vc.
+// The math follows the dense definition at lookahead_keys_attention.py:132-164 of the
+// reference; operands stay unscaled and the softmax scale is applied in fp32.
+#include "castle_tiles.h"
+#include "castle_params.h"
+
+namespace castle {
+
+extern __shared__ __attribute__((aligned(16))) unsigned char castle_smem[];
+
+template <typename T, int HD> constexpr int scan_lds_bytes() {
+  return (int)sizeof(T) * (kNB * lds_ld<T>(HD) + (HD < 32 ? 32 : HD) * lds_ld<T>(kNB));
+}
+template <typename T, int HD> constexpr int attn_lds_bytes() {
+  return (int)sizeof(T) * (4 * kNB * lds_ld<T>(HD) + (HD < 32 ? 32 : HD) * lds_ld<T>(kNB) + kNB * lds_ld<T>(128));
+}
+
+template <typename T> __device__ __forceinline__ const T* head_ptr(const View4& v, int b, int h) {
+  return reinterpret_cast<const T*>(v.ptr) + (int64_t)b * v.sb + (int64_t)h * v.sh;
+}
+template <typename T> __device__ __forceinline__ T* head_ptr_mut(const View4& v, int b, int h) {
+  return reinterpret_cast<T*>(v.ptr) + (int64_t)b * v.sb + (int64_t)h * v.sh;
+}
+
+// ---------------------------------------------------------------------------
+template <typename T, int HD>
+__global__ __launch_bounds__(kThreads) void tqv_kernel(FwdArgs a) {
+  constexpr int KS = HD / 16;
+  constexpr int TB = kNB / 32;
+  const int I = blockIdx.x, bh = blockIdx.y, b = bh / a.s.H, h = bh % a.s.H;
+  const int lane = lane_id(), c = lane & 31, g = lane >> 5;
+  const T* qc = head_ptr<T>(a.qc, b, h);
+  const T* vu = head_ptr<T>(a.vu, b, h);
+  T* tb = reinterpret_cast<T*>(a.ws.t_blk) + (int64_t)bh * a.s.Lp * kNB;
+  T* ttb = reinterpret_cast<T*>(a.ws.tt_blk) + (int64_t)bh * a.s.Lp * kNB;
+  for (int t = wave_id(); t < TB * TB; t += kThreads / 64) {
+    const int it = t / TB, jt = t % TB;
+    const int64_t i = (int64_t)I * kNB + 32 * it + c;   // A-operand row
+    const int64_t j = (int64_t)I * kNB + 32 * jt + c;   // B-operand row
+    acc_t acc;
+    zero(acc);
+#pragma unroll
+    for (int s = 0; s < KS; ++s)
+      mma(acc, ldg_nat<T>(qc, a.qc.sl, i, 16 * s + 8 * g, i < a.s.L), ldg_nat<T>(vu, a.vu.sl, j, 16 * s + 8 * g, j < a.s.L));
+    // acc[r] = T[il = 32 it + acc_row][jl = 32 jt + c]
+    const int jl = 32 * jt + c;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int il = 32 * it + acc_row(r, g);
+      if (jl > il) acc[r] = 0.f;
+      tb[((int64_t)I * kNB + il) * kNB + jl] = (T)acc[r];
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      st4<T>(ttb + ((int64_t)I * kNB + jl) * kNB + 32 * it + 8 * q + 4 * g, pack4<T>(acc, q));
+  }
+}
+
+// ---------------------------------------------------------------------------
+template <typename T, int HD>
+__global__ __launch_bounds__(kThreads) void scan_kernel(FwdArgs a) {
+  constexpr int KS = HD / 16;
+  constexpr int HDP = HD < 32 ? 32 : HD;
+  constexpr int NT = HDP / 32;
+  constexpr int JT = kNB / 32;
+  constexpr int LDK = lds_ld<T>(HD), LDV = lds_ld<T>(kNB);
+  T* s_ku = reinterpret_cast<T*>(castle_smem);   // [kNB][LDK]
+  T* s_vut = s_ku + kNB * LDK;                   // [HDP][LDV]
+
+  const int kb = blockIdx.x, bh = blockIdx.y, b = bh / a.s.H, h = bh % a.s.H;
+  const int lane = lane_id(), wave = wave_id(), c = lane & 31, g = lane >> 5;
+  const int L = a.s.L;
+  const float c1 = a.s.scale * kLog2e;
+  const int kw0 = kb * 128 + 32 * wave;
+  const int k = kw0 + c;
+  const T* qu = head_ptr<T>(a.qu, b, h);
+  const T* ku = head_ptr<T>(a.ku, b, h);
+  const T* vu = head_ptr<T>(a.vu, b, h);
+  T* snap = reinterpret_cast<T*>(a.ws.usnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
+
+  frag<T> fq[KS];
+#pragma unroll
+  for (int s = 0; s < KS; ++s) fq[s] = ldg_nat<T>(qu, a.qu.sl, k, 16 * s + 8 * g, k < L);
+  acc_t st[NT];   // state^T : rows n (head dim), columns k (lanes)
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) zero(st[nt]);
+  if (HDP > HD) lds_zero(s_vut + HD * LDV, (HDP - HD) * LDV);
+
+  const int I0 = (kb * 128) / kNB;
+  for (int I = I0; I < a.s.nblk; ++I) {
+    if (I * kNB >= kw0 + 32) {   // all keys of this wave precede block I: snapshot
+      T* dst = snap + (usnap_off(I) + k) * HD;
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int n = 32 * nt + 8 * q + 4 * g;
+          if (n < HD) st4<T>(dst + n, pack4<T>(st[nt], q));
+        }
+    }
+    __syncthreads();
+    stage_rows<T, kNB, HD>(s_ku, ku, a.ku.sl, (int64_t)I * kNB, L);
+    stage_rows_t<T, kNB, HD>(s_vut, vu, a.vu.sl, (int64_t)I * kNB, L);
+    __syncthreads();
+#pragma unroll
+    for (int jt = 0; jt < JT; ++jt) {
+      const int j0 = I * kNB + 32 * jt;
+      if (j0 + 31 <= kw0) continue;   // every j <= every k of this wave
+      acc_t aT;                       // A^T tile: rows j, columns k
+      zero(aT);
+#pragma unroll
+      for (int s = 0; s < KS; ++s) mma(aT, ld_nat<T>(s_ku, LDK, 32 * jt + c, 16 * s + 8 * g), fq[s]);
+      const bool diag = j0 <= kw0 + 31;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        float v = sigmoid_l2(aT[r] * c1);
+        if (diag && j0 + acc_row(r, g) <= k) v = 0.f;
+        aT[r] = v;
+      }
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        const frag<T> fa = chain<T>(aT, s2);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) mma(st[nt], ld_chain<T>(s_vut, LDV, 32 * nt + c, 32 * jt + 16 * s2, g), fa);
+      }
+    }
+  }
+  if (a.U.ptr != nullptr && k < L) {
+    T* dst = head_ptr_mut<T>(a.U, b, h) + (int64_t)k * a.U.sl;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = 32 * nt + 8 * q + 4 * g;
+        if (n < HD) st4<T>(dst + n, pack4<T>(st[nt], q));
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------
+template <typename T, int HD>
+__global__ __launch_bounds__(kThreads) void attn_kernel(FwdArgs a) {
+  constexpr int KS = HD / 16;
+  constexpr int HDP = HD < 32 ? 32 : HD;
+  constexpr int NT = HDP / 32;
+  constexpr int KT = kNB / 32;
+  constexpr int QB = 128;
+  constexpr int NBLK_Q = QB / kNB;   // snapshot blocks per workgroup
+  constexpr int LDK = lds_ld<T>(HD), LDV = lds_ld<T>(kNB), LDA = lds_ld<T>(QB);
+  T* s_kc = reinterpret_cast<T*>(castle_smem);   // [kNB][LDK]
+  T* s_qu = s_kc + kNB * LDK;                    // [kNB][LDK]
+  T* s_ub0 = s_qu + kNB * LDK;                   // [NBLK_Q][kNB][LDK]
+  T* s_vct = s_ub0 + NBLK_Q * kNB * LDK;         // [HDP][LDV]
+  T* s_a = s_vct + HDP * LDV;                    // [kNB][LDA]
+
+  const int qb = gridDim.x - 1 - blockIdx.x;   // longest rows first
+  const int bh = blockIdx.y, b = bh / a.s.H, h = bh % a.s.H;
+  const int lane = lane_id(), wave = wave_id(), c = lane & 31, g = lane >> 5;
+  const int L = a.s.L;
+  const float c1 = a.s.scale * kLog2e;
+  const int i0w = qb * QB + 32 * wave;
+  const int i = i0w + c;
+  const int Ifirst = (qb * QB) / kNB;
+  const int Iw = i0w / kNB;
+  const int jw = 32 * wave;                     // this wave's columns inside the A tile
+  const int cb = (jw / kNB) * kNB;              // first column of its block
+  const int nintra = ((jw % kNB) + 32) / 16;    // contraction steps of the in-block term
+
+  const T* qc = head_ptr<T>(a.qc, b, h);
+  const T* kc = head_ptr<T>(a.kc, b, h);
+  const T* vc = head_ptr<T>(a.vc, b, h);
+  const T* qu = head_ptr<T>(a.qu, b, h);
+  const T* ku = head_ptr<T>(a.ku, b, h);
+  const T* tb = reinterpret_cast<const T*>(a.ws.t_blk) + (int64_t)bh * a.s.Lp * kNB;
+  const T* snap = reinterpret_cast<const T*>(a.ws.usnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
+
+  frag<T> fqc[KS], fku[KS], ft[kNB / 16];
+#pragma unroll
+  for (int s = 0; s < KS; ++s) {
+    fqc[s] = ldg_nat<T>(qc, a.qc.sl, i, 16 * s + 8 * g, i < L);
+    fku[s] = ldg_nat<T>(ku, a.ku.sl, i, 16 * s + 8 * g, i < L);
+  }
+#pragma unroll
+  for (int s = 0; s < kNB / 16; ++s) ft[s] = ldg_nat<T>(tb, kNB, i, 16 * s + 8 * g, s < nintra);
+
+  acc_t o[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) zero(o[nt]);
+  float m = -INFINITY, l = 0.f;
+  if (HDP > HD) lds_zero(s_vct + HD * LDV, (HDP - HD) * LDV);
+
+  int nchunks = (qb * QB + QB) / kNB;
+  if (nchunks > a.s.nblk) nchunks = a.s.nblk;
+  for (int Kb = 0; Kb < nchunks; ++Kb) {
+    __syncthreads();
+    stage_rows<T, kNB, HD>(s_kc, kc, a.kc.sl, (int64_t)Kb * kNB, L);
+    stage_rows_t<T, kNB, HD>(s_vct, vc, a.vc.sl, (int64_t)Kb * kNB, L);
+    stage_rows<T, kNB, HD>(s_qu, qu, a.qu.sl, (int64_t)Kb * kNB, L);
+#pragma unroll
+    for (int q = 0; q < NBLK_Q; ++q) {
+      const int blk = Ifirst + q;
+      if (Kb < blk && blk < a.s.nblk)
+        stage_rows<T, kNB, HD>(s_ub0 + q * kNB * LDK, snap + usnap_off(blk) * HD, HD, (int64_t)Kb * kNB, (int64_t)1 << 40);
+    }
+    __syncthreads();
+    const bool active = Kb <= Iw;
+    if (active) {
+      // gate tile for this wave's 32 source rows: A^T[j rows, k lanes]
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt) {
+        acc_t aT;
+        zero(aT);
+#pragma unroll
+        for (int s = 0; s < KS; ++s) mma(aT, fku[s], ld_nat<T>(s_qu, LDK, 32 * kt + c, 16 * s + 8 * g));
+        const int kk = Kb * kNB + 32 * kt + c;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          float v = sigmoid_l2(aT[r] * c1);
+          if (i0w + acc_row(r, g) <= kk) v = 0.f;
+          aT[r] = v;
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          st4<T>(s_a + (32 * kt + c) * LDA + jw + 8 * q + 4 * g, pack4<T>(aT, q));
+      }
+    }
+    __syncthreads();
+    if (active) {
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt) {
+        const int k0 = Kb * kNB + 32 * kt;
+        if (k0 > i0w + 31) continue;
+        acc_t sc, su;
+        zero(sc);
+        zero(su);
+#pragma unroll
+        for (int s = 0; s < KS; ++s) mma(sc, ld_nat<T>(s_kc, LDK, 32 * kt + c, 16 * s + 8 * g), fqc[s]);
+        if (Kb < Iw) {
+          const T* ub = s_ub0 + (Iw - Ifirst) * kNB * LDK;
+#pragma unroll
+          for (int s = 0; s < KS; ++s) mma(su, ld_nat<T>(ub, LDK, 32 * kt + c, 16 * s + 8 * g), fqc[s]);
+        }
+#pragma unroll
+        for (int s = 0; s < kNB / 16; ++s)
+          if (s < nintra) mma(su, ld_nat<T>(s_a, LDA, 32 * kt + c, cb + 16 * s + 8 * g), ft[s]);
+
+        const bool diag = k0 + 31 > i0w;
+        float mx = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float sg = sigmoid_l2(su[r] * c1);
+          float x = __builtin_fmaf(-su[r], sg, sc[r]);
+          if (diag && k0 + acc_row(r, g) > i) x = -INFINITY;
+          sc[r] = x;
+          mx = fmaxf(mx, x);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m, mx * c1);
+        const float alpha = fast_exp2(m - m_new);
+        float ls = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float pv = fast_exp2(__builtin_fmaf(sc[r], c1, -m_new));
+          sc[r] = pv;
+          ls += pv;
+        }
+        l = l * alpha + ls;
+        m = m_new;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) o[nt][r] *= alpha;
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+          const frag<T> fp = chain<T>(sc, s2);
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) mma(o[nt], ld_chain<T>(s_vct, LDV, 32 * nt + c, 32 * kt + 16 * s2, g), fp);
+        }
+      }
+    }
+  }
+  const float lt = l + __shfl_xor(l, 32);
+  if (i < L) {
+    const float inv = 1.f / lt;
+    T* dst = head_ptr_mut<T>(a.out, b, h) + (int64_t)i * a.out.sl;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[nt][r] *= inv;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = 32 * nt + 8 * q + 4 * g;
+        if (n < HD) st4<T>(dst + n, pack4<T>(o[nt], q));
+      }
+    }
+    if (g == 0) a.ws.lse[(int64_t)bh * a.s.Lp + i] = (m + __builtin_log2f(lt)) * kLn2;
+  }
+}
+
+// ---------------------------------------------------------------------------
+template <typename T, int HD> static int launch_fwd_t(const FwdArgs& a, hipStream_t stream) {
+  const int BH = a.s.B * a.s.H;
+  constexpr int scan_lds = scan_lds_bytes<T, HD>(), attn_lds = attn_lds_bytes<T, HD>();
+  if (attn_lds > kMaxLds) return -2;   // this (dtype, head dim) pair does not fit the 160 KB LDS
+  static bool configured = false;      // raising the dynamic-LDS limit is idempotent, so a race is harmless
+  if (!configured) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&scan_kernel<T, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, scan_lds) != hipSuccess) return -3;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_kernel<T, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, attn_lds) != hipSuccess) return -3;
+    configured = true;
+  }
+  hipLaunchKernelGGL((tqv_kernel<T, HD>), dim3(a.s.nblk, BH), dim3(kThreads), 0, stream, a);
+  hipLaunchKernelGGL((scan_kernel<T, HD>), dim3(a.s.Lp / 128, BH), dim3(kThreads), scan_lds, stream, a);
+  hipLaunchKernelGGL((attn_kernel<T, HD>), dim3(a.s.Lp / 128, BH), dim3(kThreads), attn_lds, stream, a);
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+template <typename T> static int launch_fwd_d(const FwdArgs& a, hipStream_t stream) {
+  switch (a.s.d) {
+    case 16: return launch_fwd_t<T, 16>(a, stream);
+    case 32: return launch_fwd_t<T, 32>(a, stream);
+    case 64: return launch_fwd_t<T, 64>(a, stream);
+    case 128: return launch_fwd_t<T, 128>(a, stream);
+    default: return -2;
+  }
+}
+
+int launch_fwd(const FwdArgs& a, int dtype, hipStream_t stream) {
+  switch (dtype) {
+    case 0: return launch_fwd_d<float>(a, stream);
+    case 1: return launch_fwd_d<bf16_t>(a, stream);
+    case 2: return launch_fwd_d<fp16_t>(a, stream);
+    default: return -1;
+  }
+}
+
+}  // namespace castle

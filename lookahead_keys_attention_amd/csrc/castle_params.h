@@ -1,0 +1,56 @@
+// Kernel argument blocks shared by the CASTLE HIP kernels and the C-ABI layer.
+#pragma once
+#include <stdint.h>
+
+namespace castle {
+
+// A (B, H, L, d) view with unit stride along d; strides are in elements.
+struct View4 {
+  void* ptr;
+  int64_t sb, sh, sl;
+};
+
+struct CoreShape {
+  int B, H, L, d;
+  int Lp;     // L rounded up to 128
+  int nblk;   // Lp / kNB
+  float scale;
+};
+
+// Workspace written by the forward pass and read again by the backward pass.
+struct FwdWorkspace {
+  void* t_blk;    // [B*H][Lp][kNB]  T[i][j_local]  = tril(Qc_I Vu_I^T), unscaled
+  void* tt_blk;   // [B*H][Lp][kNB]  T^T per block: [j][i_local]
+  void* usnap;    // [B*H][snap_rows(nblk)][d]  forward state at block starts
+  float* lse;     // [B*H][Lp] natural-log softmax normaliser
+};
+
+struct FwdArgs {
+  CoreShape s;
+  View4 qc, kc, vc, qu, ku, vu;
+  View4 out;      // written as (B, H, L, d) through arbitrary strides
+  View4 U;        // ptr == nullptr when the final lookahead keys are not wanted
+  FwdWorkspace ws;
+};
+
+struct BwdArgs {
+  CoreShape s;
+  View4 qc, kc, vc, qu, ku, vu, out, dout;
+  View4 dqc, dkc, dvc, dqu, dku, dvu;
+  FwdWorkspace ws;
+  void* gsnap;    // [B*H][snap_rows(nblk)][d]  reverse state at block ends
+  float* delta;   // [B*H][Lp]  rowsum(dO * O)
+};
+
+struct DecodeArgs {
+  int B, H, d;
+  int t;            // rows already in the cache
+  int splits;       // partitions of the t rows per (b, h)
+  float scale;
+  View4 U, qu_cache, kc_cache, vc_cache;   // capacity buffers, row t is appended
+  View4 qc, kc, vc, qu, ku, vu;            // new token, L == 1
+  View4 out;                               // (B, H, 1, d)
+  float* part;      // [B*H][splits][d + 2]  partial (acc, m, l)
+};
+
+}  // namespace castle

@@ -1,0 +1,172 @@
+// Device-side tile toolkit for the CASTLE kernels (gfx950 / CDNA4, wave64).
+//
+// Every contraction in the kernels is a 32x32 MFMA tile:
+//   bf16 : v_mfma_f32_32x32x16_bf16   (one instruction per 16-deep step)
+//   fp16 : v_mfma_f32_32x32x16_f16
+//   fp32 : 8 x v_mfma_f32_32x32x2_f32 (same register fragments, 8 elements deep per lane)
+// Lane l = (c, g) with c = l % 32, g = l / 32.
+//   operand fragment : 8 elements of the contraction axis for free index c.
+//                      "natural" order : slot e <-> contraction index 16*s + 8*g + e
+//                      "chained" order : slot e <-> contraction index 16*s + 8*(e/4) + 4*g + e%4
+//   accumulator tile : 16 floats; register r <-> row 8*(r/4) + 4*g + r%4, column c.
+// An accumulator tile whose ROW index is the next contraction index converts in
+// registers into two operand fragments in chained order (registers 0-7 and 8-15);
+// the partner operand is then read from LDS with ld_chain().
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace castle {
+
+typedef __bf16 bf16_t;
+typedef _Float16 fp16_t;
+template <typename T, int N> using vec = T __attribute__((ext_vector_type(N)));
+typedef vec<float, 16> acc_t;
+template <typename T> using frag = vec<T, 8>;
+// memory views of the vectors: never assume more than 16-byte (or natural, if smaller) alignment
+template <typename T> using frag_mem = vec<T, 8> __attribute__((aligned(16)));
+template <typename T> using vec4_mem = vec<T, 4> __attribute__((aligned(8)));
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+constexpr int kNB = 64;        // block size of the state snapshots (rows per block)
+constexpr int kThreads = 256;  // 4 waves per workgroup in every tiled kernel
+constexpr int kMaxLds = 160 * 1024;
+
+template <typename T> struct elem_traits;
+template <> struct elem_traits<bf16_t> { static constexpr int vec16 = 8; };
+template <> struct elem_traits<fp16_t> { static constexpr int vec16 = 8; };
+template <> struct elem_traits<float> { static constexpr int vec16 = 4; };
+
+// padded leading dimension of an LDS tile with `cols` payload columns (16 bytes of pad)
+template <typename T> __host__ __device__ constexpr int lds_ld(int cols) { return cols + elem_traits<T>::vec16; }
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
+__device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
+__device__ __forceinline__ int acc_row(int r, int g) { return 8 * (r >> 2) + 4 * g + (r & 3); }
+
+__device__ __forceinline__ void mma(acc_t& c, const frag<bf16_t>& a, const frag<bf16_t>& b) {
+  c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ void mma(acc_t& c, const frag<fp16_t>& a, const frag<fp16_t>& b) {
+  c = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ void mma(acc_t& c, const frag<float>& a, const frag<float>& b) {
+#pragma unroll
+  for (int t = 0; t < 8; ++t) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t], b[t], c, 0, 0, 0);
+}
+
+__device__ __forceinline__ void zero(acc_t& c) {
+#pragma unroll
+  for (int r = 0; r < 16; ++r) c[r] = 0.f;
+}
+
+template <typename T> __device__ __forceinline__ frag<T> zero_frag() {
+  frag<T> f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) f[e] = (T)0.f;
+  return f;
+}
+
+// registers 8*s .. 8*s+7 of an accumulator tile as an operand fragment (chained order)
+template <typename T> __device__ __forceinline__ frag<T> chain(const acc_t& c, int s) {
+  vec<float, 8> v;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] = c[8 * s + e];
+  return __builtin_convertvector(v, frag<T>);
+}
+
+// 8 contiguous elements tile[row][col .. col+7]
+template <typename T> __device__ __forceinline__ frag<T> ld_nat(const T* tile, int ld, int row, int col) {
+  return *reinterpret_cast<const frag_mem<T>*>(tile + row * ld + col);
+}
+// chained order: tile[row][col0+4g .. +3] and tile[row][col0+8+4g .. +3]   (col0 multiple of 16)
+template <typename T> __device__ __forceinline__ frag<T> ld_chain(const T* tile, int ld, int row, int col0, int g) {
+  const T* p = tile + row * ld + col0 + 4 * g;
+  vec<T, 4> lo = *reinterpret_cast<const vec4_mem<T>*>(p);
+  vec<T, 4> hi = *reinterpret_cast<const vec4_mem<T>*>(p + 8);
+  frag<T> f;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) { f[e] = lo[e]; f[4 + e] = hi[e]; }
+  return f;
+}
+
+// natural fragment straight from global memory (row-major, unit inner stride); zeros when !ok
+template <typename T> __device__ __forceinline__ frag<T> ldg_nat(const T* base, int64_t row_stride, int64_t row, int col, bool ok) {
+  if (!ok) return zero_frag<T>();
+  return *reinterpret_cast<const frag_mem<T>*>(base + row * row_stride + col);
+}
+
+// ---- global -> LDS staging -------------------------------------------------
+// Copies a ROWS x COLS tile whose first row is global row `row0`; rows >= `row_end` are
+// zero-filled.  dst is row-major with leading dimension lds_ld<T>(COLS).
+template <typename T, int ROWS, int COLS>
+__device__ __forceinline__ void stage_rows(T* dst, const T* src, int64_t row_stride, int64_t row0, int64_t row_end) {
+  constexpr int V = elem_traits<T>::vec16;
+  constexpr int VPR = COLS / V;
+  constexpr int LD = lds_ld<T>(COLS);
+  typedef vec<T, V> v16;
+  for (int v = threadIdx.x; v < ROWS * VPR; v += kThreads) {
+    int r = v / VPR, cv = v % VPR;
+    v16 x;
+#pragma unroll
+    for (int e = 0; e < V; ++e) x[e] = (T)0.f;
+    if (row0 + r < row_end) x = *reinterpret_cast<const v16*>(src + (row0 + r) * row_stride + cv * V);
+    *reinterpret_cast<v16*>(dst + r * LD + cv * V) = x;
+  }
+}
+
+// Transposed copy: dst[c][r] = src[row0 + r][c]; dst has COLS payload rows (callers that
+// need more rows zero them once) and leading dimension lds_ld<T>(ROWS).
+template <typename T, int ROWS, int COLS>
+__device__ __forceinline__ void stage_rows_t(T* dst, const T* src, int64_t row_stride, int64_t row0, int64_t row_end) {
+  constexpr int V = elem_traits<T>::vec16;
+  constexpr int VPR = COLS / V;
+  constexpr int LD = lds_ld<T>(ROWS);
+  typedef vec<T, V> v16;
+  typedef vec<T, 4> v4;
+  for (int p = threadIdx.x; p < (ROWS / 4) * VPR; p += kThreads) {
+    int rg = p / VPR, cv = p % VPR;
+    v16 x[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+#pragma unroll
+      for (int e = 0; e < V; ++e) x[q][e] = (T)0.f;
+      int64_t row = row0 + 4 * rg + q;
+      if (row < row_end) x[q] = *reinterpret_cast<const v16*>(src + row * row_stride + cv * V);
+    }
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      v4 y;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) y[q] = x[q][e];
+      *reinterpret_cast<vec4_mem<T>*>(dst + (cv * V + e) * LD + 4 * rg) = y;
+    }
+  }
+}
+
+// zero `count` elements of LDS (count multiple of 8)
+template <typename T> __device__ __forceinline__ void lds_zero(T* dst, int count) {
+  for (int i = threadIdx.x * 8; i < count; i += kThreads * 8) *reinterpret_cast<frag_mem<T>*>(dst + i) = zero_frag<T>();
+}
+
+// store 4 packed elements (8 bytes for 16-bit types, 16 for fp32)
+template <typename T> __device__ __forceinline__ void st4(T* p, vec<T, 4> v) { *reinterpret_cast<vec4_mem<T>*>(p) = v; }
+
+// 4 consecutive rows (registers 4q..4q+3) of an accumulator tile as a packed vector of T
+template <typename T> __device__ __forceinline__ vec<T, 4> pack4(const acc_t& c, int q) {
+  vec<float, 4> v = {c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3]};
+  return __builtin_convertvector(v, vec<T, 4>);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+// sigmoid(y) given z = y * log2(e)
+__device__ __forceinline__ float sigmoid_l2(float z) { return fast_rcp(1.f + fast_exp2(-z)); }
+
+// offsets (in rows) of block I inside the snapshot arrays
+__host__ __device__ inline int64_t usnap_off(int64_t I) { return (int64_t)kNB * I * (I - 1) / 2; }   // I >= 1, I*kNB rows
+__host__ __device__ inline int64_t gsnap_off(int64_t I) { return (int64_t)kNB * I * (I + 1) / 2; }   // I <= nblk-2, (I+1)*kNB rows
+__host__ __device__ inline int64_t snap_rows(int64_t nblk) { return (int64_t)kNB * nblk * (nblk - 1) / 2; }
+
+}  // namespace castle
