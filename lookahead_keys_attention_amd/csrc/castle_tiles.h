@@ -42,7 +42,13 @@ template <> struct elem_traits<float> { static constexpr int vec16 = 4; };
 template <typename T> __host__ __device__ constexpr int lds_ld(int cols) { return cols + elem_traits<T>::vec16; }
 
 __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
-__device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
+// The wave index is read through readfirstlane so that the compiler knows it is uniform:
+// every branch that depends on it then becomes a scalar branch.  This matters for
+// correctness, not only speed: MFMA instructions do not honour the EXEC mask, so an MFMA
+// inside a branch the compiler believes to be per-lane can execute for a wave that should
+// have skipped it.  No MFMA in these kernels may sit under a condition that is not derived
+// from wave_id(), blockIdx or kernel arguments.
+__device__ __forceinline__ int wave_id() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
 __device__ __forceinline__ int acc_row(int r, int g) { return 8 * (r >> 2) + 4 * g + (r & 3); }
 
 __device__ __forceinline__ void mma(acc_t& c, const frag<bf16_t>& a, const frag<bf16_t>& b) {
