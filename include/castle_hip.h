@@ -29,6 +29,13 @@ extern "C" {
 #define CASTLE_BF16 1
 #define CASTLE_F16 2
 
+/* flags of castle_fwd / castle_bwd.  By default bf16 tensors are converted to fp16 when they are
+ * loaded (exact for |x| < 65504) and every operand the kernels produce internally is fp16:
+ * same MFMA rate, 3 more mantissa bits, which keeps the gradients of long sequences inside the
+ * bf16 tolerance.  CASTLE_FLAG_BF16_OPERANDS keeps bf16 MFMA operands instead (full bf16 range).
+ * castle_bwd must get the same flags as the castle_fwd call whose workspace it reads. */
+#define CASTLE_FLAG_BF16_OPERANDS 1
+
 /* error codes */
 #define CASTLE_OK 0
 #define CASTLE_ERR_DTYPE (-1)      /* unknown element type */
@@ -58,10 +65,11 @@ int64_t castle_fwd_workspace_bytes(int B, int H, int L, int d, int dtype);
  * castle_attention_triton (lookahead_keys_attention.py:122).  out: (B,H,L,d) view that is
  * written (any strides, e.g. those of a (B,L,H,d) buffer).  U: optional (NULL, or a view
  * with ptr == NULL, to skip) final lookahead keys for the decode cache
- * (lookahead_keys_attention.py:161-164).  d in {16,32,64,128}; fp32 needs d <= 64. */
+ * (lookahead_keys_attention.py:161-164).  d in {16,32,64,128}; fp32 needs d <= 64. 
+ * flags: 0 or CASTLE_FLAG_BF16_OPERANDS. */
 int castle_fwd(const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
                const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
-               int B, int H, int L, int d, int dtype, float scale,
+               int B, int H, int L, int d, int dtype, float scale, int flags,
                const castle_view4* out, const castle_view4* U,
                void* workspace, int64_t workspace_bytes, void* stream);
 
@@ -71,11 +79,11 @@ int64_t castle_bwd_workspace_bytes(int B, int H, int L, int d, int dtype);
 /* Parallel backward.  Same operands as castle_fwd plus the forward output `out`, the
  * upstream gradient `dout` and the forward workspace as castle_fwd left it.  Writes the six
  * gradients (all (B,H,L,d) views; every element is written, nothing is accumulated).
- * U carries no gradient (lookahead_keys_attention_triton.py:513-515). */
+ * U carries no gradient (lookahead_keys_attention_triton.py:513-515).  d in {16,32,64}. */
 int castle_bwd(const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
                const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
                const castle_view4* out, const castle_view4* dout,
-               int B, int H, int L, int d, int dtype, float scale,
+               int B, int H, int L, int d, int dtype, float scale, int flags,
                const castle_view4* dqc, const castle_view4* dkc, const castle_view4* dvc,
                const castle_view4* dqu, const castle_view4* dku, const castle_view4* dvu,
                const void* fwd_workspace, int64_t fwd_workspace_bytes,

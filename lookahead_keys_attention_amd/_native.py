@@ -17,6 +17,7 @@ LIB_PATH = os.path.join(_HERE, "libcastle_hip.so")
 ABI_VERSION = 1
 DTYPE_CODES = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
 SUPPORTED_HEAD_DIMS = (16, 32, 64, 128)
+FLAG_BF16_OPERANDS = 1   # keep bf16 MFMA operands for bf16 tensors (default: fp16 operands)
 
 EXPORTED_SYMBOLS = (
     "castle_abi_version",
@@ -59,9 +60,9 @@ def _declare(lib):
     lib.castle_decode_workspace_bytes.restype = i64
     lib.castle_decode_workspace_bytes.argtypes = [i, i, i, i]
     lib.castle_fwd.restype = i
-    lib.castle_fwd.argtypes = [_VP] * 6 + [i, i, i, i, i, f, _VP, _VP, vp, i64, vp]
+    lib.castle_fwd.argtypes = [_VP] * 6 + [i, i, i, i, i, f, i, _VP, _VP, vp, i64, vp]
     lib.castle_bwd.restype = i
-    lib.castle_bwd.argtypes = [_VP] * 8 + [i, i, i, i, i, f] + [_VP] * 6 + [vp, i64, vp, i64, vp]
+    lib.castle_bwd.argtypes = [_VP] * 8 + [i, i, i, i, i, f, i] + [_VP] * 6 + [vp, i64, vp, i64, vp]
     lib.castle_decode_step.restype = i
     lib.castle_decode_step.argtypes = [_VP] * 4 + [i] + [_VP] * 6 + [i, i, i, i, f, _VP, vp, i64, vp]
 

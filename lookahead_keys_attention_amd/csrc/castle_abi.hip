@@ -8,8 +8,8 @@
 #include "castle_tiles.h"
 
 namespace castle {
-int launch_fwd(const FwdArgs& a, int dtype, hipStream_t stream);
-int launch_bwd(const BwdArgs& a, int dtype, hipStream_t stream);
+int launch_fwd(const FwdArgs& a, int dtype, bool bf16_operands, hipStream_t stream);
+int launch_bwd(const BwdArgs& a, int dtype, bool bf16_operands, hipStream_t stream);
 int launch_decode(const DecodeArgs& a, int dtype, hipStream_t stream);
 int decode_pick_splits(int BH, int t);
 }  // namespace castle
@@ -117,7 +117,7 @@ int64_t castle_fwd_workspace_bytes(int B, int H, int L, int d, int dtype) {
 
 int castle_fwd(const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
                const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
-               int B, int H, int L, int d, int dtype, float scale,
+               int B, int H, int L, int d, int dtype, float scale, int flags,
                const castle_view4* out, const castle_view4* U,
                void* workspace, int64_t workspace_bytes, void* stream) {
   int rc = check_core(B, H, L, d, dtype);
@@ -139,7 +139,7 @@ int castle_fwd(const castle_view4* qc, const castle_view4* kc, const castle_view
   a.out = to_view(out);
   a.U = to_view(want_U ? U : nullptr);
   a.ws = carve(workspace, g);
-  return castle::launch_fwd(a, dtype, static_cast<hipStream_t>(stream));
+  return castle::launch_fwd(a, dtype, (flags & CASTLE_FLAG_BF16_OPERANDS) != 0, static_cast<hipStream_t>(stream));
 }
 
 int64_t castle_bwd_workspace_bytes(int B, int H, int L, int d, int dtype) {
@@ -152,7 +152,7 @@ int64_t castle_bwd_workspace_bytes(int B, int H, int L, int d, int dtype) {
 int castle_bwd(const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
                const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
                const castle_view4* out, const castle_view4* dout,
-               int B, int H, int L, int d, int dtype, float scale,
+               int B, int H, int L, int d, int dtype, float scale, int flags,
                const castle_view4* dqc, const castle_view4* dkc, const castle_view4* dvc,
                const castle_view4* dqu, const castle_view4* dku, const castle_view4* dvu,
                const void* fwd_workspace, int64_t fwd_workspace_bytes,
@@ -180,7 +180,7 @@ int castle_bwd(const castle_view4* qc, const castle_view4* kc, const castle_view
   a.ws = carve(const_cast<void*>(fwd_workspace), g);
   a.gsnap = bwd_workspace;
   a.delta = reinterpret_cast<float*>(static_cast<char*>(bwd_workspace) + g.snap_bytes);
-  return castle::launch_bwd(a, dtype, static_cast<hipStream_t>(stream));
+  return castle::launch_bwd(a, dtype, (flags & CASTLE_FLAG_BF16_OPERANDS) != 0, static_cast<hipStream_t>(stream));
 }
 
 int64_t castle_decode_workspace_bytes(int B, int H, int d, int t_max) {

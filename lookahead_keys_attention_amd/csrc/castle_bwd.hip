@@ -71,7 +71,7 @@ struct Carver {
 constexpr int a16(int bytes) { return (bytes + 15) / 16 * 16; }
 
 // [n rows, lanes] accumulator tiles -> (row = lane index, 4 consecutive n) stores, scaled
-template <typename T, int HD, int NT>
+template <typename T, int HD, int NT>   // T: element type of the destination tensor
 __device__ __forceinline__ void store_rows(T* dst_row, acc_t (&acc)[NT], float mul, int g) {
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
@@ -123,7 +123,7 @@ template <typename T, int HD> constexpr int bwd_key_lds_bytes() {
   return b;
 }
 
-template <typename T, int HD>
+template <typename T, typename TI, int HD>
 __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   constexpr int KS = HD / 16;
   constexpr int HDP = HD < 32 ? 32 : HD;
@@ -155,13 +155,13 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   const int kw0 = kb * 128 + 32 * wave;
   const int k = kw0 + c;
   const int Iw = kw0 / kNB;
-  const T* qc = head_ptr<T>(a.qc, b, h);
-  const T* kc = head_ptr<T>(a.kc, b, h);
-  const T* vc = head_ptr<T>(a.vc, b, h);
-  const T* qu = head_ptr<T>(a.qu, b, h);
-  const T* ku = head_ptr<T>(a.ku, b, h);
-  const T* vu = head_ptr<T>(a.vu, b, h);
-  const T* dout = head_ptr<T>(a.dout, b, h);
+  const TI* qc = head_ptr<TI>(a.qc, b, h);
+  const TI* kc = head_ptr<TI>(a.kc, b, h);
+  const TI* vc = head_ptr<TI>(a.vc, b, h);
+  const TI* qu = head_ptr<TI>(a.qu, b, h);
+  const TI* ku = head_ptr<TI>(a.ku, b, h);
+  const TI* vu = head_ptr<TI>(a.vu, b, h);
+  const TI* dout = head_ptr<TI>(a.dout, b, h);
   const T* tb = reinterpret_cast<const T*>(a.ws.t_blk) + (int64_t)bh * a.s.Lp * kNB;
   const T* ttb = reinterpret_cast<const T*>(a.ws.tt_blk) + (int64_t)bh * a.s.Lp * kNB;
   const T* usnap = reinterpret_cast<const T*>(a.ws.usnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
@@ -172,9 +172,9 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   frag<T> fkc[KS], fvc[KS], fqu[KS], fub[KS];
 #pragma unroll
   for (int s = 0; s < KS; ++s) {
-    fkc[s] = ldg_nat<T>(kc, a.kc.sl, k, 16 * s + 8 * g, k < L);
-    fvc[s] = ldg_nat<T>(vc, a.vc.sl, k, 16 * s + 8 * g, k < L);
-    fqu[s] = ldg_nat<T>(qu, a.qu.sl, k, 16 * s + 8 * g, k < L);
+    fkc[s] = ldg_nat<T, TI>(kc, a.kc.sl, k, 16 * s + 8 * g, k < L);
+    fvc[s] = ldg_nat<T, TI>(vc, a.vc.sl, k, 16 * s + 8 * g, k < L);
+    fqu[s] = ldg_nat<T, TI>(qu, a.qu.sl, k, 16 * s + 8 * g, k < L);
     fub[s] = zero_frag<T>();
   }
   acc_t dvc[NT], dkc[NT], dqu[NT], G[NT];   // [n rows, k lanes]
@@ -205,15 +205,15 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
     }
     __syncthreads();
     const int64_t r0 = (int64_t)I * kNB;
-    stage_rows<T, kNB, HD>(s_qc, qc, a.qc.sl, r0, L);
-    stage_rows<T, kNB, HD>(s_do, dout, a.dout.sl, r0, L);
-    stage_rows<T, kNB, HD>(s_ku, ku, a.ku.sl, r0, L);
-    stage_rows<T, kNB, HD>(s_vu, vu, a.vu.sl, r0, L);
+    stage_rows<T, kNB, HD, TI>(s_qc, qc, a.qc.sl, r0, L);
+    stage_rows<T, kNB, HD, TI>(s_do, dout, a.dout.sl, r0, L);
+    stage_rows<T, kNB, HD, TI>(s_ku, ku, a.ku.sl, r0, L);
+    stage_rows<T, kNB, HD, TI>(s_vu, vu, a.vu.sl, r0, L);
     stage_rows<T, kNB, kNB>(s_t, tb, kNB, r0, (int64_t)1 << 40);
     if constexpr (TC) {
-      stage_rows_t<T, kNB, HD>(s_qct, qc, a.qc.sl, r0, L);
-      stage_rows_t<T, kNB, HD>(s_dot, dout, a.dout.sl, r0, L);
-      stage_rows_t<T, kNB, HD>(s_kut, ku, a.ku.sl, r0, L);
+      stage_rows_t<T, kNB, HD, TI>(s_qct, qc, a.qc.sl, r0, L);
+      stage_rows_t<T, kNB, HD, TI>(s_dot, dout, a.dout.sl, r0, L);
+      stage_rows_t<T, kNB, HD, TI>(s_kut, ku, a.ku.sl, r0, L);
       stage_rows<T, kNB, kNB>(s_tt, ttb, kNB, r0, (int64_t)1 << 40);
     }
     if (threadIdx.x < kNB) {
@@ -321,9 +321,9 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
     }
   }
   if (k < L) {
-    store_rows<T, HD, NT>(head_ptr_mut<T>(a.dkc, b, h) + (int64_t)k * a.dkc.sl, dkc, c0, g);
-    store_rows<T, HD, NT>(head_ptr_mut<T>(a.dvc, b, h) + (int64_t)k * a.dvc.sl, dvc, 1.f, g);
-    store_rows<T, HD, NT>(head_ptr_mut<T>(a.dqu, b, h) + (int64_t)k * a.dqu.sl, dqu, c0 * c0, g);
+    store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dkc, b, h) + (int64_t)k * a.dkc.sl, dkc, c0, g);
+    store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvc, b, h) + (int64_t)k * a.dvc.sl, dvc, 1.f, g);
+    store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqu, b, h) + (int64_t)k * a.dqu.sl, dqu, c0 * c0, g);
   }
 }
 
@@ -346,7 +346,7 @@ template <typename T, int HD> constexpr int bwd_query_lds_bytes() {
   return b > e ? b : e;
 }
 
-template <typename T, int HD>
+template <typename T, typename TI, int HD>
 __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
   constexpr int KS = HD / 16;
   constexpr int HDP = HD < 32 ? 32 : HD;
@@ -396,13 +396,13 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
   const int ifirst = lw / 16;                 // first step covering queries i >= j
   const bool has_g = Iw <= a.s.nblk - 2;
 
-  const T* qc = head_ptr<T>(a.qc, b, h);
-  const T* kc = head_ptr<T>(a.kc, b, h);
-  const T* vc = head_ptr<T>(a.vc, b, h);
-  const T* qu = head_ptr<T>(a.qu, b, h);
-  const T* ku = head_ptr<T>(a.ku, b, h);
-  const T* vu = head_ptr<T>(a.vu, b, h);
-  const T* dout = head_ptr<T>(a.dout, b, h);
+  const TI* qc = head_ptr<TI>(a.qc, b, h);
+  const TI* kc = head_ptr<TI>(a.kc, b, h);
+  const TI* vc = head_ptr<TI>(a.vc, b, h);
+  const TI* qu = head_ptr<TI>(a.qu, b, h);
+  const TI* ku = head_ptr<TI>(a.ku, b, h);
+  const TI* vu = head_ptr<TI>(a.vu, b, h);
+  const TI* dout = head_ptr<TI>(a.dout, b, h);
   const T* tb = reinterpret_cast<const T*>(a.ws.t_blk) + (int64_t)bh * a.s.Lp * kNB;
   const T* ttb = reinterpret_cast<const T*>(a.ws.tt_blk) + (int64_t)bh * a.s.Lp * kNB;
   const T* usnap = reinterpret_cast<const T*>(a.ws.usnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
@@ -411,10 +411,10 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
   frag<T> fqc[KS], fdo[KS], fku[KS], fvu[KS], ft[TS], ftt[TS];
 #pragma unroll
   for (int s = 0; s < KS; ++s) {
-    fqc[s] = ldg_nat<T>(qc, a.qc.sl, i, 16 * s + 8 * g, i < L);
-    fdo[s] = ldg_nat<T>(dout, a.dout.sl, i, 16 * s + 8 * g, i < L);
-    fku[s] = ldg_nat<T>(ku, a.ku.sl, i, 16 * s + 8 * g, i < L);
-    fvu[s] = ldg_nat<T>(vu, a.vu.sl, i, 16 * s + 8 * g, i < L);
+    fqc[s] = ldg_nat<T, TI>(qc, a.qc.sl, i, 16 * s + 8 * g, i < L);
+    fdo[s] = ldg_nat<T, TI>(dout, a.dout.sl, i, 16 * s + 8 * g, i < L);
+    fku[s] = ldg_nat<T, TI>(ku, a.ku.sl, i, 16 * s + 8 * g, i < L);
+    fvu[s] = ldg_nat<T, TI>(vu, a.vu.sl, i, 16 * s + 8 * g, i < L);
   }
 #pragma unroll
   for (int s = 0; s < TS; ++s) {
@@ -444,12 +444,12 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
   for (int k0 = 0; k0 < kend; k0 += kCK) {
     const int Kb = k0 / kNB;
     __syncthreads();
-    stage_rows<T, kCK, HD>(s_kc, kc, a.kc.sl, k0, L);
-    stage_rows<T, kCK, HD>(s_vc, vc, a.vc.sl, k0, L);
-    stage_rows<T, kCK, HD>(s_qu, qu, a.qu.sl, k0, L);
+    stage_rows<T, kCK, HD, TI>(s_kc, kc, a.kc.sl, k0, L);
+    stage_rows<T, kCK, HD, TI>(s_vc, vc, a.vc.sl, k0, L);
+    stage_rows<T, kCK, HD, TI>(s_qu, qu, a.qu.sl, k0, L);
     if constexpr (TC) {
-      stage_rows_t<T, kCK, HD>(s_kct, kc, a.kc.sl, k0, L);
-      stage_rows_t<T, kCK, HD>(s_qut, qu, a.qu.sl, k0, L);
+      stage_rows_t<T, kCK, HD, TI>(s_kct, kc, a.kc.sl, k0, L);
+      stage_rows_t<T, kCK, HD, TI>(s_qut, qu, a.qu.sl, k0, L);
     }
 #pragma unroll
     for (int q = 0; q < NQ; ++q) {
@@ -574,15 +574,15 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
 #pragma unroll
   for (int q = 0; q < NQ; ++q) {
     const int64_t r0 = (int64_t)(Ifirst + q) * kNB;
-    stage_rows<T, kNB, HD>(e_vu[q], vu, a.vu.sl, r0, L);
-    stage_rows<T, kNB, HD>(e_qc[q], qc, a.qc.sl, r0, L);
+    stage_rows<T, kNB, HD, TI>(e_vu[q], vu, a.vu.sl, r0, L);
+    stage_rows<T, kNB, HD, TI>(e_qc[q], qc, a.qc.sl, r0, L);
     if constexpr (TC) {
       if (HDP > HD) {
         lds_zero(e_vut[q] + HD * LDV, (HDP - HD) * LDV);
         lds_zero(e_qct[q] + HD * LDV, (HDP - HD) * LDV);
       }
-      stage_rows_t<T, kNB, HD>(e_vut[q], vu, a.vu.sl, r0, L);
-      stage_rows_t<T, kNB, HD>(e_qct[q], qc, a.qc.sl, r0, L);
+      stage_rows_t<T, kNB, HD, TI>(e_vut[q], vu, a.vu.sl, r0, L);
+      stage_rows_t<T, kNB, HD, TI>(e_qct[q], qc, a.qc.sl, r0, L);
     }
   }
   // dT^T[j rows, i lanes] masked to j <= i, shared as e_dt[j][i] for the source-side product
@@ -616,44 +616,46 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
       mma(dvu[nt], ld_tr_nat<T>(e_qct[qw], LDV, e_qc[qw], LDK, 32 * nt + c, HD, 16 * s, g), fdt);
   }
   if (i < L) {
-    store_rows<T, HD, NT>(head_ptr_mut<T>(a.dqc, b, h) + (int64_t)i * a.dqc.sl, dqc, c0, g);
-    store_rows<T, HD, NT>(head_ptr_mut<T>(a.dku, b, h) + (int64_t)i * a.dku.sl, dku, c0 * c0, g);
-    store_rows<T, HD, NT>(head_ptr_mut<T>(a.dvu, b, h) + (int64_t)i * a.dvu.sl, dvu, c0, g);
+    store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqc, b, h) + (int64_t)i * a.dqc.sl, dqc, c0, g);
+    store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dku, b, h) + (int64_t)i * a.dku.sl, dku, c0 * c0, g);
+    store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvu, b, h) + (int64_t)i * a.dvu.sl, dvu, c0, g);
   }
 }
 
 // ---------------------------------------------------------------------------
-template <typename T, int HD> static int launch_bwd_t(const BwdArgs& a, hipStream_t stream) {
+template <typename T, typename TI, int HD> static int launch_bwd_t(const BwdArgs& a, hipStream_t stream) {
   const int BH = a.s.B * a.s.H;
   constexpr int key_lds = bwd_key_lds_bytes<T, HD>(), query_lds = bwd_query_lds_bytes<T, HD>();
   if (key_lds > kMaxLds || query_lds > kMaxLds) return -2;
   static bool configured = false;   // raising the dynamic-LDS limit is idempotent, so a race is harmless
   if (!configured) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_key_kernel<T, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, key_lds) != hipSuccess) return -3;
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_query_kernel<T, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, query_lds) != hipSuccess) return -3;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_key_kernel<T, TI, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, key_lds) != hipSuccess) return -3;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_query_kernel<T, TI, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, query_lds) != hipSuccess) return -3;
     configured = true;
   }
   constexpr int RPB = kThreads / (HD / elem_traits<T>::vec16);
-  hipLaunchKernelGGL((delta_kernel<T, HD>), dim3((a.s.Lp + RPB - 1) / RPB, BH), dim3(kThreads), 0, stream, a);
-  hipLaunchKernelGGL((bwd_key_kernel<T, HD>), dim3(a.s.Lp / 128, BH), dim3(kThreads), key_lds, stream, a);
-  hipLaunchKernelGGL((bwd_query_kernel<T, HD>), dim3(a.s.Lp / 128, BH), dim3(kThreads), query_lds, stream, a);
+  hipLaunchKernelGGL((delta_kernel<TI, HD>), dim3((a.s.Lp + RPB - 1) / RPB, BH), dim3(kThreads), 0, stream, a);
+  hipLaunchKernelGGL((bwd_key_kernel<T, TI, HD>), dim3(a.s.Lp / 128, BH), dim3(kThreads), key_lds, stream, a);
+  hipLaunchKernelGGL((bwd_query_kernel<T, TI, HD>), dim3(a.s.Lp / 128, BH), dim3(kThreads), query_lds, stream, a);
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
-template <typename T> static int launch_bwd_d(const BwdArgs& a, hipStream_t stream) {
+template <typename T, typename TI> static int launch_bwd_d(const BwdArgs& a, hipStream_t stream) {
   switch (a.s.d) {
-    case 16: return launch_bwd_t<T, 16>(a, stream);
-    case 32: return launch_bwd_t<T, 32>(a, stream);
-    case 64: return launch_bwd_t<T, 64>(a, stream);
+    case 16: return launch_bwd_t<T, TI, 16>(a, stream);
+    case 32: return launch_bwd_t<T, TI, 32>(a, stream);
+    case 64: return launch_bwd_t<T, TI, 64>(a, stream);
     default: return -2;   // d = 128: the register budget of the key-stationary kernel is exceeded
   }
 }
 
-int launch_bwd(const BwdArgs& a, int dtype, hipStream_t stream) {
+// bf16 tensors use fp16 MFMA operands unless bf16_operands is set (must match the forward pass,
+// whose workspace holds operands in the compute type)
+int launch_bwd(const BwdArgs& a, int dtype, bool bf16_operands, hipStream_t stream) {
   switch (dtype) {
-    case 0: return launch_bwd_d<float>(a, stream);
-    case 1: return launch_bwd_d<bf16_t>(a, stream);
-    case 2: return launch_bwd_d<fp16_t>(a, stream);
+    case 0: return launch_bwd_d<float, float>(a, stream);
+    case 1: return bf16_operands ? launch_bwd_d<bf16_t, bf16_t>(a, stream) : launch_bwd_d<fp16_t, bf16_t>(a, stream);
+    case 2: return launch_bwd_d<fp16_t, fp16_t>(a, stream);
     default: return -1;
   }
 }

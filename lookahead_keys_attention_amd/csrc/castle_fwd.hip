@@ -33,14 +33,14 @@ template <typename T> __device__ __forceinline__ T* head_ptr_mut(const View4& v,
 }
 
 // ---------------------------------------------------------------------------
-template <typename T, int HD>
+template <typename T, typename TI, int HD>
 __global__ __launch_bounds__(kThreads) void tqv_kernel(FwdArgs a) {
   constexpr int KS = HD / 16;
   constexpr int TB = kNB / 32;
   const int I = blockIdx.x, bh = blockIdx.y, b = bh / a.s.H, h = bh % a.s.H;
   const int lane = lane_id(), c = lane & 31, g = lane >> 5;
-  const T* qc = head_ptr<T>(a.qc, b, h);
-  const T* vu = head_ptr<T>(a.vu, b, h);
+  const TI* qc = head_ptr<TI>(a.qc, b, h);
+  const TI* vu = head_ptr<TI>(a.vu, b, h);
   T* tb = reinterpret_cast<T*>(a.ws.t_blk) + (int64_t)bh * a.s.Lp * kNB;
   T* ttb = reinterpret_cast<T*>(a.ws.tt_blk) + (int64_t)bh * a.s.Lp * kNB;
   for (int t = wave_id(); t < TB * TB; t += kThreads / 64) {
@@ -51,7 +51,7 @@ __global__ __launch_bounds__(kThreads) void tqv_kernel(FwdArgs a) {
     zero(acc);
 #pragma unroll
     for (int s = 0; s < KS; ++s)
-      mma(acc, ldg_nat<T>(qc, a.qc.sl, i, 16 * s + 8 * g, i < a.s.L), ldg_nat<T>(vu, a.vu.sl, j, 16 * s + 8 * g, j < a.s.L));
+      mma(acc, ldg_nat<T, TI>(qc, a.qc.sl, i, 16 * s + 8 * g, i < a.s.L), ldg_nat<T, TI>(vu, a.vu.sl, j, 16 * s + 8 * g, j < a.s.L));
     // acc[r] = T[il = 32 it + acc_row][jl = 32 jt + c]
     const int jl = 32 * jt + c;
 #pragma unroll
@@ -67,7 +67,7 @@ __global__ __launch_bounds__(kThreads) void tqv_kernel(FwdArgs a) {
 }
 
 // ---------------------------------------------------------------------------
-template <typename T, int HD>
+template <typename T, typename TI, int HD>
 __global__ __launch_bounds__(kThreads) void scan_kernel(FwdArgs a) {
   constexpr int KS = HD / 16;
   constexpr int HDP = HD < 32 ? 32 : HD;
@@ -83,14 +83,14 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(FwdArgs a) {
   const float c1 = a.s.scale * kLog2e;
   const int kw0 = kb * 128 + 32 * wave;
   const int k = kw0 + c;
-  const T* qu = head_ptr<T>(a.qu, b, h);
-  const T* ku = head_ptr<T>(a.ku, b, h);
-  const T* vu = head_ptr<T>(a.vu, b, h);
+  const TI* qu = head_ptr<TI>(a.qu, b, h);
+  const TI* ku = head_ptr<TI>(a.ku, b, h);
+  const TI* vu = head_ptr<TI>(a.vu, b, h);
   T* snap = reinterpret_cast<T*>(a.ws.usnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
 
   frag<T> fq[KS];
 #pragma unroll
-  for (int s = 0; s < KS; ++s) fq[s] = ldg_nat<T>(qu, a.qu.sl, k, 16 * s + 8 * g, k < L);
+  for (int s = 0; s < KS; ++s) fq[s] = ldg_nat<T, TI>(qu, a.qu.sl, k, 16 * s + 8 * g, k < L);
   acc_t st[NT];   // state^T : rows n (head dim), columns k (lanes)
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) zero(st[nt]);
@@ -109,8 +109,8 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(FwdArgs a) {
         }
     }
     __syncthreads();
-    stage_rows<T, kNB, HD>(s_ku, ku, a.ku.sl, (int64_t)I * kNB, L);
-    stage_rows_t<T, kNB, HD>(s_vut, vu, a.vu.sl, (int64_t)I * kNB, L);
+    stage_rows<T, kNB, HD, TI>(s_ku, ku, a.ku.sl, (int64_t)I * kNB, L);
+    stage_rows_t<T, kNB, HD, TI>(s_vut, vu, a.vu.sl, (int64_t)I * kNB, L);
     __syncthreads();
 #pragma unroll
     for (int jt = 0; jt < JT; ++jt) {
@@ -136,19 +136,19 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(FwdArgs a) {
     }
   }
   if (a.U.ptr != nullptr && k < L) {
-    T* dst = head_ptr_mut<T>(a.U, b, h) + (int64_t)k * a.U.sl;
+    TI* dst = head_ptr_mut<TI>(a.U, b, h) + (int64_t)k * a.U.sl;
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int n = 32 * nt + 8 * q + 4 * g;
-        if (n < HD) st4<T>(dst + n, pack4<T>(st[nt], q));
+        if (n < HD) st4<TI>(dst + n, pack4<TI>(st[nt], q));
       }
   }
 }
 
 // ---------------------------------------------------------------------------
-template <typename T, int HD>
+template <typename T, typename TI, int HD>
 __global__ __launch_bounds__(kThreads) void attn_kernel(FwdArgs a) {
   constexpr int KS = HD / 16;
   constexpr int HDP = HD < 32 ? 32 : HD;
@@ -176,19 +176,19 @@ __global__ __launch_bounds__(kThreads) void attn_kernel(FwdArgs a) {
   const int cb = (jw / kNB) * kNB;              // first column of its block
   const int nintra = ((jw % kNB) + 32) / 16;    // contraction steps of the in-block term
 
-  const T* qc = head_ptr<T>(a.qc, b, h);
-  const T* kc = head_ptr<T>(a.kc, b, h);
-  const T* vc = head_ptr<T>(a.vc, b, h);
-  const T* qu = head_ptr<T>(a.qu, b, h);
-  const T* ku = head_ptr<T>(a.ku, b, h);
+  const TI* qc = head_ptr<TI>(a.qc, b, h);
+  const TI* kc = head_ptr<TI>(a.kc, b, h);
+  const TI* vc = head_ptr<TI>(a.vc, b, h);
+  const TI* qu = head_ptr<TI>(a.qu, b, h);
+  const TI* ku = head_ptr<TI>(a.ku, b, h);
   const T* tb = reinterpret_cast<const T*>(a.ws.t_blk) + (int64_t)bh * a.s.Lp * kNB;
   const T* snap = reinterpret_cast<const T*>(a.ws.usnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
 
   frag<T> fqc[KS], fku[KS], ft[kNB / 16];
 #pragma unroll
   for (int s = 0; s < KS; ++s) {
-    fqc[s] = ldg_nat<T>(qc, a.qc.sl, i, 16 * s + 8 * g, i < L);
-    fku[s] = ldg_nat<T>(ku, a.ku.sl, i, 16 * s + 8 * g, i < L);
+    fqc[s] = ldg_nat<T, TI>(qc, a.qc.sl, i, 16 * s + 8 * g, i < L);
+    fku[s] = ldg_nat<T, TI>(ku, a.ku.sl, i, 16 * s + 8 * g, i < L);
   }
 #pragma unroll
   for (int s = 0; s < kNB / 16; ++s) ft[s] = ldg_nat<T>(tb, kNB, i, 16 * s + 8 * g, s < nintra);
@@ -203,9 +203,9 @@ __global__ __launch_bounds__(kThreads) void attn_kernel(FwdArgs a) {
   if (nchunks > a.s.nblk) nchunks = a.s.nblk;
   for (int Kb = 0; Kb < nchunks; ++Kb) {
     __syncthreads();
-    stage_rows<T, kNB, HD>(s_kc, kc, a.kc.sl, (int64_t)Kb * kNB, L);
-    stage_rows_t<T, kNB, HD>(s_vct, vc, a.vc.sl, (int64_t)Kb * kNB, L);
-    stage_rows<T, kNB, HD>(s_qu, qu, a.qu.sl, (int64_t)Kb * kNB, L);
+    stage_rows<T, kNB, HD, TI>(s_kc, kc, a.kc.sl, (int64_t)Kb * kNB, L);
+    stage_rows_t<T, kNB, HD, TI>(s_vct, vc, a.vc.sl, (int64_t)Kb * kNB, L);
+    stage_rows<T, kNB, HD, TI>(s_qu, qu, a.qu.sl, (int64_t)Kb * kNB, L);
 #pragma unroll
     for (int q = 0; q < NBLK_Q; ++q) {
       const int blk = Ifirst + q;
@@ -292,7 +292,7 @@ __global__ __launch_bounds__(kThreads) void attn_kernel(FwdArgs a) {
   const float lt = l + __shfl_xor(l, 32);
   if (i < L) {
     const float inv = 1.f / lt;
-    T* dst = head_ptr_mut<T>(a.out, b, h) + (int64_t)i * a.out.sl;
+    TI* dst = head_ptr_mut<TI>(a.out, b, h) + (int64_t)i * a.out.sl;
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
 #pragma unroll
@@ -300,7 +300,7 @@ __global__ __launch_bounds__(kThreads) void attn_kernel(FwdArgs a) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int n = 32 * nt + 8 * q + 4 * g;
-        if (n < HD) st4<T>(dst + n, pack4<T>(o[nt], q));
+        if (n < HD) st4<TI>(dst + n, pack4<TI>(o[nt], q));
       }
     }
     if (g == 0) a.ws.lse[(int64_t)bh * a.s.Lp + i] = (m + __builtin_log2f(lt)) * kLn2;
@@ -308,37 +308,39 @@ __global__ __launch_bounds__(kThreads) void attn_kernel(FwdArgs a) {
 }
 
 // ---------------------------------------------------------------------------
-template <typename T, int HD> static int launch_fwd_t(const FwdArgs& a, hipStream_t stream) {
+template <typename T, typename TI, int HD> static int launch_fwd_t(const FwdArgs& a, hipStream_t stream) {
   const int BH = a.s.B * a.s.H;
   constexpr int scan_lds = scan_lds_bytes<T, HD>(), attn_lds = attn_lds_bytes<T, HD>();
   if (attn_lds > kMaxLds) return -2;   // this (dtype, head dim) pair does not fit the 160 KB LDS
   static bool configured = false;      // raising the dynamic-LDS limit is idempotent, so a race is harmless
   if (!configured) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&scan_kernel<T, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, scan_lds) != hipSuccess) return -3;
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_kernel<T, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, attn_lds) != hipSuccess) return -3;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&scan_kernel<T, TI, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, scan_lds) != hipSuccess) return -3;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_kernel<T, TI, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, attn_lds) != hipSuccess) return -3;
     configured = true;
   }
-  hipLaunchKernelGGL((tqv_kernel<T, HD>), dim3(a.s.nblk, BH), dim3(kThreads), 0, stream, a);
-  hipLaunchKernelGGL((scan_kernel<T, HD>), dim3(a.s.Lp / 128, BH), dim3(kThreads), scan_lds, stream, a);
-  hipLaunchKernelGGL((attn_kernel<T, HD>), dim3(a.s.Lp / 128, BH), dim3(kThreads), attn_lds, stream, a);
+  hipLaunchKernelGGL((tqv_kernel<T, TI, HD>), dim3(a.s.nblk, BH), dim3(kThreads), 0, stream, a);
+  hipLaunchKernelGGL((scan_kernel<T, TI, HD>), dim3(a.s.Lp / 128, BH), dim3(kThreads), scan_lds, stream, a);
+  hipLaunchKernelGGL((attn_kernel<T, TI, HD>), dim3(a.s.Lp / 128, BH), dim3(kThreads), attn_lds, stream, a);
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
-template <typename T> static int launch_fwd_d(const FwdArgs& a, hipStream_t stream) {
+template <typename T, typename TI> static int launch_fwd_d(const FwdArgs& a, hipStream_t stream) {
   switch (a.s.d) {
-    case 16: return launch_fwd_t<T, 16>(a, stream);
-    case 32: return launch_fwd_t<T, 32>(a, stream);
-    case 64: return launch_fwd_t<T, 64>(a, stream);
-    case 128: return launch_fwd_t<T, 128>(a, stream);
+    case 16: return launch_fwd_t<T, TI, 16>(a, stream);
+    case 32: return launch_fwd_t<T, TI, 32>(a, stream);
+    case 64: return launch_fwd_t<T, TI, 64>(a, stream);
+    case 128: return launch_fwd_t<T, TI, 128>(a, stream);
     default: return -2;
   }
 }
 
-int launch_fwd(const FwdArgs& a, int dtype, hipStream_t stream) {
+// bf16 tensors: operands are converted to fp16 on load (exact inside the fp16 range) and every
+// operand produced inside the kernels is fp16, unless bf16_operands asks for bf16 MFMA operands.
+int launch_fwd(const FwdArgs& a, int dtype, bool bf16_operands, hipStream_t stream) {
   switch (dtype) {
-    case 0: return launch_fwd_d<float>(a, stream);
-    case 1: return launch_fwd_d<bf16_t>(a, stream);
-    case 2: return launch_fwd_d<fp16_t>(a, stream);
+    case 0: return launch_fwd_d<float, float>(a, stream);
+    case 1: return bf16_operands ? launch_fwd_d<bf16_t, bf16_t>(a, stream) : launch_fwd_d<fp16_t, bf16_t>(a, stream);
+    case 2: return launch_fwd_d<fp16_t, fp16_t>(a, stream);
     default: return -1;
   }
 }

@@ -97,39 +97,53 @@ template <typename T> __device__ __forceinline__ frag<T> ld_chain(const T* tile,
   return f;
 }
 
+// element-wise conversion between the I/O type TI and the compute type T (same width);
+// bf16 -> fp16 goes through fp32 and is exact for values inside the fp16 range
+template <typename T, typename TI, int N> __device__ __forceinline__ vec<T, N> cvt_vec(vec<TI, N> x) {
+  if constexpr (__is_same(T, TI)) {
+    return x;
+  } else {
+    static_assert(sizeof(T) == sizeof(TI), "I/O and compute types must have the same width");
+    return __builtin_convertvector(__builtin_convertvector(x, vec<float, N>), vec<T, N>);
+  }
+}
+
 // natural fragment straight from global memory (row-major, unit inner stride); zeros when !ok
-template <typename T> __device__ __forceinline__ frag<T> ldg_nat(const T* base, int64_t row_stride, int64_t row, int col, bool ok) {
+template <typename T, typename TI = T>
+__device__ __forceinline__ frag<T> ldg_nat(const TI* base, int64_t row_stride, int64_t row, int col, bool ok) {
   if (!ok) return zero_frag<T>();
-  return *reinterpret_cast<const frag_mem<T>*>(base + row * row_stride + col);
+  return cvt_vec<T, TI, 8>(*reinterpret_cast<const frag_mem<TI>*>(base + row * row_stride + col));
 }
 
 // ---- global -> LDS staging -------------------------------------------------
 // Copies a ROWS x COLS tile whose first row is global row `row0`; rows >= `row_end` are
 // zero-filled.  dst is row-major with leading dimension lds_ld<T>(COLS).
-template <typename T, int ROWS, int COLS>
-__device__ __forceinline__ void stage_rows(T* dst, const T* src, int64_t row_stride, int64_t row0, int64_t row_end) {
+template <typename T, int ROWS, int COLS, typename TI = T>
+__device__ __forceinline__ void stage_rows(T* dst, const TI* src, int64_t row_stride, int64_t row0, int64_t row_end) {
   constexpr int V = elem_traits<T>::vec16;
   constexpr int VPR = COLS / V;
   constexpr int LD = lds_ld<T>(COLS);
   typedef vec<T, V> v16;
+  typedef vec<TI, V> v16i;
   for (int v = threadIdx.x; v < ROWS * VPR; v += kThreads) {
     int r = v / VPR, cv = v % VPR;
     v16 x;
 #pragma unroll
     for (int e = 0; e < V; ++e) x[e] = (T)0.f;
-    if (row0 + r < row_end) x = *reinterpret_cast<const v16*>(src + (row0 + r) * row_stride + cv * V);
+    if (row0 + r < row_end) x = cvt_vec<T, TI, V>(*reinterpret_cast<const v16i*>(src + (row0 + r) * row_stride + cv * V));
     *reinterpret_cast<v16*>(dst + r * LD + cv * V) = x;
   }
 }
 
 // Transposed copy: dst[c][r] = src[row0 + r][c]; dst has COLS payload rows (callers that
 // need more rows zero them once) and leading dimension lds_ld<T>(ROWS).
-template <typename T, int ROWS, int COLS>
-__device__ __forceinline__ void stage_rows_t(T* dst, const T* src, int64_t row_stride, int64_t row0, int64_t row_end) {
+template <typename T, int ROWS, int COLS, typename TI = T>
+__device__ __forceinline__ void stage_rows_t(T* dst, const TI* src, int64_t row_stride, int64_t row0, int64_t row_end) {
   constexpr int V = elem_traits<T>::vec16;
   constexpr int VPR = COLS / V;
   constexpr int LD = lds_ld<T>(ROWS);
   typedef vec<T, V> v16;
+  typedef vec<TI, V> v16i;
   typedef vec<T, 4> v4;
   for (int p = threadIdx.x; p < (ROWS / 4) * VPR; p += kThreads) {
     int rg = p / VPR, cv = p % VPR;
@@ -139,7 +153,7 @@ __device__ __forceinline__ void stage_rows_t(T* dst, const T* src, int64_t row_s
 #pragma unroll
       for (int e = 0; e < V; ++e) x[q][e] = (T)0.f;
       int64_t row = row0 + 4 * rg + q;
-      if (row < row_end) x[q] = *reinterpret_cast<const v16*>(src + row * row_stride + cv * V);
+      if (row < row_end) x[q] = cvt_vec<T, TI, V>(*reinterpret_cast<const v16i*>(src + row * row_stride + cv * V));
     }
 #pragma unroll
     for (int e = 0; e < V; ++e) {

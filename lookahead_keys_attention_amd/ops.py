@@ -20,6 +20,11 @@ import torch
 from . import _native as N
 
 
+# flags handed to castle_fwd / castle_bwd (0, or _native.FLAG_BF16_OPERANDS); read when the
+# forward runs and remembered for its backward
+DEFAULT_FLAGS = 0
+
+
 def _require_gpu(t: torch.Tensor, what: str):
     if not t.is_cuda:
         raise RuntimeError(f"{what}: the HIP kernels need tensors on the GPU (got {t.device})")
@@ -32,7 +37,7 @@ def _check_dims(d: int, dtype: torch.dtype):
         raise ValueError("float32 HIP kernels support dim_head <= 64")
 
 
-def _fwd_raw(qc, kc, vc, qu, ku, vu, scale, out, U):
+def _fwd_raw(qc, kc, vc, qu, ku, vu, scale, out, U, flags=0):
     """Launch castle_fwd; returns the forward workspace tensor."""
     B, H, L, d = qc.shape
     code = N.dtype_code(qc.dtype)
@@ -43,12 +48,12 @@ def _fwd_raw(qc, kc, vc, qu, ku, vu, scale, out, U):
     vo = N.view4(out)
     vU = N.view4(U) if U is not None else N.View4(None, 0, 0, 0)
     with torch.cuda.device(qc.device):
-        rc = lib.castle_fwd(*views, B, H, L, d, code, float(scale), vo, vU, ws.data_ptr(), nbytes, N.stream_ptr(qc.device))
+        rc = lib.castle_fwd(*views, B, H, L, d, code, float(scale), int(flags), vo, vU, ws.data_ptr(), nbytes, N.stream_ptr(qc.device))
     N.check(rc, "castle_fwd")
     return ws
 
 
-def _bwd_raw(qc, kc, vc, qu, ku, vu, out, dout, scale, grads, ws):
+def _bwd_raw(qc, kc, vc, qu, ku, vu, out, dout, scale, grads, ws, flags=0):
     B, H, L, d = qc.shape
     code = N.dtype_code(qc.dtype)
     lib = N.lib()
@@ -57,7 +62,7 @@ def _bwd_raw(qc, kc, vc, qu, ku, vu, out, dout, scale, grads, ws):
     views = [N.view4(t) for t in (qc, kc, vc, qu, ku, vu, out, dout)]
     gviews = [N.view4(t) for t in grads]
     with torch.cuda.device(qc.device):
-        rc = lib.castle_bwd(*views, B, H, L, d, code, float(scale), *gviews,
+        rc = lib.castle_bwd(*views, B, H, L, d, code, float(scale), int(flags), *gviews,
                             ws.data_ptr(), ws.numel(), bws.data_ptr(), nbytes, N.stream_ptr(qc.device))
     N.check(rc, "castle_bwd")
 
@@ -77,7 +82,8 @@ class _CastleAttention(torch.autograd.Function):
         ops = [_as_readable(t) for t in (q, k, v, qu, ku, vu)]
         out = torch.empty((B, L, H, d), dtype=q.dtype, device=q.device).permute(0, 2, 1, 3)
         U = torch.empty((B, H, L, d), dtype=q.dtype, device=q.device) if want_U else None
-        ws = _fwd_raw(*ops, scale, out, U)
+        ctx.flags = DEFAULT_FLAGS
+        ws = _fwd_raw(*ops, scale, out, U, ctx.flags)
         ctx.save_for_backward(*ops, out, ws)
         ctx.scale = scale
         if want_U:
@@ -92,7 +98,7 @@ class _CastleAttention(torch.autograd.Function):
         dout = _as_readable(dout)
         packed = torch.empty((6, B, H, L, d), dtype=out.dtype, device=out.device)
         grads = list(packed.unbind(0))
-        _bwd_raw(*ops, out, dout, ctx.scale, grads, ws)
+        _bwd_raw(*ops, out, dout, ctx.scale, grads, ws, ctx.flags)
         return (*grads, None, None)
 
 
@@ -111,7 +117,8 @@ class _CastleAttentionPacked(torch.autograd.Function):
         qu, ku, vu, qc, kc, vc = six.unbind(0)
         merged = torch.empty((B, L, heads * d), dtype=proj.dtype, device=proj.device)
         out = merged.view(B, L, heads, d).permute(0, 2, 1, 3)
-        ws = _fwd_raw(qc, kc, vc, qu, ku, vu, scale, out, U_out)
+        ctx.flags = DEFAULT_FLAGS
+        ws = _fwd_raw(qc, kc, vc, qu, ku, vu, scale, out, U_out, ctx.flags)
         ctx.save_for_backward(proj, merged, ws)
         ctx.heads, ctx.scale = heads, scale
         return merged
@@ -129,7 +136,7 @@ class _CastleAttentionPacked(torch.autograd.Function):
         dout = dmerged.view(B, L, heads, d).permute(0, 2, 1, 3)
         dproj = torch.empty_like(proj)
         dqu, dku, dvu, dqc, dkc, dvc = dproj.view(B, L, 6, heads, d).permute(2, 0, 3, 1, 4).unbind(0)
-        _bwd_raw(qc, kc, vc, qu, ku, vu, out, dout, scale, (dqc, dkc, dvc, dqu, dku, dvu), ws)
+        _bwd_raw(qc, kc, vc, qu, ku, vu, out, dout, scale, (dqc, dkc, dvc, dqu, dku, dvu), ws, ctx.flags)
         return dproj, None, None, None
 
 

@@ -1,0 +1,211 @@
+"""Module-level parity on the GPU: the reference's GPU tests re-stated for the native path
+(tests/test_lookahead.py:67-143, 185-222, 225-282 of the reference) and the BASELINE configs at
+their full sizes, checked through the oracle on sampled heads and through size-independent
+properties (parallel == cached sequential, causality / prefix invariance)."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from oracle import castle_oracle as O
+
+DEV = "cuda:0"
+
+
+def make(dim, heads, d, dtype=torch.float32, prenorm=False, rotary=False, seed=0):
+    from lookahead_keys_attention_amd import Castle
+
+    torch.manual_seed(seed)
+    m = Castle(dim, heads=heads, dim_head=d, use_triton=True, prenorm=prenorm, rotary_emb=rotary)
+    return m.to(DEV).to(dtype)
+
+
+def cpu_params(m):
+    return {k: v.detach().cpu().float() for k, v in m.state_dict().items()}
+
+
+def bf16_close(got, ref, what):
+    got, ref = got.detach().cpu().double(), ref.detach().cpu().double()
+    err = (got - ref).abs().max().item()
+    rel = ((got - ref).norm() / ref.norm()).item()
+    assert err <= 2e-2 * ref.abs().max().item() and rel <= 2e-2, f"{what}: max err {err:.3e} (max {ref.abs().max():.3e}), rel {rel:.3e}"
+
+
+@pytest.mark.parametrize("prenorm", [False, True])
+def test_native_vs_oracle_forward_and_grads(prenorm):
+    # reference: test_castle_triton_vs_reference, B2 L256 dim128 d64 H2, fwd 1e-3, grads 2e-2
+    m = make(128, 2, 64, prenorm=prenorm)
+    p = {k: v.clone().requires_grad_() for k, v in cpu_params(m).items()}
+    x = torch.randn(2, 256, 128, generator=torch.Generator().manual_seed(1))
+    gy = torch.randn(2, 256, 128, generator=torch.Generator().manual_seed(2))
+    xg = x.to(DEV).requires_grad_()
+    y = m(xg)
+    y.backward(gy.to(DEV))
+    xr = x.clone().requires_grad_()
+    yr = O.module_forward(xr, p, 2)
+    yr.backward(gy)
+    assert (y.detach().cpu() - yr.detach()).abs().max() <= 1e-3
+    assert (xg.grad.cpu() - xr.grad).abs().max() <= 2e-2
+    for name, par in m.named_parameters():
+        assert (par.grad.cpu() - p[name].grad).abs().max() <= 2e-2, name
+
+
+@pytest.mark.parametrize("prenorm", [False, True])
+def test_native_causality(prenorm):
+    # reference: test_castle_causality_triton, B2 L64 dim128 d64 H2, atol 1e-3
+    m = make(128, 2, 64, prenorm=prenorm).eval()
+    x = torch.randn(2, 64, 128, generator=torch.Generator().manual_seed(3)).to(DEV)
+    with torch.no_grad():
+        assert (m(x)[:, :32] - m(x[:, :32])).abs().max() <= 1e-3
+
+
+@pytest.mark.parametrize("prenorm", [False, True])
+@pytest.mark.parametrize("rotary", [False, True])
+def test_native_parallel_vs_sequential(prenorm, rotary):
+    # reference: test_castle_triton_parallel_vs_sequential, B2 L16 dim32 d16 H2 split 8, atol 1e-3.
+    # Here the cached steps run in HIP as well, and the rotary variant is included.
+    from lookahead_keys_attention_amd import Cache
+
+    m = make(32, 2, 16, prenorm=prenorm, rotary=rotary).eval()
+    x = torch.randn(2, 16, 32, generator=torch.Generator().manual_seed(4)).to(DEV)
+    with torch.no_grad():
+        y0, cache = m(x[:, :8], return_next_cache=True)
+        ys = [y0]
+        for t in range(8, 16):
+            y, cache = m(x[:, t:t + 1], cache=cache, return_next_cache=True)
+            ys.append(y)
+        full = m(x)
+    assert isinstance(cache, Cache) and cache.U.shape == (2, 2, 16, 16)
+    assert (torch.cat(ys, 1) - full).abs().max() <= 1e-3
+
+
+def test_decode_from_scratch_and_from_plain_tuple():
+    m = make(64, 2, 32).eval()
+    p = cpu_params(m)
+    x = torch.randn(2, 6, 64, generator=torch.Generator().manual_seed(5))
+    with torch.no_grad():
+        cache, ys = None, []
+        for t in range(6):
+            y, cache = m(x[:, t:t + 1].to(DEV), cache=cache)
+            ys.append(y)
+        ref = O.module_forward(x, p, 2)
+        assert (torch.cat(ys, 1).cpu() - ref).abs().max() <= 1e-3
+        # a foreign 4-tuple (e.g. produced by the dense formulation) is copied, then advanced
+        _, oc = O.module_forward(x[:, :5], p, 2, return_next_cache=True)
+        y5, c5 = m(x[:, 5:].to(DEV), cache=tuple(t.to(DEV) for t in oc))
+        assert (y5.cpu() - ref[:, 5:]).abs().max() <= 1e-3 and c5.U.shape[-2] == 6
+        # an already-advanced native cache cannot be replayed
+        _, c_old = m(x[:, :3].to(DEV), return_next_cache=True)
+        m(x[:, 3:4].to(DEV), cache=c_old)
+        with pytest.raises(RuntimeError, match="in place"):
+            m(x[:, 3:4].to(DEV), cache=c_old)
+
+
+def test_multi_token_with_cache_is_rejected():
+    m = make(32, 2, 16)
+    x = torch.randn(1, 4, 32).to(DEV)
+    _, cache = m(x, return_next_cache=True)
+    with pytest.raises(AssertionError):
+        m(x, cache=cache)
+
+
+def test_config1_readme_fp32_parallel_vs_sequential():
+    # BASELINE config 1: Castle(512, 8, 64), x (2,128,512) fp32, parallel vs 128 cached steps, atol 1e-3
+    m = make(512, 8, 64, seed=0).eval()
+    x = torch.randn(2, 128, 512, generator=torch.Generator().manual_seed(0))
+    with torch.no_grad():
+        full = m(x.to(DEV))
+        cache, ys = None, []
+        for t in range(128):
+            y, cache = m(x[:, t:t + 1].to(DEV), cache=cache)
+            ys.append(y)
+    seq = torch.cat(ys, 1)
+    assert (seq - full).abs().max() <= 1e-3
+    ref = O.module_forward(x, cpu_params(m), 8)
+    assert (full.cpu() - ref).abs().max() <= 1e-3 and (seq.cpu() - ref).abs().max() <= 1e-3
+
+
+def _head_oracle_check(proj, dmerged, merged, dproj, heads, d, b, h):
+    """fp32 oracle for one (b, h) slice of a packed bf16 run: out and the six gradients."""
+    B, L, _ = proj.shape
+    six = proj.view(B, L, 6, heads, d)
+    qu, ku, vu, qc, kc, vc = [six[b, :, i, h].float().cpu() for i in range(6)]
+    do = dmerged.view(B, L, heads, d)[b, :, h].float().cpu()
+    s = d ** -0.5
+    out = O.parallel_core(qc, kc, vc, qu, ku, vu, s)
+    bf16_close(merged.view(B, L, heads, d)[b, :, h], out, f"out[{b},{h}]")
+    grads = O.closed_form_grads(qc, kc, vc, qu, ku, vu, s, do)
+    g6 = dproj.view(B, L, 6, heads, d)
+    for name, idx, r in zip(("dqc", "dkc", "dvc", "dqu", "dku", "dvu"), (3, 4, 5, 0, 1, 2), grads):
+        bf16_close(g6[b, :, idx, h], r, f"{name}[{b},{h}]")
+
+
+def test_config2_bf16_full_size_sampled_heads():
+    # BASELINE config 2: dim 512, H8, d64, B4, L4096, bf16, forward + backward
+    from lookahead_keys_attention_amd import ops
+
+    m = make(512, 8, 64, dtype=torch.bfloat16, seed=0)
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(4, 4096, 512, generator=g).bfloat16().to(DEV)
+    gy = torch.randn(4, 4096, 512, generator=g).bfloat16().to(DEV)
+    proj = m.to_all_qkv(x).detach().requires_grad_()
+    merged = ops.castle_attention_packed(proj, 8, m.scale)
+    dmerged = (gy @ m.combine_heads.weight.detach())
+    merged.backward(dmerged)
+    assert torch.isfinite(merged).all() and torch.isfinite(proj.grad).all()
+    for b, h in ((0, 0), (3, 5)):
+        _head_oracle_check(proj.detach(), dmerged, merged.detach(), proj.grad, 8, 64, b, h)
+    # causality at full size: the first 1024 positions do not depend on the rest
+    short = ops.castle_attention_packed(proj.detach()[:, :1024].contiguous(), 8, m.scale)
+    bf16_close(merged.detach()[:, :1024], short, "prefix invariance")
+
+
+def test_config3_bf16_long_context_forward():
+    # BASELINE config 3 (forward): dim 2048, H16, d128, B1, L16384, bf16
+    from lookahead_keys_attention_amd import ops
+
+    m = make(2048, 16, 128, dtype=torch.bfloat16, seed=0)
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(1, 16384, 2048, generator=g).bfloat16().to(DEV)
+    with torch.no_grad():
+        proj = m.to_all_qkv(x)
+        merged = ops.castle_attention_packed(proj, 16, m.scale)
+        assert torch.isfinite(merged).all()
+        short = ops.castle_attention_packed(proj[:, :2048].contiguous(), 16, m.scale)
+        bf16_close(merged[:, :2048], short, "prefix invariance")
+        six = proj.view(1, 16384, 6, 16, 128)
+        qu, ku, vu, qc, kc, vc = [six[0, :2048, i, 7].float().cpu() for i in range(6)]
+        ref = O.parallel_core(qc, kc, vc, qu, ku, vu, m.scale)
+        bf16_close(short.view(1, 2048, 16, 128)[0, :, 7], ref, "head 7 vs oracle")
+
+
+def test_config4_bf16_decode_after_prefill():
+    # BASELINE config 4: B32, prefill 2048 through the parallel path, then cached steps
+    m = make(512, 8, 64, dtype=torch.bfloat16, seed=0).eval()
+    g = torch.Generator().manual_seed(0)
+    steps = 4
+    x = torch.randn(32, 2048 + steps, 512, generator=g).bfloat16().to(DEV)
+    with torch.no_grad():
+        _, cache = m(x[:, :2048], return_next_cache=True)
+        ys = []
+        for t in range(2048, 2048 + steps):
+            y, cache = m(x[:, t:t + 1], cache=cache)
+            ys.append(y)
+        full = m(x)
+    assert cache.U.shape == (32, 8, 2048 + steps, 64)
+    bf16_close(torch.cat(ys, 1), full[:, 2048:], "cached steps vs parallel")
+    # one (b, h) slice of the first step against the oracle's cached step in fp32
+    with torch.no_grad():
+        proj = m.to_all_qkv(x[:, :2049]).view(32, 2049, 6, 8, 64)
+    b, h = 17, 3
+    qu, ku, vu, qc, kc, vc = [proj[b, :, i, h].float().cpu() for i in range(6)]
+    _, U0 = O.parallel_core(*[t[:2048] for t in (qc, kc, vc, qu, ku, vu)], m.scale, want_U=True)
+    step, _ = O.decode_core((U0, qu[:2048], kc[:2048], vc[:2048]), *[t[2048:] for t in (qc, kc, vc, qu, ku, vu)], m.scale)
+    w = m.combine_heads.weight.detach().float().cpu()
+    # compare pre-projection head output: recompute native merged output for that head via the cache-free parallel path
+    from lookahead_keys_attention_amd import ops
+
+    with torch.no_grad():
+        merged = ops.castle_attention_packed(m.to_all_qkv(x[:, :2049]), 8, m.scale)
+    bf16_close(merged.view(32, 2049, 8, 64)[b, 2048, h], step[0], "row 2048 of head vs oracle decode")
+    del w

@@ -1,0 +1,145 @@
+"""Parity of the HIP path (through the C ABI) with the CPU oracle, on the GPU.
+
+Tolerances (binding, from the north star and the reference's own tests):
+  fp32 : outputs max|a-b| <= 1e-3, gradients <= 2e-2        (tests/test_lookahead.py:114,135 of the reference)
+  bf16 : against the oracle evaluated in fp64 on the same bf16-rounded inputs,
+         max|a-b| <= 2e-2 * max|b|  and  ||a-b|| <= 2e-2 * ||b||
+"""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from oracle import castle_oracle as O
+
+DEV = "cuda:0"
+NAMES = ("dqc", "dkc", "dvc", "dqu", "dku", "dvu")
+
+
+def H():
+    from lookahead_keys_attention_amd import ops
+
+    return ops
+
+
+def rand_ops(B, Hh, L, d, dtype, seed, scale=0.6):
+    g = torch.Generator().manual_seed(seed)
+    ops = [(torch.randn(B, Hh, L, d, generator=g) * scale).to(dtype) for _ in range(6)]
+    dout = torch.randn(B, Hh, L, d, generator=g).to(dtype)
+    return ops, dout
+
+
+def assert_close(got, ref, dtype, what, fp32_atol):
+    got, ref = got.detach().cpu().double(), ref.double()
+    err = (got - ref).abs().max().item()
+    if dtype == torch.float32:
+        assert err <= fp32_atol, f"{what}: max err {err:.3e} > {fp32_atol}"
+    else:
+        assert err <= 2e-2 * ref.abs().max().item(), f"{what}: max err {err:.3e} vs max {ref.abs().max():.3e}"
+        rel = ((got - ref).norm() / ref.norm()).item()
+        assert rel <= 2e-2, f"{what}: relative norm error {rel:.3e}"
+
+
+FWD_CASES = [
+    (1, 1, 1, 64, torch.float32), (1, 2, 7, 16, torch.float32), (2, 2, 64, 64, torch.float32),
+    (1, 2, 65, 32, torch.float32), (2, 2, 200, 32, torch.float32), (1, 2, 257, 64, torch.float32),
+    (1, 1, 384, 16, torch.float32), (2, 2, 384, 64, torch.bfloat16), (1, 2, 300, 128, torch.bfloat16),
+    (1, 2, 130, 32, torch.bfloat16), (1, 2, 256, 64, torch.float16),
+]
+
+
+@pytest.mark.parametrize("B,Hh,L,d,dtype", FWD_CASES)
+def test_operator_forward(B, Hh, L, d, dtype):
+    ops, _ = rand_ops(B, Hh, L, d, dtype, seed=L + d)
+    s = d ** -0.5
+    out, U = H().castle_attention_hip(*[t.to(DEV) for t in ops], s, True)
+    ref_out, ref_U = O.parallel_core(*[t.double() for t in ops], s, want_U=True)
+    assert out.shape == (B, Hh, L, d) and U.shape == (B, Hh, L, d) and out.dtype == dtype
+    assert_close(out, ref_out, dtype, "out", 1e-3)
+    if L > 1:
+        assert_close(U, ref_U, dtype, "U", 1e-3)
+    assert torch.all(U[:, :, -1] == 0)
+
+
+BWD_CASES = [
+    (1, 1, 1, 64, torch.float32), (1, 2, 9, 16, torch.float32), (2, 2, 64, 64, torch.float32),
+    (1, 2, 200, 32, torch.float32), (1, 2, 321, 64, torch.float32), (2, 2, 384, 64, torch.bfloat16),
+    (1, 2, 300, 32, torch.bfloat16), (1, 2, 256, 16, torch.bfloat16), (1, 2, 256, 64, torch.float16),
+]
+
+
+@pytest.mark.parametrize("B,Hh,L,d,dtype", BWD_CASES)
+def test_operator_backward(B, Hh, L, d, dtype):
+    ops, dout = rand_ops(B, Hh, L, d, dtype, seed=3 * L + d)
+    s = d ** -0.5
+    leaves = [t.to(DEV).requires_grad_() for t in ops]
+    H().castle_attention_hip(*leaves, s).backward(dout.to(DEV))
+    ref = O.closed_form_grads(*[t.double() for t in ops], s, dout.double())
+    for name, leaf, r in zip(NAMES, leaves, ref):
+        assert_close(leaf.grad, r, dtype, name, 2e-2)
+        if dtype == torch.float32:      # far inside the bound in practice
+            assert (leaf.grad.cpu().double() - r).abs().max() <= 1e-4, name
+
+
+def test_lookahead_keys_carry_no_gradient():
+    ops, dout = rand_ops(1, 1, 40, 16, torch.float32, seed=5)
+    leaves = [t.to(DEV).requires_grad_() for t in ops]
+    out, U = H().castle_attention_hip(*leaves, 0.25, True)
+    assert out.requires_grad and not U.requires_grad   # lookahead_keys_attention_triton.py:513-515
+
+
+def test_zero_lookahead_values_equal_sdpa():
+    ops, _ = rand_ops(2, 2, 150, 64, torch.float32, seed=6)
+    qc, kc, vc, qu, ku, vu = [t.to(DEV) for t in ops]
+    out = H().castle_attention_hip(qc, kc, vc, qu, ku, torch.zeros_like(vu), 64 ** -0.5)
+    ref = torch.nn.functional.scaled_dot_product_attention(*[t.double() for t in ops[:3]], is_causal=True)
+    assert (out.cpu().double() - ref).abs().max() <= 1e-4
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_packed_operator_equals_unpacked(dtype):
+    B, L, heads, d = 2, 200, 2, 64
+    g = torch.Generator().manual_seed(8)
+    proj = (torch.randn(B, L, 6 * heads * d, generator=g) * 0.6).to(dtype).to(DEV).requires_grad_()
+    dmerged = torch.randn(B, L, heads * d, generator=g).to(dtype).to(DEV)
+    merged, U = H().castle_attention_packed(proj, heads, d ** -0.5, True)
+    merged.backward(dmerged)
+    g_packed = proj.grad.clone()
+    proj.grad = None
+    qu, ku, vu, qc, kc, vc = proj.view(B, L, 6, heads, d).permute(2, 0, 3, 1, 4).unbind(0)
+    out2, U2 = H().castle_attention_hip(qc, kc, vc, qu, ku, vu, d ** -0.5, True)
+    merged2 = out2.permute(0, 2, 1, 3).reshape(B, L, heads * d)
+    merged2.backward(dmerged)
+    assert torch.equal(merged, merged2) and torch.equal(U, U2)
+    assert torch.equal(g_packed, proj.grad)
+
+
+DEC_CASES = [(2, 2, 0, 40, 64, torch.float32), (2, 2, 100, 30, 64, torch.float32), (1, 3, 300, 20, 16, torch.float32),
+             (1, 2, 70, 10, 32, torch.float32), (2, 2, 200, 20, 64, torch.bfloat16), (1, 2, 130, 10, 128, torch.bfloat16)]
+
+
+@pytest.mark.parametrize("B,Hh,t0,steps,d,dtype", DEC_CASES)
+def test_decode_steps(B, Hh, t0, steps, d, dtype):
+    L = t0 + steps
+    ops, _ = rand_ops(B, Hh, L, d, dtype, seed=11 * L + d)
+    s = d ** -0.5
+    ref = [t.double() for t in ops]
+    ref_out, ref_U = O.parallel_core(*ref, s, want_U=True)
+    bufs = [torch.zeros(B, Hh, L + 3, d, dtype=dtype, device=DEV) for _ in range(4)]
+    if t0:
+        _, U0 = O.parallel_core(*[t[:, :, :t0] for t in ref], s, want_U=True)
+        for buf, src in zip(bufs, (U0.to(dtype), ops[3][:, :, :t0], ops[1][:, :, :t0], ops[2][:, :, :t0])):
+            buf[:, :, :t0] = src.to(DEV)
+    ws = H().decode_workspace(B, Hh, d, DEV)
+    dev_ops = [t.to(DEV) for t in ops]
+    outs = []
+    for t in range(t0, L):
+        o = torch.empty(B, Hh, 1, d, dtype=dtype, device=DEV)
+        H().castle_decode_step_hip(*bufs, t, *[x[:, :, t:t + 1] for x in dev_ops], s, o, ws)
+        outs.append(o)
+    got = torch.cat(outs, 2)
+    assert_close(got, ref_out[:, :, t0:], dtype, "decode out", 1e-3)
+    if dtype == torch.float32:
+        assert_close(bufs[0][:, :, :L], ref_U, dtype, "U", 1e-3)
+    assert torch.equal(bufs[1][:, :, :L].cpu(), ops[3]) and torch.equal(bufs[2][:, :, :L].cpu(), ops[1])
+    assert torch.equal(bufs[3][:, :, :L].cpu(), ops[2])
