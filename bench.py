@@ -1,0 +1,229 @@
+#!/usr/bin/env python3
+"""Benchmark of the CASTLE hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-decode] [--no-cpu]
+
+Workload (BASELINE config 2): one Castle layer (dim 512, 8 heads, dim_head 64), bf16,
+x and the upstream gradient ~ N(0,1) of shape (4, 4096, 512), seeded random-init weights;
+one step = forward + backward of the layer (projection GEMMs included), inputs resident in
+HBM.  Prints ONE JSON line:
+  value        layer TFLOP/s = (19*B*H*L^2*d core flop + projection GEMM flop) / step time
+  core         the same for the attention core alone, from per-kernel HIP-event times
+  roofline     the longest-running kernel against the bf16 MFMA peak (2.5 PFLOP/s)
+  decode       BASELINE config 4 (B32, prefill 2048, 512 cached steps): tokens/s and the decode
+               stream kernel against the HBM peak (8 TB/s)
+  cpu_baseline the CPU oracle (dense PyTorch restatement of the reference's non-Triton path)
+               on a bounded sample of the same workload, host cores stated
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16/fp16 MFMA
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+# algorithmic contractions (unit: B*H*L^2*d flop = 2*d flop per causal pair) attributed to each kernel
+KERNEL_UNITS = {"tqv": 0.0, "scan": 2.0, "attn": 3.0, "delta": 0.0, "bwd_key": 9.0, "bwd_query": 4.0}
+
+
+def cfg2_flops(B, H, L, d, dim):
+    unit = float(B) * H * L * L * d
+    core = 19.0 * unit
+    gemm = 3.0 * (2.0 * B * L * dim * 6 * H * d + 2.0 * B * L * H * d * dim)
+    return unit, core, gemm
+
+
+def bench_layer(steps, warmup):
+    import torch
+
+    from lookahead_keys_attention_amd import Castle, _native
+
+    dev = torch.device("cuda:0")
+    B, L, dim, H, d = 4, 4096, 512, 8, 64
+    torch.manual_seed(0)
+    model = Castle(dim, heads=H, dim_head=d, use_triton=True).to(dev).bfloat16()
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(B, L, dim, generator=g).bfloat16().to(dev).requires_grad_()
+    gy = torch.randn(B, L, dim, generator=g).bfloat16().to(dev)
+
+    def step():
+        model.zero_grad(set_to_none=True)
+        x.grad = None
+        y = model(x)
+        y.backward(gy)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
+
+    # per-kernel durations: HIP events recorded by the library on the launch stream
+    _native.profile_enable(True)
+    for _ in range(steps):
+        step()
+    records = _native.profile_read()
+    _native.profile_enable(False)
+    per = {}
+    for name, ms in records:
+        per.setdefault(name, []).append(ms)
+    kernels = {k: sum(v) / len(v) for k, v in per.items()}
+    unit, core, gemm = cfg2_flops(B, H, L, d, dim)
+    core_ms = sum(kernels.values())
+    table = {k: {"ms": round(v, 4), "tflops": round(KERNEL_UNITS[k] * unit / (v * 1e-3) / 1e12, 2)} for k, v in kernels.items()}
+    dom = max(kernels, key=kernels.get)
+    achieved = KERNEL_UNITS[dom] * unit / (kernels[dom] * 1e-3) / 1e12
+    return {
+        "ms_per_step": ms_per_step,
+        "value": (core + gemm) / (ms_per_step * 1e-3) / 1e12,
+        "core": {"flop": core, "ms": round(core_ms, 4), "tflops": round(core / (core_ms * 1e-3) / 1e12, 2),
+                 "frac_of_peak": round(core / (core_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4), "kernels": table},
+        "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None},
+        "global_batch": B, "seq_len": L,
+    }
+
+
+def bench_decode(n_steps=512, prefill=2048):
+    import torch
+
+    from lookahead_keys_attention_amd import Castle, _native
+
+    dev = torch.device("cuda:0")
+    B, dim, H, d = 32, 512, 8, 64
+    torch.manual_seed(0)
+    model = Castle(dim, heads=H, dim_head=d, use_triton=True).to(dev).bfloat16().eval()
+    g = torch.Generator().manual_seed(1)
+    x0 = torch.randn(B, prefill, dim, generator=g).bfloat16().to(dev)
+    xs = torch.randn(B, n_steps, dim, generator=g).bfloat16().to(dev)
+    out = {}
+    with torch.no_grad():
+        for timed in (False, True):            # first round warms up, second is timed
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            _, cache = model(x0, return_next_cache=True)
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            for t in range(n_steps):
+                _, cache = model(xs[:, t:t + 1], cache=cache)
+            torch.cuda.synchronize()
+            t2 = time.perf_counter()
+        out["prefill_tokens_per_s"] = B * prefill / (t1 - t0)
+        out["tokens_per_s"] = B * n_steps / (t2 - t1)
+        out["ms_per_decode_step"] = (t2 - t1) * 1e3 / n_steps
+        # kernel-level: bytes the stream kernel must move per step, B*H*(5*t*d + 8*d)*2, against its duration
+        _, cache = model(x0, return_next_cache=True)
+        _native.profile_enable(True)
+        for t in range(n_steps):
+            _, cache = model(xs[:, t:t + 1], cache=cache)
+        rec = _native.profile_read()
+        _native.profile_enable(False)
+    stream_ms = [ms for name, ms in rec if name == "decode_stream"]
+    finish_ms = [ms for name, ms in rec if name == "decode_finish"]
+    bytes_total = sum(B * H * (5 * (prefill + i) * d + 8 * d) * 2 for i in range(len(stream_ms)))
+    kern_s = (sum(stream_ms) + sum(finish_ms)) * 1e-3
+    gbs = bytes_total / (sum(stream_ms) * 1e-3) / 1e9
+    out["kernel_ms_per_step"] = round(kern_s * 1e3 / max(1, len(stream_ms)), 4)
+    out["kernel_tokens_per_s"] = round(B * len(stream_ms) / kern_s, 1)
+    out["roofline"] = {"bound": "hbm", "kernel": "decode_stream", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
+                       "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None}
+    out["workload"] = f"config 4: B{B} H{H} d{d} bf16, prefill {prefill}, {n_steps} cached steps"
+    for k in ("prefill_tokens_per_s", "tokens_per_s", "ms_per_decode_step"):
+        out[k] = round(out[k], 3)
+    return out
+
+
+def cpu_baseline(budget_s=20.0):
+    """Dense oracle (fp32, autograd backward) on single heads of config 2, as many as fit the budget."""
+    import torch
+
+    from oracle import castle_oracle as O
+
+    cores = os.cpu_count() or 1
+    try:
+        cores = min(cores, len(os.sched_getaffinity(0)))
+    except AttributeError:
+        pass
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    L, d = 4096, 64
+    g = torch.Generator().manual_seed(0)
+    done, t_used = 0, 0.0
+    while done < 32 and (done == 0 or t_used + t_used / done < budget_s):
+        ops = [(torch.randn(L, d, generator=g) * 0.6).requires_grad_() for _ in range(6)]
+        do = torch.randn(L, d, generator=g)
+        t0 = time.perf_counter()
+        out = O.parallel_core(*ops, d ** -0.5)
+        out.backward(do)
+        t_used += time.perf_counter() - t0
+        done += 1
+    flop = 19.0 * L * L * d * done
+    return {"value": round(flop / t_used / 1e12, 5), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"{done} of 32 (batch, head) slices of config 2, dense fp32 forward + autograd backward, "
+                      f"{t_used:.1f} s; same algorithmic flop count (19*L^2*d per slice)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-decode", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (no collectives, no sharding); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from lookahead_keys_attention_amd import _native
+
+    if not _native.is_built():
+        from lookahead_keys_attention_amd.build import build
+
+        build()
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+
+    layer = bench_layer(args.steps, args.warmup)
+    line = {
+        "metric": "CASTLE fwd+bwd TFLOP/s (bf16, L=4096)",
+        "value": round(layer["value"], 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(layer["ms_per_step"], 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "config 2: one Castle layer forward+backward, dim 512, 8 heads, dim_head 64, "
+                               "batch 4, seq 4096, bf16 tensors (fp16 MFMA operands, fp32 accumulation)",
+                   "global_batch": layer["global_batch"], "seq_len": layer["seq_len"], "parallelism": "single GPU"},
+        "core": layer["core"],
+        "roofline": layer["roofline"],
+    }
+    if not args.no_decode:
+        line["decode"] = bench_decode()
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

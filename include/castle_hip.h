@@ -107,6 +107,16 @@ int castle_decode_step(const castle_view4* U, const castle_view4* qu_cache,
                        const castle_view4* out,
                        void* workspace, int64_t workspace_bytes, void* stream);
 
+/* Per-kernel timing (no counterpart in the reference; for benchmarks).  While enabled, every
+ * kernel launched by the entry points above is bracketed by a HIP event pair on its stream.
+ * castle_profile_enable(on) also discards pending records.  castle_profile_read waits for the
+ * recorded kernels, writes up to max_records (slot, milliseconds) pairs in launch order, clears
+ * the records and returns their number (< 0 on error).  Slots: 0 T-blocks, 1 forward scan,
+ * 2 forward attention, 3 delta, 4 backward key-stationary, 5 backward query-stationary,
+ * 6 decode stream, 7 decode finish. */
+int castle_profile_enable(int on);
+int castle_profile_read(int* slots, float* ms, int max_records);
+
 #ifdef __cplusplus
 }
 #endif

@@ -28,6 +28,8 @@ EXPORTED_SYMBOLS = (
     "castle_bwd",
     "castle_decode_workspace_bytes",
     "castle_decode_step",
+    "castle_profile_enable",
+    "castle_profile_read",
 )
 
 
@@ -63,6 +65,10 @@ def _declare(lib):
     lib.castle_fwd.argtypes = [_VP] * 6 + [i, i, i, i, i, f, i, _VP, _VP, vp, i64, vp]
     lib.castle_bwd.restype = i
     lib.castle_bwd.argtypes = [_VP] * 8 + [i, i, i, i, i, f, i] + [_VP] * 6 + [vp, i64, vp, i64, vp]
+    lib.castle_profile_enable.restype = i
+    lib.castle_profile_enable.argtypes = [i]
+    lib.castle_profile_read.restype = i
+    lib.castle_profile_read.argtypes = [ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_float), i]
     lib.castle_decode_step.restype = i
     lib.castle_decode_step.argtypes = [_VP] * 4 + [i] + [_VP] * 6 + [i, i, i, i, f, _VP, vp, i64, vp]
 
@@ -123,3 +129,18 @@ def vector_ok(t: torch.Tensor) -> bool:
 
 def stream_ptr(device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
+
+
+PROFILE_SLOTS = ("tqv", "scan", "attn", "delta", "bwd_key", "bwd_query", "decode_stream", "decode_finish")
+
+
+def profile_enable(on: bool):
+    check(lib().castle_profile_enable(1 if on else 0), "castle_profile_enable")
+
+
+def profile_read(max_records: int = 65536):
+    """[(slot name, milliseconds), ...] of the kernels launched since profiling was enabled."""
+    slots = (ctypes.c_int * max_records)()
+    ms = (ctypes.c_float * max_records)()
+    n = check(lib().castle_profile_read(slots, ms, max_records), "castle_profile_read")
+    return [(PROFILE_SLOTS[slots[i]], ms[i]) for i in range(n)]

@@ -16,7 +16,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "libcastle_hip.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
-SOURCES = ("castle_fwd.hip", "castle_bwd.hip", "castle_decode.hip", "castle_abi.hip")
+SOURCES = ("castle_fwd.hip", "castle_bwd.hip", "castle_decode.hip", "castle_profile.hip", "castle_abi.hip")
 ARCH = "gfx950"
 # packed fp32 VALU instructions stay disabled on purpose (hipcc's host pass warns that it
 # does not know the feature; that warning is harmless)

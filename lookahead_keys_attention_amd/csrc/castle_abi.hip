@@ -5,6 +5,7 @@
 
 #include "../../include/castle_hip.h"
 #include "castle_params.h"
+#include "castle_profile.h"
 #include "castle_tiles.h"
 
 namespace castle {
@@ -217,6 +218,13 @@ int castle_decode_step(const castle_view4* U, const castle_view4* qu_cache,
   a.out = to_view(out);
   a.part = static_cast<float*>(workspace);
   return castle::launch_decode(a, dtype, static_cast<hipStream_t>(stream));
+}
+
+int castle_profile_enable(int on) { return castle::profile_enable(on); }
+
+int castle_profile_read(int* slots, float* ms, int max_records) {
+  if (slots == nullptr || ms == nullptr || max_records < 0) return CASTLE_ERR_ARG;
+  return castle::profile_read(slots, ms, max_records);
 }
 
 }  // extern "C"

@@ -19,6 +19,7 @@
 //   dKu = s^2 dZ_raw^T Qu;  dVu = s (A^T G_raw + dT^T Qc),   dZ_raw = dA_raw A (1 - A).
 #include "castle_tiles.h"
 #include "castle_params.h"
+#include "castle_profile.h"
 
 namespace castle {
 
@@ -634,9 +635,18 @@ template <typename T, typename TI, int HD> static int launch_bwd_t(const BwdArgs
     configured = true;
   }
   constexpr int RPB = kThreads / (HD / elem_traits<T>::vec16);
-  hipLaunchKernelGGL((delta_kernel<TI, HD>), dim3((a.s.Lp + RPB - 1) / RPB, BH), dim3(kThreads), 0, stream, a);
-  hipLaunchKernelGGL((bwd_key_kernel<T, TI, HD>), dim3(a.s.Lp / 128, BH), dim3(kThreads), key_lds, stream, a);
-  hipLaunchKernelGGL((bwd_query_kernel<T, TI, HD>), dim3(a.s.Lp / 128, BH), dim3(kThreads), query_lds, stream, a);
+  {
+    ProfScope ps(kSlotDelta, stream);
+    hipLaunchKernelGGL((delta_kernel<TI, HD>), dim3((a.s.Lp + RPB - 1) / RPB, BH), dim3(kThreads), 0, stream, a);
+  }
+  {
+    ProfScope ps(kSlotBwdKey, stream);
+    hipLaunchKernelGGL((bwd_key_kernel<T, TI, HD>), dim3(a.s.Lp / 128, BH), dim3(kThreads), key_lds, stream, a);
+  }
+  {
+    ProfScope ps(kSlotBwdQuery, stream);
+    hipLaunchKernelGGL((bwd_query_kernel<T, TI, HD>), dim3(a.s.Lp / 128, BH), dim3(kThreads), query_lds, stream, a);
+  }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 

@@ -10,6 +10,7 @@
 // decode_finish_kernel merges the partials, folds in row t and appends the new rows.
 #include "castle_tiles.h"
 #include "castle_params.h"
+#include "castle_profile.h"
 
 namespace castle {
 
@@ -180,8 +181,14 @@ __global__ __launch_bounds__(64) void decode_finish_kernel(DecodeArgs a) {
 
 template <typename T, int HD> static int launch_decode_t(const DecodeArgs& a, hipStream_t stream) {
   const int BH = a.B * a.H;
-  if (a.t > 0) hipLaunchKernelGGL((decode_stream_kernel<T, HD>), dim3(a.splits, BH), dim3(kThreads), 0, stream, a);
-  hipLaunchKernelGGL((decode_finish_kernel<T, HD>), dim3(BH), dim3(64), 0, stream, a);
+  if (a.t > 0) {
+    ProfScope ps(kSlotDecodeStream, stream);
+    hipLaunchKernelGGL((decode_stream_kernel<T, HD>), dim3(a.splits, BH), dim3(kThreads), 0, stream, a);
+  }
+  {
+    ProfScope ps(kSlotDecodeFinish, stream);
+    hipLaunchKernelGGL((decode_finish_kernel<T, HD>), dim3(BH), dim3(64), 0, stream, a);
+  }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 

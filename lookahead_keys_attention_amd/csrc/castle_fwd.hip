@@ -13,6 +13,7 @@
 // reference; operands stay unscaled and the softmax scale is applied in fp32.
 #include "castle_tiles.h"
 #include "castle_params.h"
+#include "castle_profile.h"
 
 namespace castle {
 
@@ -318,9 +319,18 @@ template <typename T, typename TI, int HD> static int launch_fwd_t(const FwdArgs
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_kernel<T, TI, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, attn_lds) != hipSuccess) return -3;
     configured = true;
   }
-  hipLaunchKernelGGL((tqv_kernel<T, TI, HD>), dim3(a.s.nblk, BH), dim3(kThreads), 0, stream, a);
-  hipLaunchKernelGGL((scan_kernel<T, TI, HD>), dim3(a.s.Lp / 128, BH), dim3(kThreads), scan_lds, stream, a);
-  hipLaunchKernelGGL((attn_kernel<T, TI, HD>), dim3(a.s.Lp / 128, BH), dim3(kThreads), attn_lds, stream, a);
+  {
+    ProfScope ps(kSlotTqv, stream);
+    hipLaunchKernelGGL((tqv_kernel<T, TI, HD>), dim3(a.s.nblk, BH), dim3(kThreads), 0, stream, a);
+  }
+  {
+    ProfScope ps(kSlotScan, stream);
+    hipLaunchKernelGGL((scan_kernel<T, TI, HD>), dim3(a.s.Lp / 128, BH), dim3(kThreads), scan_lds, stream, a);
+  }
+  {
+    ProfScope ps(kSlotAttn, stream);
+    hipLaunchKernelGGL((attn_kernel<T, TI, HD>), dim3(a.s.Lp / 128, BH), dim3(kThreads), attn_lds, stream, a);
+  }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
