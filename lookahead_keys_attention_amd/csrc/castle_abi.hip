@@ -77,7 +77,8 @@ castle::View4 to_view(const castle_view4* v) {
 int check_core(int B, int H, int L, int d, int dtype) {
   if (elem_size(dtype) == 0) return CASTLE_ERR_DTYPE;
   if (B <= 0 || H <= 0 || L <= 0 || !head_dim_ok(d)) return CASTLE_ERR_SHAPE;
-  if ((int64_t)B * H > 65535) return CASTLE_ERR_SHAPE;   // grid.y
+  if ((int64_t)B * H > 65535) return CASTLE_ERR_SHAPE;   // grid.y of the small kernels
+  if ((int64_t)B * H * ((L + 127) / 128) > 2147483647LL) return CASTLE_ERR_SHAPE;   // 1-D grid
   if (dtype == CASTLE_F32 && d > 64) return CASTLE_ERR_SHAPE;
   return CASTLE_OK;
 }

@@ -149,7 +149,9 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   float* s_lse = cv.take<float>(kNB);
   float* s_delta = cv.take<float>(kNB);
 
-  const int kb = blockIdx.x, bh = blockIdx.y, b = bh / a.s.H, h = bh % a.s.H;
+  int kb, bh;   // key group 0 meets every query block: rank order = kb
+  work_item(a.s.B * a.s.H, kb, bh);
+  const int b = bh / a.s.H, h = bh % a.s.H;
   const int lane = lane_id(), wave = wave_id(), c = lane & 31, g = lane >> 5;
   const int L = a.s.L;
   const float c0 = a.s.scale, c1 = a.s.scale * kLog2e;
@@ -380,8 +382,10 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
   T* s_at = s_a;
   if constexpr (TC) s_at = cv.take<T>(QB * LDC);
 
-  const int qb = gridDim.x - 1 - blockIdx.x;
-  const int bh = blockIdx.y, b = bh / a.s.H, h = bh % a.s.H;
+  int rank, bh;
+  work_item(a.s.B * a.s.H, rank, bh);
+  const int qb = a.s.Lp / 128 - 1 - rank;   // the last row block meets the most keys
+  const int b = bh / a.s.H, h = bh % a.s.H;
   const int lane = lane_id(), wave = wave_id(), c = lane & 31, g = lane >> 5;
   const int L = a.s.L;
   const float c0 = a.s.scale, c1 = a.s.scale * kLog2e;
@@ -641,11 +645,11 @@ template <typename T, typename TI, int HD> static int launch_bwd_t(const BwdArgs
   }
   {
     ProfScope ps(kSlotBwdKey, stream);
-    hipLaunchKernelGGL((bwd_key_kernel<T, TI, HD>), dim3(a.s.Lp / 128, BH), dim3(kThreads), key_lds, stream, a);
+    hipLaunchKernelGGL((bwd_key_kernel<T, TI, HD>), dim3(a.s.Lp / 128 * BH), dim3(kThreads), key_lds, stream, a);
   }
   {
     ProfScope ps(kSlotBwdQuery, stream);
-    hipLaunchKernelGGL((bwd_query_kernel<T, TI, HD>), dim3(a.s.Lp / 128, BH), dim3(kThreads), query_lds, stream, a);
+    hipLaunchKernelGGL((bwd_query_kernel<T, TI, HD>), dim3(a.s.Lp / 128 * BH), dim3(kThreads), query_lds, stream, a);
   }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }

@@ -78,7 +78,9 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(FwdArgs a) {
   T* s_ku = reinterpret_cast<T*>(castle_smem);   // [kNB][LDK]
   T* s_vut = s_ku + kNB * LDK;                   // [HDP][LDV]
 
-  const int kb = blockIdx.x, bh = blockIdx.y, b = bh / a.s.H, h = bh % a.s.H;
+  int kb, bh;   // key group 0 sweeps every source block: rank order = kb
+  work_item(a.s.B * a.s.H, kb, bh);
+  const int b = bh / a.s.H, h = bh % a.s.H;
   const int lane = lane_id(), wave = wave_id(), c = lane & 31, g = lane >> 5;
   const int L = a.s.L;
   const float c1 = a.s.scale * kLog2e;
@@ -164,8 +166,10 @@ __global__ __launch_bounds__(kThreads) void attn_kernel(FwdArgs a) {
   T* s_vct = s_ub0 + NBLK_Q * kNB * LDK;         // [HDP][LDV]
   T* s_a = s_vct + HDP * LDV;                    // [kNB][LDA]
 
-  const int qb = gridDim.x - 1 - blockIdx.x;   // longest rows first
-  const int bh = blockIdx.y, b = bh / a.s.H, h = bh % a.s.H;
+  int rank, bh;
+  work_item(a.s.B * a.s.H, rank, bh);
+  const int qb = a.s.Lp / 128 - 1 - rank;   // the last query block sees the most keys
+  const int b = bh / a.s.H, h = bh % a.s.H;
   const int lane = lane_id(), wave = wave_id(), c = lane & 31, g = lane >> 5;
   const int L = a.s.L;
   const float c1 = a.s.scale * kLog2e;
@@ -325,11 +329,11 @@ template <typename T, typename TI, int HD> static int launch_fwd_t(const FwdArgs
   }
   {
     ProfScope ps(kSlotScan, stream);
-    hipLaunchKernelGGL((scan_kernel<T, TI, HD>), dim3(a.s.Lp / 128, BH), dim3(kThreads), scan_lds, stream, a);
+    hipLaunchKernelGGL((scan_kernel<T, TI, HD>), dim3(a.s.Lp / 128 * BH), dim3(kThreads), scan_lds, stream, a);
   }
   {
     ProfScope ps(kSlotAttn, stream);
-    hipLaunchKernelGGL((attn_kernel<T, TI, HD>), dim3(a.s.Lp / 128, BH), dim3(kThreads), attn_lds, stream, a);
+    hipLaunchKernelGGL((attn_kernel<T, TI, HD>), dim3(a.s.Lp / 128 * BH), dim3(kThreads), attn_lds, stream, a);
   }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }

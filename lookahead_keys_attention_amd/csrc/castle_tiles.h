@@ -184,6 +184,17 @@ __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcp
 // sigmoid(y) given z = y * log2(e)
 __device__ __forceinline__ float sigmoid_l2(float z) { return fast_rcp(1.f + fast_exp2(-z)); }
 
+// Work-item order of the row-block kernels.  The grid is 1-D with nrow * BH workgroups; item
+// `id` maps to row block `rank = id / BH` of head `bh = id % BH`.  Callers order `rank` from the
+// longest row block to the shortest, so across ALL heads the expensive blocks are dispatched
+// first (the causal triangle otherwise leaves a long tail), and because workgroups are dealt
+// round-robin to the 8 XCDs, head bh always lands on XCD (bh % 8) whenever BH is a multiple of
+// 8: the K/V/state rows of one head stay in one L2.
+__device__ __forceinline__ void work_item(int BH, int& rank, int& bh) {
+  rank = blockIdx.x / BH;
+  bh = blockIdx.x % BH;
+}
+
 // offsets (in rows) of block I inside the snapshot arrays
 __host__ __device__ inline int64_t usnap_off(int64_t I) { return (int64_t)kNB * I * (I - 1) / 2; }   // I >= 1, I*kNB rows
 __host__ __device__ inline int64_t gsnap_off(int64_t I) { return (int64_t)kNB * I * (I + 1) / 2; }   // I <= nblk-2, (I+1)*kNB rows
