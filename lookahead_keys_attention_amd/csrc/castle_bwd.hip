@@ -13,10 +13,14 @@
 //                     keys streamed in chunks of 32: dQc (rows as queries) and dKu, dVu
 //                     (rows as lookahead sources), using the forward snapshots usnap and gsnap.
 //
-// Units: operands stay unscaled.  With s = softmax scale, Su = s Su_raw etc.
-//   dS, dSu are d/dS, d/dSu of the true scores;  dA_raw = dSu^T T_raw + G_raw Vu^T;
-//   dKc = s dS^T Qc;  dVc = P^T dO;  dQu = s^2 dZ_raw Ku;  dQc = s (dS Kc + dSu U + dT Vu);
-//   dKu = s^2 dZ_raw^T Qu;  dVu = s (A^T G_raw + dT^T Qc),   dZ_raw = dA_raw A (1 - A).
+// Units (s = softmax scale, c1 = s log2 e).  As in the forward pass the resident query operand is
+// Qc' = c1 Qc, the stored T blocks are T' = c1 tril(Qc Vu^T) and the resident gate operand is
+// multiplied by -c1, so scores come out of the MFMA in log2 units.  dS and dSu are the gradients
+// with respect to the TRUE scores.  Everything that is built from Qc' or T' carries a factor c1:
+//   G' = sum dSu^T Qc' = c1 G,   dA' = dSu^T T' + G' Vu^T = c1 dA,   dZ' = dA' A (1 - A)
+// and the outputs are rescaled once at the end:
+//   dKc = ln2 (dS^T Qc')      dVc = P^T dO              dQu = s ln2 (dZ' Ku)
+//   dQc = s (dS Kc + dSu U + dT Vu)   dKu = s ln2 (dZ'^T Qu)   dVu = ln2 (A^T G' + dT^T Qc')
 #include "castle_tiles.h"
 #include "castle_params.h"
 #include "castle_profile.h"
@@ -114,11 +118,12 @@ template <typename T, int HD> constexpr int bwd_key_lds_bytes() {
   constexpr int HDP = HD < 32 ? 32 : HD;
   constexpr bool TC = sizeof(T) == 2;
   int b = 0;
-  b += 4 * a16((int)sizeof(T) * kNB * lds_ld<T>(HD));     // qc, do, ku, vu
-  b += a16((int)sizeof(T) * kNB * lds_ld<T>(kNB));        // T
+  b += 3 * a16((int)sizeof(T) * kNB * lds_ld<T>(HD));           // qc, do, ku
+  b += a16((int)sizeof(T) * kNB * lds_ld_chain<T>(HD));         // vu
+  b += a16((int)sizeof(T) * kNB * lds_ld_chain<T>(kNB));        // T
   if (TC) {
-    b += 3 * a16((int)sizeof(T) * HDP * lds_ld<T>(kNB));  // qc^T, do^T, ku^T
-    b += a16((int)sizeof(T) * kNB * lds_ld<T>(kNB));      // T^T
+    b += 3 * a16((int)sizeof(T) * HDP * lds_ld_chain<T>(kNB));  // qc^T, do^T, ku^T
+    b += a16((int)sizeof(T) * kNB * lds_ld_chain<T>(kNB));      // T^T
   }
   b += 2 * a16(4 * kNB);                                  // lse, delta
   return b;
@@ -131,13 +136,13 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   constexpr int NT = HDP / 32;
   constexpr int BT = kNB / 32;   // 32-row sub-tiles per block
   constexpr bool TC = sizeof(T) == 2;
-  constexpr int LDK = lds_ld<T>(HD), LDV = lds_ld<T>(kNB), LDT = lds_ld<T>(kNB);
+  constexpr int LDK = lds_ld<T>(HD), LDU = lds_ld_chain<T>(HD), LDV = lds_ld_chain<T>(kNB), LDT = lds_ld_chain<T>(kNB);
 
   Carver cv{castle_smem};
   T* s_qc = cv.take<T>(kNB * LDK);
   T* s_do = cv.take<T>(kNB * LDK);
   T* s_ku = cv.take<T>(kNB * LDK);
-  T* s_vu = cv.take<T>(kNB * LDK);
+  T* s_vu = cv.take<T>(kNB * LDU);
   T* s_t = cv.take<T>(kNB * LDT);
   T* s_qct = s_qc; T* s_dot = s_do; T* s_kut = s_ku; T* s_tt = s_t;
   if constexpr (TC) {
@@ -158,6 +163,7 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   const int kw0 = kb * 128 + 32 * wave;
   const int k = kw0 + c;
   const int Iw = kw0 / kNB;
+  const int sgroup = wave >> 1, slt = threadIdx.x & 127;   // staging group and index inside it
   const TI* qc = head_ptr<TI>(a.qc, b, h);
   const TI* kc = head_ptr<TI>(a.kc, b, h);
   const TI* vc = head_ptr<TI>(a.vc, b, h);
@@ -177,7 +183,7 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   for (int s = 0; s < KS; ++s) {
     fkc[s] = ldg_nat<T, TI>(kc, a.kc.sl, k, 16 * s + 8 * g, k < L);
     fvc[s] = ldg_nat<T, TI>(vc, a.vc.sl, k, 16 * s + 8 * g, k < L);
-    fqu[s] = ldg_nat<T, TI>(qu, a.qu.sl, k, 16 * s + 8 * g, k < L);
+    fqu[s] = ldg_nat_scaled<T, TI>(qu, a.qu.sl, k, 16 * s + 8 * g, k < L, -c1);
     fub[s] = zero_frag<T>();
   }
   acc_t dvc[NT], dkc[NT], dqu[NT], G[NT];   // [n rows, k lanes]
@@ -208,16 +214,28 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
     }
     __syncthreads();
     const int64_t r0 = (int64_t)I * kNB;
-    stage_rows<T, kNB, HD, TI>(s_qc, qc, a.qc.sl, r0, L);
-    stage_rows<T, kNB, HD, TI>(s_do, dout, a.dout.sl, r0, L);
-    stage_rows<T, kNB, HD, TI>(s_ku, ku, a.ku.sl, r0, L);
-    stage_rows<T, kNB, HD, TI>(s_vu, vu, a.vu.sl, r0, L);
-    stage_rows<T, kNB, kNB>(s_t, tb, kNB, r0, (int64_t)1 << 40);
-    if constexpr (TC) {
-      stage_rows_t<T, kNB, HD, TI>(s_qct, qc, a.qc.sl, r0, L);
-      stage_rows_t<T, kNB, HD, TI>(s_dot, dout, a.dout.sl, r0, L);
-      stage_rows_t<T, kNB, HD, TI>(s_kut, ku, a.ku.sl, r0, L);
-      stage_rows<T, kNB, kNB>(s_tt, ttb, kNB, r0, (int64_t)1 << 40);
+    // two thread groups (waves 0-1 / waves 2-3) stage three tiles each; all loads are issued first
+    {
+      PatchStage<T, TI, kNB, HD, 128> pa, pb;
+      PatchStage<T, T, kNB, kNB, 128> pt;
+      if (sgroup == 0) {
+        pa.load(slt, qc, a.qc.sl, r0, L);
+        pb.load(slt, ku, a.ku.sl, r0, L);
+        pt.load(slt, tb, kNB, r0, (int64_t)1 << 40);
+        pa.store_rows(slt, s_qc, LDK, c1);
+        if constexpr (TC) pa.store_cols(slt, s_qct, LDV, c1);
+        pb.store_rows(slt, s_ku, LDK);
+        if constexpr (TC) pb.store_cols(slt, s_kut, LDV);
+        pt.template store_rows<true>(slt, s_t, LDT);
+      } else {
+        pa.load(slt, dout, a.dout.sl, r0, L);
+        pb.load(slt, vu, a.vu.sl, r0, L);
+        if constexpr (TC) pt.load(slt, ttb, kNB, r0, (int64_t)1 << 40);
+        pa.store_rows(slt, s_do, LDK);
+        if constexpr (TC) pa.store_cols(slt, s_dot, LDV);
+        pb.template store_rows<true>(slt, s_vu, LDU);
+        if constexpr (TC) pt.template store_rows<true>(slt, s_tt, LDT);
+      }
     }
     if (threadIdx.x < kNB) {
       const int64_t i = r0 + threadIdx.x;
@@ -237,10 +255,11 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
       for (int s = 0; s < KS; ++s) mma(aT[jt], ld_nat<T>(s_ku, LDK, 32 * jt + c, 16 * s + 8 * g), fqu[s]);
       const int j0 = I * kNB + 32 * jt;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float v = sigmoid_l2(aT[jt][r] * c1);
-        if (j0 + acc_row(r, g) <= k) v = 0.f;
-        aT[jt][r] = v;
+      for (int r = 0; r < 16; ++r) aT[jt][r] = fast_rcp(1.f + fast_exp2(aT[jt][r]));
+      if (j0 <= kw0 + 31) {   // tile touches the diagonal: keep j > k only
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if (j0 + acc_row(r, g) <= k) aT[jt][r] = 0.f;
       }
       fa[jt][0] = chain<T>(aT[jt], 0);
       fa[jt][1] = chain<T>(aT[jt], 1);
@@ -252,7 +271,7 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
       zero(dA[jt]);
 #pragma unroll
       for (int s = 0; s < KS; ++s)
-        mma(dA[jt], ld_chain<T>(s_vu, LDK, 32 * jt + c, 16 * s, g), chain<T>(G[s / 2], s % 2));
+        mma(dA[jt], ld_chain<T>(s_vu, LDU, 32 * jt + c, 16 * s, g), chain<T>(G[s / 2], s % 2));
     }
     // (c) query sub-tiles of the block
 #pragma unroll
@@ -275,15 +294,16 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
         for (int s2 = 0; s2 < 2; ++s2) mma(su, ld_chain<T>(s_t, LDT, 32 * it + c, 32 * jt + 16 * s2, g), fa[jt][s2]);
       }
       acc_t ds, dsu;
+      const bool diag = i0 < kw0 + 31;   // tile touches the diagonal
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int il = 32 * it + acc_row(r, g);
-        const float sg = sigmoid_l2(su[r] * c1);
+        const float sg = fast_rcp(1.f + fast_exp2(-su[r]));
         const float x = __builtin_fmaf(-su[r], sg, sc[r]);
-        float p = fast_exp2(__builtin_fmaf(x, c1, -s_lse[il]));
-        if (I * kNB + il < k) p = 0.f;
+        float p = fast_exp2(x - s_lse[il]);
+        if (diag && I * kNB + il < k) p = 0.f;
         const float dsv = p * (dp[r] - s_delta[il]);
-        const float y = su[r] * c0;
+        const float y = su[r] * kLn2;                     // true Su
         const float t = __builtin_fmaf(-y, sg, y);        // y (1 - sigmoid)
         const float sp = __builtin_fmaf(sg, t, sg);       // silu'(y)
         sc[r] = p;
@@ -324,9 +344,9 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
     }
   }
   if (k < L) {
-    store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dkc, b, h) + (int64_t)k * a.dkc.sl, dkc, c0, g);
+    store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dkc, b, h) + (int64_t)k * a.dkc.sl, dkc, kLn2, g);
     store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvc, b, h) + (int64_t)k * a.dvc.sl, dvc, 1.f, g);
-    store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqu, b, h) + (int64_t)k * a.dqu.sl, dqu, c0 * c0, g);
+    store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqu, b, h) + (int64_t)k * a.dqu.sl, dqu, c0 * kLn2, g);
   }
 }
 
@@ -338,13 +358,13 @@ template <typename T, int HD> constexpr int bwd_query_lds_bytes() {
   constexpr bool TC = sizeof(T) == 2;
   int b = 0;
   b += 7 * a16((int)sizeof(T) * kCK * lds_ld<T>(HD));            // kc, vc, qu, ub[2], g[2]
-  if (TC) b += 6 * a16((int)sizeof(T) * HDP * lds_ld<T>(kCK));   // kc^T, qu^T, ub^T[2], g^T[2]
-  b += 2 * a16((int)sizeof(T) * kCK * lds_ld<T>(128));           // A, dSu
-  if (TC) b += a16((int)sizeof(T) * 128 * lds_ld<T>(kCK));       // A^T
-  // epilogue (reuses the same memory): vu[2] (+^T), qc[2] (+^T), dT[2]
+  if (TC) b += 6 * a16((int)sizeof(T) * HDP * lds_ld_chain<T>(kCK));   // kc^T, qu^T, ub^T[2], g^T[2]
+  b += 2 * a16((int)sizeof(T) * kCK * lds_ld<T>(128));                 // A, dSu
+  if (TC) b += a16((int)sizeof(T) * 128 * lds_ld_chain<T>(kCK));       // A^T
+  // epilogue (reuses the same memory): vu[2], qc[2], vu^T[2], qc^T[2], dT[2]
   int e = 0;
   e += 4 * a16((int)sizeof(T) * kNB * lds_ld<T>(HD));
-  if (TC) e += 4 * a16((int)sizeof(T) * HDP * lds_ld<T>(kNB));
+  if (TC) e += 2 * a16((int)sizeof(T) * HDP * lds_ld_chain<T>(kNB)) + 2 * a16((int)sizeof(T) * HDP * lds_ld<T>(kNB));
   e += 2 * a16((int)sizeof(T) * kNB * lds_ld<T>(kNB));
   return b > e ? b : e;
 }
@@ -359,8 +379,8 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
   constexpr int QB = 128;
   constexpr int NQ = QB / kNB;
   constexpr bool TC = sizeof(T) == 2;
-  constexpr int LDK = lds_ld<T>(HD), LDC = lds_ld<T>(kCK), LDA = lds_ld<T>(QB);
-  constexpr int LDV = lds_ld<T>(kNB), LDT = lds_ld<T>(kNB);
+  constexpr int LDK = lds_ld<T>(HD), LDC = lds_ld_chain<T>(kCK), LDA = lds_ld<T>(QB);
+  constexpr int LDV = lds_ld_chain<T>(kNB), LDQ = lds_ld<T>(kNB), LDT = lds_ld<T>(kNB);
 
   Carver cv{castle_smem};
   T* s_kc = cv.take<T>(kCK * LDK);
@@ -416,9 +436,9 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
   frag<T> fqc[KS], fdo[KS], fku[KS], fvu[KS], ft[TS], ftt[TS];
 #pragma unroll
   for (int s = 0; s < KS; ++s) {
-    fqc[s] = ldg_nat<T, TI>(qc, a.qc.sl, i, 16 * s + 8 * g, i < L);
+    fqc[s] = ldg_nat_scaled<T, TI>(qc, a.qc.sl, i, 16 * s + 8 * g, i < L, c1);
     fdo[s] = ldg_nat<T, TI>(dout, a.dout.sl, i, 16 * s + 8 * g, i < L);
-    fku[s] = ldg_nat<T, TI>(ku, a.ku.sl, i, 16 * s + 8 * g, i < L);
+    fku[s] = ldg_nat_scaled<T, TI>(ku, a.ku.sl, i, 16 * s + 8 * g, i < L, -c1);
     fvu[s] = ldg_nat<T, TI>(vu, a.vu.sl, i, 16 * s + 8 * g, i < L);
   }
 #pragma unroll
@@ -449,26 +469,32 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
   for (int k0 = 0; k0 < kend; k0 += kCK) {
     const int Kb = k0 / kNB;
     __syncthreads();
-    stage_rows<T, kCK, HD, TI>(s_kc, kc, a.kc.sl, k0, L);
-    stage_rows<T, kCK, HD, TI>(s_vc, vc, a.vc.sl, k0, L);
-    stage_rows<T, kCK, HD, TI>(s_qu, qu, a.qu.sl, k0, L);
-    if constexpr (TC) {
-      stage_rows_t<T, kCK, HD, TI>(s_kct, kc, a.kc.sl, k0, L);
-      stage_rows_t<T, kCK, HD, TI>(s_qut, qu, a.qu.sl, k0, L);
-    }
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) {
+    // one wave per tile: wave 0 kc + ub[0], wave 1 qu + ub[1], wave 2 vc + g[0], wave 3 g[1]
+    {
+      PatchStage<T, TI, kCK, HD, 64> pi;
+      PatchStage<T, T, kCK, HD, 64> pw;
+      const int q = wave & 1;                       // which of the two row blocks the workspace tile serves
       const int blk = Ifirst + q;
-      if (blk >= a.s.nblk) continue;
-      if (Kb < blk) {
-        const T* src = usnap + usnap_off(blk) * HD;
-        stage_rows<T, kCK, HD>(s_ub[q], src, HD, k0, (int64_t)1 << 40);
-        if constexpr (TC) stage_rows_t<T, kCK, HD>(s_ubt[q], src, HD, k0, (int64_t)1 << 40);
+      const bool want_u = wave < 2 && blk < a.s.nblk && Kb < blk;
+      const bool want_g = wave >= 2 && blk <= a.s.nblk - 2 && Kb <= blk;
+      const TI* isrc = wave == 0 ? kc : (wave == 1 ? qu : vc);
+      const int64_t istride = wave == 0 ? a.kc.sl : (wave == 1 ? a.qu.sl : a.vc.sl);
+      if (wave < 3) pi.load(lane, isrc, istride, k0, L);
+      if (want_u) pw.load(lane, usnap + usnap_off(blk) * HD, HD, k0, (int64_t)1 << 40);
+      if (want_g) pw.load(lane, gsnap + gsnap_off(blk) * HD, HD, k0, (int64_t)1 << 40);
+      if (wave < 3) {
+        pi.store_rows(lane, wave == 0 ? s_kc : (wave == 1 ? s_qu : s_vc), LDK);
+        if constexpr (TC) {
+          if (wave < 2) pi.store_cols(lane, wave == 0 ? s_kct : s_qut, LDC);
+        }
       }
-      if (Kb <= blk && blk <= a.s.nblk - 2) {
-        const T* src = gsnap + gsnap_off(blk) * HD;
-        stage_rows<T, kCK, HD>(s_g[q], src, HD, k0, (int64_t)1 << 40);
-        if constexpr (TC) stage_rows_t<T, kCK, HD>(s_gt[q], src, HD, k0, (int64_t)1 << 40);
+      if (want_u) {
+        pw.store_rows(lane, s_ub[q], LDK);
+        if constexpr (TC) pw.store_cols(lane, s_ubt[q], LDC);
+      }
+      if (want_g) {
+        pw.store_rows(lane, s_g[q], LDK);
+        if constexpr (TC) pw.store_cols(lane, s_gt[q], LDC);
       }
     }
     __syncthreads();
@@ -481,12 +507,14 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
 #pragma unroll
       for (int s = 0; s < KS; ++s) mma(aK, ld_nat<T>(s_qu, LDK, c, 16 * s + 8 * g), fku[s]);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float v = sigmoid_l2(aK[r] * c1);
-        if (i <= k0 + acc_row(r, g)) v = 0.f;
-        aK[r] = v;
-        s_a[acc_row(r, g) * LDA + jw + c] = (T)v;
+      for (int r = 0; r < 16; ++r) aK[r] = fast_rcp(1.f + fast_exp2(aK[r]));
+      if (k0 + 31 >= i0w) {   // chunk reaches the diagonal: keep j > k only
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if (i <= k0 + acc_row(r, g)) aK[r] = 0.f;
       }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s_a[acc_row(r, g) * LDA + jw + c] = (T)aK[r];
       if constexpr (TC) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) st4<T>(s_at + (jw + c) * LDC + 8 * q + 4 * g, pack4<T>(aK, q));
@@ -508,14 +536,15 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
       for (int s = 0; s < TS; ++s)
         if (s < nintra) mma(su, ld_nat<T>(s_a, LDA, c, cb + 16 * s + 8 * g), ft[s]);
       acc_t ds, dsu;
+      const bool diag = k0 + 31 > i0w;   // chunk reaches the diagonal
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const float sg = sigmoid_l2(su[r] * c1);
+        const float sg = fast_rcp(1.f + fast_exp2(-su[r]));
         const float x = __builtin_fmaf(-su[r], sg, sc[r]);
-        float p = fast_exp2(__builtin_fmaf(x, c1, -lse2));
-        if (k0 + acc_row(r, g) > i) p = 0.f;
+        float p = fast_exp2(x - lse2);
+        if (diag && k0 + acc_row(r, g) > i) p = 0.f;
         const float dsv = p * (dp[r] - dlt);
-        const float y = su[r] * c0;
+        const float y = su[r] * kLn2;                     // true Su
         const float t = __builtin_fmaf(-y, sg, y);
         const float sp = __builtin_fmaf(sg, t, sg);
         ds[r] = dsv;
@@ -573,21 +602,23 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
   for (int q = 0; q < NQ; ++q) { e_vut[q] = e_vu[q]; e_qct[q] = e_qc[q]; }
   if constexpr (TC) {
     for (int q = 0; q < NQ; ++q) e_vut[q] = ce.take<T>(HDP * LDV);
-    for (int q = 0; q < NQ; ++q) e_qct[q] = ce.take<T>(HDP * LDV);
+    for (int q = 0; q < NQ; ++q) e_qct[q] = ce.take<T>(HDP * LDQ);
   }
   for (int q = 0; q < NQ; ++q) e_dt[q] = ce.take<T>(kNB * LDT);
 #pragma unroll
   for (int q = 0; q < NQ; ++q) {
     const int64_t r0 = (int64_t)(Ifirst + q) * kNB;
-    stage_rows<T, kNB, HD, TI>(e_vu[q], vu, a.vu.sl, r0, L);
-    stage_rows<T, kNB, HD, TI>(e_qc[q], qc, a.qc.sl, r0, L);
+    RowStage<T, TI, kNB, HD> st;
+    st.load(vu, a.vu.sl, r0, L); st.store(e_vu[q], LDK);
+    st.load(qc, a.qc.sl, r0, L); st.store_scaled(e_qc[q], LDK, c1);
     if constexpr (TC) {
       if (HDP > HD) {
         lds_zero(e_vut[q] + HD * LDV, (HDP - HD) * LDV);
-        lds_zero(e_qct[q] + HD * LDV, (HDP - HD) * LDV);
+        lds_zero(e_qct[q] + HD * LDQ, (HDP - HD) * LDQ);
       }
-      stage_rows_t<T, kNB, HD, TI>(e_vut[q], vu, a.vu.sl, r0, L);
-      stage_rows_t<T, kNB, HD, TI>(e_qct[q], qc, a.qc.sl, r0, L);
+      ColStage<T, TI, kNB, HD> ct;
+      ct.load(vu, a.vu.sl, r0, L); ct.store(e_vut[q], LDV);
+      ct.load(qc, a.qc.sl, r0, L); ct.store(e_qct[q], LDQ, c1);
     }
   }
   // dT^T[j rows, i lanes] masked to j <= i, shared as e_dt[j][i] for the source-side product
@@ -618,12 +649,12 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
     const frag<T> fdt = ld_nat<T>(e_dt[qw], LDT, lw + c, 16 * s + 8 * g);   // (source j, queries i)
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
-      mma(dvu[nt], ld_tr_nat<T>(e_qct[qw], LDV, e_qc[qw], LDK, 32 * nt + c, HD, 16 * s, g), fdt);
+      mma(dvu[nt], ld_tr_nat<T>(e_qct[qw], LDQ, e_qc[qw], LDK, 32 * nt + c, HD, 16 * s, g), fdt);
   }
   if (i < L) {
     store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqc, b, h) + (int64_t)i * a.dqc.sl, dqc, c0, g);
-    store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dku, b, h) + (int64_t)i * a.dku.sl, dku, c0 * c0, g);
-    store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvu, b, h) + (int64_t)i * a.dvu.sl, dvu, c0, g);
+    store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dku, b, h) + (int64_t)i * a.dku.sl, dku, c0 * kLn2, g);
+    store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvu, b, h) + (int64_t)i * a.dvu.sl, dvu, kLn2, g);
   }
 }
 

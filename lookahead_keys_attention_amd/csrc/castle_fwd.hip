@@ -10,7 +10,8 @@
 //                  Su = Qc_I usnap[I][K]^T + T_II A_KI^T,  S = s(Sc - Su sigmoid(s Su)),
 //                online softmax over keys, O = P Vc.
 // The math follows the dense definition at lookahead_keys_attention.py:132-164 of the
-// reference; operands stay unscaled and the softmax scale is applied in fp32.
+// reference.  The softmax scale (times log2 e) is folded once into the operand fragments each
+// wave keeps in registers; K/V/state operands stay unscaled.
 #include "castle_tiles.h"
 #include "castle_params.h"
 #include "castle_profile.h"
@@ -19,12 +20,20 @@ namespace castle {
 
 extern __shared__ __attribute__((aligned(16))) unsigned char castle_smem[];
 
+// Units.  With c1 = scale * log2(e) the kernels work on "log2-domain" scores:
+//   Qc' = c1 Qc            so that  Sc' = Qc' Kc^T        = c1 * (Qc Kc^T)
+//   T'  = tril(Qc' Vu^T)   so that  Su' = Qc' U^T + T' A^T = log2(e) * Su
+//   gate operand (Qu or Ku, whichever is resident) is multiplied by -c1, so that
+//   A = 1 / (1 + exp2(acc)) needs no multiply.
+// Then sigmoid(Su) = 1/(1+exp2(-Su')), S' = Sc' - Su' sigmoid(Su) = log2(e) S, P = exp2(S' - m').
 template <typename T, int HD> constexpr int scan_lds_bytes() {
-  return (int)sizeof(T) * (kNB * lds_ld<T>(HD) + (HD < 32 ? 32 : HD) * lds_ld<T>(kNB));
+  return (int)sizeof(T) * (kNB * lds_ld<T>(HD) + (HD < 32 ? 32 : HD) * lds_ld_chain<T>(kNB));
 }
 template <typename T, int HD> constexpr int attn_lds_bytes() {
-  return (int)sizeof(T) * (4 * kNB * lds_ld<T>(HD) + (HD < 32 ? 32 : HD) * lds_ld<T>(kNB) + kNB * lds_ld<T>(128));
+  return (int)sizeof(T) * (4 * kNB * lds_ld<T>(HD) + (HD < 32 ? 32 : HD) * lds_ld_chain<T>(kNB) + kNB * lds_ld<T>(128));
 }
+// register prefetch of the next tile is affordable for 16-bit operands up to d = 64
+template <typename T, int HD> constexpr bool use_prefetch() { return sizeof(T) == 2 && HD <= 64; }
 
 template <typename T> __device__ __forceinline__ const T* head_ptr(const View4& v, int b, int h) {
   return reinterpret_cast<const T*>(v.ptr) + (int64_t)b * v.sb + (int64_t)h * v.sh;
@@ -40,6 +49,7 @@ __global__ __launch_bounds__(kThreads) void tqv_kernel(FwdArgs a) {
   constexpr int TB = kNB / 32;
   const int I = blockIdx.x, bh = blockIdx.y, b = bh / a.s.H, h = bh % a.s.H;
   const int lane = lane_id(), c = lane & 31, g = lane >> 5;
+  const float c1 = a.s.scale * kLog2e;
   const TI* qc = head_ptr<TI>(a.qc, b, h);
   const TI* vu = head_ptr<TI>(a.vu, b, h);
   T* tb = reinterpret_cast<T*>(a.ws.t_blk) + (int64_t)bh * a.s.Lp * kNB;
@@ -53,12 +63,12 @@ __global__ __launch_bounds__(kThreads) void tqv_kernel(FwdArgs a) {
 #pragma unroll
     for (int s = 0; s < KS; ++s)
       mma(acc, ldg_nat<T, TI>(qc, a.qc.sl, i, 16 * s + 8 * g, i < a.s.L), ldg_nat<T, TI>(vu, a.vu.sl, j, 16 * s + 8 * g, j < a.s.L));
-    // acc[r] = T[il = 32 it + acc_row][jl = 32 jt + c]
+    // acc[r] = (Qc Vu^T)[il = 32 it + acc_row][jl = 32 jt + c]; stored as T' = c1 * tril(.)
     const int jl = 32 * jt + c;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int il = 32 * it + acc_row(r, g);
-      if (jl > il) acc[r] = 0.f;
+      acc[r] = jl > il ? 0.f : acc[r] * c1;
       tb[((int64_t)I * kNB + il) * kNB + jl] = (T)acc[r];
     }
 #pragma unroll
@@ -74,7 +84,8 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(FwdArgs a) {
   constexpr int HDP = HD < 32 ? 32 : HD;
   constexpr int NT = HDP / 32;
   constexpr int JT = kNB / 32;
-  constexpr int LDK = lds_ld<T>(HD), LDV = lds_ld<T>(kNB);
+  constexpr int LDK = lds_ld<T>(HD), LDV = lds_ld_chain<T>(kNB);
+  constexpr bool PF = use_prefetch<T, HD>();
   T* s_ku = reinterpret_cast<T*>(castle_smem);   // [kNB][LDK]
   T* s_vut = s_ku + kNB * LDK;                   // [HDP][LDV]
 
@@ -91,15 +102,21 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(FwdArgs a) {
   const TI* vu = head_ptr<TI>(a.vu, b, h);
   T* snap = reinterpret_cast<T*>(a.ws.usnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
 
-  frag<T> fq[KS];
+  frag<T> fq[KS];   // -c1 * Qu rows of this wave
 #pragma unroll
-  for (int s = 0; s < KS; ++s) fq[s] = ldg_nat<T, TI>(qu, a.qu.sl, k, 16 * s + 8 * g, k < L);
+  for (int s = 0; s < KS; ++s) fq[s] = ldg_nat_scaled<T, TI>(qu, a.qu.sl, k, 16 * s + 8 * g, k < L, -c1);
   acc_t st[NT];   // state^T : rows n (head dim), columns k (lanes)
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) zero(st[nt]);
   if (HDP > HD) lds_zero(s_vut + HD * LDV, (HDP - HD) * LDV);
 
+  RowStage<T, TI, kNB, HD> pku;
+  ColStage<T, TI, kNB, HD> pvu;
   const int I0 = (kb * 128) / kNB;
+  if (PF) {
+    pku.load(ku, a.ku.sl, (int64_t)I0 * kNB, L);
+    pvu.load(vu, a.vu.sl, (int64_t)I0 * kNB, L);
+  }
   for (int I = I0; I < a.s.nblk; ++I) {
     if (I * kNB >= kw0 + 32) {   // all keys of this wave precede block I: snapshot
       T* dst = snap + (usnap_off(I) + k) * HD;
@@ -112,8 +129,16 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(FwdArgs a) {
         }
     }
     __syncthreads();
-    stage_rows<T, kNB, HD, TI>(s_ku, ku, a.ku.sl, (int64_t)I * kNB, L);
-    stage_rows_t<T, kNB, HD, TI>(s_vut, vu, a.vu.sl, (int64_t)I * kNB, L);
+    if (!PF) {
+      pku.load(ku, a.ku.sl, (int64_t)I * kNB, L);
+      pvu.load(vu, a.vu.sl, (int64_t)I * kNB, L);
+    }
+    pku.store(s_ku, LDK);
+    pvu.store(s_vut, LDV);
+    if (PF && I + 1 < a.s.nblk) {   // in flight while this block is processed
+      pku.load(ku, a.ku.sl, (int64_t)(I + 1) * kNB, L);
+      pvu.load(vu, a.vu.sl, (int64_t)(I + 1) * kNB, L);
+    }
     __syncthreads();
 #pragma unroll
     for (int jt = 0; jt < JT; ++jt) {
@@ -123,12 +148,12 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(FwdArgs a) {
       zero(aT);
 #pragma unroll
       for (int s = 0; s < KS; ++s) mma(aT, ld_nat<T>(s_ku, LDK, 32 * jt + c, 16 * s + 8 * g), fq[s]);
-      const bool diag = j0 <= kw0 + 31;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float v = sigmoid_l2(aT[r] * c1);
-        if (diag && j0 + acc_row(r, g) <= k) v = 0.f;
-        aT[r] = v;
+      for (int r = 0; r < 16; ++r) aT[r] = fast_rcp(1.f + fast_exp2(aT[r]));
+      if (j0 <= kw0 + 31) {           // tile touches the diagonal: keep j > k only
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if (j0 + acc_row(r, g) <= k) aT[r] = 0.f;
       }
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
@@ -152,14 +177,15 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(FwdArgs a) {
 
 // ---------------------------------------------------------------------------
 template <typename T, typename TI, int HD>
-__global__ __launch_bounds__(kThreads) void attn_kernel(FwdArgs a) {
+__global__ __launch_bounds__(kThreads, (sizeof(T) == 2 && HD <= 64) ? 2 : 1) void attn_kernel(FwdArgs a) {
   constexpr int KS = HD / 16;
   constexpr int HDP = HD < 32 ? 32 : HD;
   constexpr int NT = HDP / 32;
   constexpr int KT = kNB / 32;
   constexpr int QB = 128;
   constexpr int NBLK_Q = QB / kNB;   // snapshot blocks per workgroup
-  constexpr int LDK = lds_ld<T>(HD), LDV = lds_ld<T>(kNB), LDA = lds_ld<T>(QB);
+  constexpr int LDK = lds_ld<T>(HD), LDV = lds_ld_chain<T>(kNB), LDA = lds_ld<T>(QB);
+  constexpr bool PF = use_prefetch<T, HD>();
   T* s_kc = reinterpret_cast<T*>(castle_smem);   // [kNB][LDK]
   T* s_qu = s_kc + kNB * LDK;                    // [kNB][LDK]
   T* s_ub0 = s_qu + kNB * LDK;                   // [NBLK_Q][kNB][LDK]
@@ -189,11 +215,11 @@ __global__ __launch_bounds__(kThreads) void attn_kernel(FwdArgs a) {
   const T* tb = reinterpret_cast<const T*>(a.ws.t_blk) + (int64_t)bh * a.s.Lp * kNB;
   const T* snap = reinterpret_cast<const T*>(a.ws.usnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
 
-  frag<T> fqc[KS], fku[KS], ft[kNB / 16];
+  frag<T> fqc[KS], fku[KS], ft[kNB / 16];   // c1 Qc rows, -c1 Ku rows, T' rows of this wave
 #pragma unroll
   for (int s = 0; s < KS; ++s) {
-    fqc[s] = ldg_nat<T, TI>(qc, a.qc.sl, i, 16 * s + 8 * g, i < L);
-    fku[s] = ldg_nat<T, TI>(ku, a.ku.sl, i, 16 * s + 8 * g, i < L);
+    fqc[s] = ldg_nat_scaled<T, TI>(qc, a.qc.sl, i, 16 * s + 8 * g, i < L, c1);
+    fku[s] = ldg_nat_scaled<T, TI>(ku, a.ku.sl, i, 16 * s + 8 * g, i < L, -c1);
   }
 #pragma unroll
   for (int s = 0; s < kNB / 16; ++s) ft[s] = ldg_nat<T>(tb, kNB, i, 16 * s + 8 * g, s < nintra);
@@ -206,17 +232,37 @@ __global__ __launch_bounds__(kThreads) void attn_kernel(FwdArgs a) {
 
   int nchunks = (qb * QB + QB) / kNB;
   if (nchunks > a.s.nblk) nchunks = a.s.nblk;
-  for (int Kb = 0; Kb < nchunks; ++Kb) {
-    __syncthreads();
-    stage_rows<T, kNB, HD, TI>(s_kc, kc, a.kc.sl, (int64_t)Kb * kNB, L);
-    stage_rows_t<T, kNB, HD, TI>(s_vct, vc, a.vc.sl, (int64_t)Kb * kNB, L);
-    stage_rows<T, kNB, HD, TI>(s_qu, qu, a.qu.sl, (int64_t)Kb * kNB, L);
+
+  RowStage<T, TI, kNB, HD> pkc, pqu;
+  ColStage<T, TI, kNB, HD> pvc;
+  RowStage<T, T, kNB, HD> pub[NBLK_Q];
+  auto load_chunk = [&](int Kb) {
+    pkc.load(kc, a.kc.sl, (int64_t)Kb * kNB, L);
+    pvc.load(vc, a.vc.sl, (int64_t)Kb * kNB, L);
+    pqu.load(qu, a.qu.sl, (int64_t)Kb * kNB, L);
 #pragma unroll
     for (int q = 0; q < NBLK_Q; ++q) {
       const int blk = Ifirst + q;
-      if (Kb < blk && blk < a.s.nblk)
-        stage_rows<T, kNB, HD>(s_ub0 + q * kNB * LDK, snap + usnap_off(blk) * HD, HD, (int64_t)Kb * kNB, (int64_t)1 << 40);
+      if (Kb < blk && blk < a.s.nblk) pub[q].load(snap + usnap_off(blk) * HD, HD, (int64_t)Kb * kNB, (int64_t)1 << 40);
     }
+  };
+  auto store_chunk = [&](int Kb) {
+    pkc.store(s_kc, LDK);
+    pvc.store(s_vct, LDV);
+    pqu.store(s_qu, LDK);
+#pragma unroll
+    for (int q = 0; q < NBLK_Q; ++q) {
+      const int blk = Ifirst + q;
+      if (Kb < blk && blk < a.s.nblk) pub[q].store(s_ub0 + q * kNB * LDK, LDK);
+    }
+  };
+
+  if (PF) load_chunk(0);
+  for (int Kb = 0; Kb < nchunks; ++Kb) {
+    __syncthreads();
+    if (!PF) load_chunk(Kb);
+    store_chunk(Kb);
+    if (PF && Kb + 1 < nchunks) load_chunk(Kb + 1);   // in flight while this chunk is processed
     __syncthreads();
     const bool active = Kb <= Iw;
     if (active) {
@@ -227,16 +273,16 @@ __global__ __launch_bounds__(kThreads) void attn_kernel(FwdArgs a) {
         zero(aT);
 #pragma unroll
         for (int s = 0; s < KS; ++s) mma(aT, fku[s], ld_nat<T>(s_qu, LDK, 32 * kt + c, 16 * s + 8 * g));
-        const int kk = Kb * kNB + 32 * kt + c;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          float v = sigmoid_l2(aT[r] * c1);
-          if (i0w + acc_row(r, g) <= kk) v = 0.f;
-          aT[r] = v;
+        for (int r = 0; r < 16; ++r) aT[r] = fast_rcp(1.f + fast_exp2(aT[r]));
+        if (Kb == Iw) {
+          const int kk = Kb * kNB + 32 * kt + c;
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            if (i0w + acc_row(r, g) <= kk) aT[r] = 0.f;
         }
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
-          st4<T>(s_a + (32 * kt + c) * LDA + jw + 8 * q + 4 * g, pack4<T>(aT, q));
+        for (int q = 0; q < 4; ++q) st4<T>(s_a + (32 * kt + c) * LDA + jw + 8 * q + 4 * g, pack4<T>(aT, q));
       }
     }
     __syncthreads();
@@ -259,32 +305,36 @@ __global__ __launch_bounds__(kThreads) void attn_kernel(FwdArgs a) {
         for (int s = 0; s < kNB / 16; ++s)
           if (s < nintra) mma(su, ld_nat<T>(s_a, LDA, 32 * kt + c, cb + 16 * s + 8 * g), ft[s]);
 
-        const bool diag = k0 + 31 > i0w;
+        // scores in log2 units: x = Sc' - Su' * sigmoid(Su)
         float mx = -INFINITY;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const float sg = sigmoid_l2(su[r] * c1);
-          float x = __builtin_fmaf(-su[r], sg, sc[r]);
-          if (diag && k0 + acc_row(r, g) > i) x = -INFINITY;
-          sc[r] = x;
-          mx = fmaxf(mx, x);
+          const float sg = fast_rcp(1.f + fast_exp2(-su[r]));
+          sc[r] = __builtin_fmaf(-su[r], sg, sc[r]);
         }
+        if (k0 + 31 > i0w) {   // tile touches the diagonal: causal mask
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            if (k0 + acc_row(r, g) > i) sc[r] = -INFINITY;
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sc[r]);
         mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m, mx * c1);
-        const float alpha = fast_exp2(m - m_new);
-        float ls = 0.f;
+        if (__builtin_amdgcn_ballot_w64(mx > m) != 0) {   // some row maximum moved: rescale
+          const float m_new = fmaxf(m, mx);
+          const float alpha = fast_exp2(m - m_new);
+          l *= alpha;
+          m = m_new;
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[nt][r] *= alpha;
+        }
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const float pv = fast_exp2(__builtin_fmaf(sc[r], c1, -m_new));
-          sc[r] = pv;
-          ls += pv;
+          sc[r] = fast_exp2(sc[r] - m);
+          l += sc[r];
         }
-        l = l * alpha + ls;
-        m = m_new;
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) o[nt][r] *= alpha;
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
           const frag<T> fp = chain<T>(sc, s2);

@@ -82,6 +82,9 @@ template <typename T> __device__ __forceinline__ frag<T> chain(const acc_t& c, i
   return __builtin_convertvector(v, frag<T>);
 }
 
+// store 4 packed elements (8 bytes for 16-bit types, 16 for fp32)
+template <typename T> __device__ __forceinline__ void st4(T* p, vec<T, 4> v) { *reinterpret_cast<vec4_mem<T>*>(p) = v; }
+
 // 8 contiguous elements tile[row][col .. col+7]
 template <typename T> __device__ __forceinline__ frag<T> ld_nat(const T* tile, int ld, int row, int col) {
   return *reinterpret_cast<const frag_mem<T>*>(tile + row * ld + col);
@@ -170,8 +173,6 @@ template <typename T> __device__ __forceinline__ void lds_zero(T* dst, int count
   for (int i = threadIdx.x * 8; i < count; i += kThreads * 8) *reinterpret_cast<frag_mem<T>*>(dst + i) = zero_frag<T>();
 }
 
-// store 4 packed elements (8 bytes for 16-bit types, 16 for fp32)
-template <typename T> __device__ __forceinline__ void st4(T* p, vec<T, 4> v) { *reinterpret_cast<vec4_mem<T>*>(p) = v; }
 
 // 4 consecutive rows (registers 4q..4q+3) of an accumulator tile as a packed vector of T
 template <typename T> __device__ __forceinline__ vec<T, 4> pack4(const acc_t& c, int q) {
@@ -183,6 +184,220 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 // sigmoid(y) given z = y * log2(e)
 __device__ __forceinline__ float sigmoid_l2(float z) { return fast_rcp(1.f + fast_exp2(-z)); }
+
+// natural fragment from global memory multiplied by `mul` in fp32 before the conversion to T
+template <typename T, typename TI = T>
+__device__ __forceinline__ frag<T> ldg_nat_scaled(const TI* base, int64_t row_stride, int64_t row, int col, bool ok, float mul) {
+  if (!ok) return zero_frag<T>();
+  vec<float, 8> v = __builtin_convertvector(*reinterpret_cast<const frag_mem<TI>*>(base + row * row_stride + col), vec<float, 8>);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] *= mul;
+  return __builtin_convertvector(v, frag<T>);
+}
+
+// leading dimension of a tile that is read with ld_chain (8-byte halves): 8 bytes of pad for
+// 16-bit types make both the transposed stores and the chained reads bank-conflict free
+template <typename T> __host__ __device__ constexpr int lds_ld_chain(int cols) { return cols + 4; }
+
+// Two-phase staging of a ROWS x COLS tile: load() brings the 16-byte pieces of this thread into
+// registers (zeros beyond row_end), store() converts them to T and writes the row-major LDS tile.
+// Splitting the phases lets a kernel issue the loads of the next tile before computing on the
+// current one.
+template <typename T, typename TI, int ROWS, int COLS>
+struct RowStage {
+  static constexpr int V = elem_traits<T>::vec16;
+  static constexpr int VPR = COLS / V;
+  static constexpr int TOTAL = ROWS * VPR;
+  static constexpr int N = (TOTAL + kThreads - 1) / kThreads;
+  vec<TI, V> r[N];
+
+  __device__ __forceinline__ void load(const TI* src, int64_t row_stride, int64_t row0, int64_t row_end) {
+#pragma unroll
+    for (int n = 0; n < N; ++n) {
+      const int v = threadIdx.x + n * kThreads;
+#pragma unroll
+      for (int e = 0; e < V; ++e) r[n][e] = (TI)0.f;
+      if (v < TOTAL && row0 + v / VPR < row_end)
+        r[n] = *reinterpret_cast<const vec<TI, V>*>(src + (row0 + v / VPR) * row_stride + (v % VPR) * V);
+    }
+  }
+  __device__ __forceinline__ void store(T* dst, int ld) const {
+#pragma unroll
+    for (int n = 0; n < N; ++n) {
+      const int v = threadIdx.x + n * kThreads;
+      if (v < TOTAL) *reinterpret_cast<vec<T, V>*>(dst + (v / VPR) * ld + (v % VPR) * V) = cvt_vec<T, TI, V>(r[n]);
+    }
+  }
+  // for tiles whose rows are only 8-byte aligned (leading dimension from lds_ld_chain)
+  __device__ __forceinline__ void store_halves(T* dst, int ld) const {
+    constexpr int HV = V / 2;
+#pragma unroll
+    for (int n = 0; n < N; ++n) {
+      const int v = threadIdx.x + n * kThreads;
+      if (v < TOTAL) {
+        const vec<T, V> x = cvt_vec<T, TI, V>(r[n]);
+        typedef vec<T, HV> __attribute__((aligned(8))) half_mem;
+        vec<T, HV> lo, hi;
+#pragma unroll
+        for (int e = 0; e < HV; ++e) { lo[e] = x[e]; hi[e] = x[HV + e]; }
+        T* q = dst + (v / VPR) * ld + (v % VPR) * V;
+        *reinterpret_cast<half_mem*>(q) = lo;
+        *reinterpret_cast<half_mem*>(q + HV) = hi;
+      }
+    }
+  }
+  __device__ __forceinline__ void store_scaled(T* dst, int ld, float mul) const {
+#pragma unroll
+    for (int n = 0; n < N; ++n) {
+      const int v = threadIdx.x + n * kThreads;
+      if (v < TOTAL) {
+        vec<float, V> f = __builtin_convertvector(r[n], vec<float, V>);
+#pragma unroll
+        for (int e = 0; e < V; ++e) f[e] *= mul;
+        *reinterpret_cast<vec<T, V>*>(dst + (v / VPR) * ld + (v % VPR) * V) = __builtin_convertvector(f, vec<T, V>);
+      }
+    }
+  }
+};
+
+// Same for the transposed copy dst[c][r] = src[row0 + r][c].  A thread owns 4 rows x V columns.
+// Lane -> patch map: within 16 consecutive lanes the patches cover 2 column groups x 8 row
+// groups, which makes the 8-byte LDS stores hit 16 distinct bank pairs while every load
+// instruction of a wave still reads 8 complete rows.
+template <typename T, typename TI, int ROWS, int COLS>
+struct ColStage {
+  static constexpr int V = elem_traits<T>::vec16;
+  static constexpr int VPR = COLS / V;
+  static constexpr int RG = ROWS / 4;
+  static constexpr int TOTAL = RG * VPR;
+  static constexpr int N = (TOTAL + kThreads - 1) / kThreads;
+  static_assert(VPR % 2 == 0 && RG % 8 == 0, "tile shape not supported by the patch map");
+  vec<TI, V> r[N][4];
+
+  static __device__ __forceinline__ void patch(int p, int& rg, int& cv) {
+    const int rest = p >> 4;
+    cv = (rest % (VPR / 2)) * 2 + (p & 1);
+    rg = (rest / (VPR / 2)) * 8 + ((p >> 1) & 7);
+  }
+  __device__ __forceinline__ void load(const TI* src, int64_t row_stride, int64_t row0, int64_t row_end) {
+#pragma unroll
+    for (int n = 0; n < N; ++n) {
+      const int p = threadIdx.x + n * kThreads;
+      int rg, cv;
+      patch(p, rg, cv);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+#pragma unroll
+        for (int e = 0; e < V; ++e) r[n][q][e] = (TI)0.f;
+        const int64_t row = row0 + 4 * rg + q;
+        if (p < TOTAL && row < row_end) r[n][q] = *reinterpret_cast<const vec<TI, V>*>(src + row * row_stride + cv * V);
+      }
+    }
+  }
+  __device__ __forceinline__ void store(T* dst, int ld, float mul = 1.f) const {
+#pragma unroll
+    for (int n = 0; n < N; ++n) {
+      const int p = threadIdx.x + n * kThreads;
+      if (p >= TOTAL) continue;
+      int rg, cv;
+      patch(p, rg, cv);
+      vec<float, V> f[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) f[q] = __builtin_convertvector(r[n][q], vec<float, V>);
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        vec<float, 4> y = {f[0][e] * mul, f[1][e] * mul, f[2][e] * mul, f[3][e] * mul};
+        st4<T>(dst + (cv * V + e) * ld + 4 * rg, __builtin_convertvector(y, vec<T, 4>));
+      }
+    }
+  }
+};
+
+// Patch staging: a group of GROUP threads stages one ROWS x COLS tile; a thread owns 4-row x
+// 16-byte patches, loaded once from global memory, from which it can write the row-major LDS
+// tile, the transposed LDS tile, or both.  load() only issues the global loads, so several
+// tiles (one PatchStage each, handled by different waves) are in flight together and the
+// loads of the next tile can be issued before the current one is consumed.  `lt` is the index
+// of the thread inside its group (0 .. GROUP-1).
+template <typename T, typename TI, int ROWS, int COLS, int GROUP>
+struct PatchStage {
+  static constexpr int V = elem_traits<T>::vec16;
+  static constexpr int VPR = COLS / V;
+  static constexpr int RG = ROWS / 4;
+  static constexpr int TOTAL = RG * VPR;
+  static constexpr int N = (TOTAL + GROUP - 1) / GROUP;
+  static_assert(VPR % 2 == 0 && RG % 8 == 0, "tile shape not supported by the patch map");
+  vec<TI, V> r[N][4];
+
+  static __device__ __forceinline__ void patch(int p, int& rg, int& cv) {
+    const int rest = p >> 4;
+    cv = (rest % (VPR / 2)) * 2 + (p & 1);
+    rg = (rest / (VPR / 2)) * 8 + ((p >> 1) & 7);
+  }
+  __device__ __forceinline__ void load(int lt, const TI* src, int64_t row_stride, int64_t row0, int64_t row_end) {
+#pragma unroll
+    for (int n = 0; n < N; ++n) {
+      const int p = lt + n * GROUP;
+      int rg, cv;
+      patch(p, rg, cv);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+#pragma unroll
+        for (int e = 0; e < V; ++e) r[n][q][e] = (TI)0.f;
+        const int64_t row = row0 + 4 * rg + q;
+        if (p < TOTAL && row < row_end) r[n][q] = *reinterpret_cast<const vec<TI, V>*>(src + row * row_stride + cv * V);
+      }
+    }
+  }
+  // row-major tile dst[r][c]; HALVES = true writes 8-byte halves (rows only 8-byte aligned)
+  template <bool HALVES = false>
+  __device__ __forceinline__ void store_rows(int lt, T* dst, int ld, float mul = 1.f) const {
+    constexpr int HV = V / 2;
+    typedef vec<T, HV> __attribute__((aligned(8))) half_mem;
+#pragma unroll
+    for (int n = 0; n < N; ++n) {
+      const int p = lt + n * GROUP;
+      if (p >= TOTAL) continue;
+      int rg, cv;
+      patch(p, rg, cv);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        vec<float, V> f = __builtin_convertvector(r[n][q], vec<float, V>);
+#pragma unroll
+        for (int e = 0; e < V; ++e) f[e] *= mul;
+        const vec<T, V> x = __builtin_convertvector(f, vec<T, V>);
+        T* w = dst + (4 * rg + q) * ld + cv * V;
+        if constexpr (HALVES) {
+          vec<T, HV> lo, hi;
+#pragma unroll
+          for (int e = 0; e < HV; ++e) { lo[e] = x[e]; hi[e] = x[HV + e]; }
+          *reinterpret_cast<half_mem*>(w) = lo;
+          *reinterpret_cast<half_mem*>(w + HV) = hi;
+        } else {
+          *reinterpret_cast<vec<T, V>*>(w) = x;
+        }
+      }
+    }
+  }
+  // transposed tile dst[c][r]
+  __device__ __forceinline__ void store_cols(int lt, T* dst, int ld, float mul = 1.f) const {
+#pragma unroll
+    for (int n = 0; n < N; ++n) {
+      const int p = lt + n * GROUP;
+      if (p >= TOTAL) continue;
+      int rg, cv;
+      patch(p, rg, cv);
+      vec<float, V> f[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) f[q] = __builtin_convertvector(r[n][q], vec<float, V>);
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        vec<float, 4> y = {f[0][e] * mul, f[1][e] * mul, f[2][e] * mul, f[3][e] * mul};
+        st4<T>(dst + (cv * V + e) * ld + 4 * rg, __builtin_convertvector(y, vec<T, 4>));
+      }
+    }
+  }
+};
 
 // Work-item order of the row-block kernels.  The grid is 1-D with nrow * BH workgroups; item
 // `id` maps to row block `rank = id / BH` of head `bh = id % BH`.  Callers order `rank` from the
