@@ -195,7 +195,37 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
     lds_zero(s_kut + HD * LDV, (HDP - HD) * LDV);
   }
 
+  PatchStage<T, TI, kNB, HD, 128> pa, pb;
+  PatchStage<T, T, kNB, kNB, 128> pt;
+  auto stage_load = [&](int I) __attribute__((always_inline)) {
+    const int64_t r0 = (int64_t)I * kNB;
+    if (sgroup == 0) {
+      pa.load(slt, qc, a.qc.sl, r0, L);
+      pb.load(slt, ku, a.ku.sl, r0, L);
+      pt.load(slt, tb, kNB, r0, (int64_t)1 << 40);
+    } else {
+      pa.load(slt, dout, a.dout.sl, r0, L);
+      pb.load(slt, vu, a.vu.sl, r0, L);
+      if constexpr (TC) pt.load(slt, ttb, kNB, r0, (int64_t)1 << 40);
+    }
+  };
+  auto stage_store = [&]() __attribute__((always_inline)) {
+    if (sgroup == 0) {
+      pa.store_rows(slt, s_qc, LDK, c1);
+      if constexpr (TC) pa.store_cols(slt, s_qct, LDV, c1);
+      pb.store_rows(slt, s_ku, LDK);
+      if constexpr (TC) pb.store_cols(slt, s_kut, LDV);
+      pt.template store_rows<true>(slt, s_t, LDT);
+    } else {
+      pa.store_rows(slt, s_do, LDK);
+      if constexpr (TC) pa.store_cols(slt, s_dot, LDV);
+      pb.template store_rows<true>(slt, s_vu, LDU);
+      if constexpr (TC) pt.template store_rows<true>(slt, s_tt, LDT);
+    }
+  };
+
   const int I0 = (kb * 128) / kNB;
+  stage_load(a.s.nblk - 1);
   for (int I = a.s.nblk - 1; I >= I0; --I) {
     const bool active = I >= Iw;
     if (active && I <= a.s.nblk - 2) {   // reverse state as of block I
@@ -214,29 +244,10 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
     }
     __syncthreads();
     const int64_t r0 = (int64_t)I * kNB;
-    // two thread groups (waves 0-1 / waves 2-3) stage three tiles each; all loads are issued first
-    {
-      PatchStage<T, TI, kNB, HD, 128> pa, pb;
-      PatchStage<T, T, kNB, kNB, 128> pt;
-      if (sgroup == 0) {
-        pa.load(slt, qc, a.qc.sl, r0, L);
-        pb.load(slt, ku, a.ku.sl, r0, L);
-        pt.load(slt, tb, kNB, r0, (int64_t)1 << 40);
-        pa.store_rows(slt, s_qc, LDK, c1);
-        if constexpr (TC) pa.store_cols(slt, s_qct, LDV, c1);
-        pb.store_rows(slt, s_ku, LDK);
-        if constexpr (TC) pb.store_cols(slt, s_kut, LDV);
-        pt.template store_rows<true>(slt, s_t, LDT);
-      } else {
-        pa.load(slt, dout, a.dout.sl, r0, L);
-        pb.load(slt, vu, a.vu.sl, r0, L);
-        if constexpr (TC) pt.load(slt, ttb, kNB, r0, (int64_t)1 << 40);
-        pa.store_rows(slt, s_do, LDK);
-        if constexpr (TC) pa.store_cols(slt, s_dot, LDV);
-        pb.template store_rows<true>(slt, s_vu, LDU);
-        if constexpr (TC) pt.template store_rows<true>(slt, s_tt, LDT);
-      }
-    }
+    // two thread groups (waves 0-1 / waves 2-3) stage three tiles each from the registers the
+    // previous iteration filled, then issue the loads of the next block
+    stage_store();
+    if (I > I0) stage_load(I - 1);
     if (threadIdx.x < kNB) {
       const int64_t i = r0 + threadIdx.x;
       s_lse[threadIdx.x] = i < L ? lse[i] * kLog2e : INFINITY;
@@ -464,39 +475,45 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
     }
   }
 
+  PatchStage<T, TI, kCK, HD, 64> pi;
+  PatchStage<T, T, kCK, HD, 64> pw;
+  const int sq = wave & 1;                          // which of the two row blocks the workspace tile serves
+  const int sblk = Ifirst + sq;
+  const TI* isrc = wave == 0 ? kc : (wave == 1 ? qu : vc);
+  const int64_t istride = wave == 0 ? a.kc.sl : (wave == 1 ? a.qu.sl : a.vc.sl);
+// issue the global loads of the chunk that starts at key K0 (each wave its own tiles)
+#define CASTLE_BQ_WANT_U(K0) (wave < 2 && sblk < a.s.nblk && (K0) / kNB < sblk)
+#define CASTLE_BQ_WANT_G(K0) (wave >= 2 && sblk <= a.s.nblk - 2 && (K0) / kNB <= sblk)
+#define CASTLE_BQ_LOAD(K0)                                                                          \
+  do {                                                                                              \
+    if (wave < 3) pi.load(lane, isrc, istride, (K0), L);                                            \
+    if (CASTLE_BQ_WANT_U(K0)) pw.load(lane, usnap + usnap_off(sblk) * HD, HD, (K0), (int64_t)1 << 40); \
+    if (CASTLE_BQ_WANT_G(K0)) pw.load(lane, gsnap + gsnap_off(sblk) * HD, HD, (K0), (int64_t)1 << 40); \
+  } while (0)
+
   int kend = qb * QB + QB;
   if (kend > a.s.Lp) kend = a.s.Lp;
+  CASTLE_BQ_LOAD(0);
   for (int k0 = 0; k0 < kend; k0 += kCK) {
     const int Kb = k0 / kNB;
     __syncthreads();
-    // one wave per tile: wave 0 kc + ub[0], wave 1 qu + ub[1], wave 2 vc + g[0], wave 3 g[1]
-    {
-      PatchStage<T, TI, kCK, HD, 64> pi;
-      PatchStage<T, T, kCK, HD, 64> pw;
-      const int q = wave & 1;                       // which of the two row blocks the workspace tile serves
-      const int blk = Ifirst + q;
-      const bool want_u = wave < 2 && blk < a.s.nblk && Kb < blk;
-      const bool want_g = wave >= 2 && blk <= a.s.nblk - 2 && Kb <= blk;
-      const TI* isrc = wave == 0 ? kc : (wave == 1 ? qu : vc);
-      const int64_t istride = wave == 0 ? a.kc.sl : (wave == 1 ? a.qu.sl : a.vc.sl);
-      if (wave < 3) pi.load(lane, isrc, istride, k0, L);
-      if (want_u) pw.load(lane, usnap + usnap_off(blk) * HD, HD, k0, (int64_t)1 << 40);
-      if (want_g) pw.load(lane, gsnap + gsnap_off(blk) * HD, HD, k0, (int64_t)1 << 40);
-      if (wave < 3) {
-        pi.store_rows(lane, wave == 0 ? s_kc : (wave == 1 ? s_qu : s_vc), LDK);
-        if constexpr (TC) {
-          if (wave < 2) pi.store_cols(lane, wave == 0 ? s_kct : s_qut, LDC);
-        }
-      }
-      if (want_u) {
-        pw.store_rows(lane, s_ub[q], LDK);
-        if constexpr (TC) pw.store_cols(lane, s_ubt[q], LDC);
-      }
-      if (want_g) {
-        pw.store_rows(lane, s_g[q], LDK);
-        if constexpr (TC) pw.store_cols(lane, s_gt[q], LDC);
+    // one wave per tile (wave 0: kc + ub[0], wave 1: qu + ub[1], wave 2: vc + g[0], wave 3: g[1]),
+    // written from the registers the previous iteration filled; then the next chunk's loads go out
+    if (wave < 3) {
+      pi.store_rows(lane, wave == 0 ? s_kc : (wave == 1 ? s_qu : s_vc), LDK);
+      if constexpr (TC) {
+        if (wave < 2) pi.store_cols(lane, wave == 0 ? s_kct : s_qut, LDC);
       }
     }
+    if (CASTLE_BQ_WANT_U(k0)) {
+      pw.store_rows(lane, sq == 0 ? s_ub[0] : s_ub[1], LDK);
+      if constexpr (TC) pw.store_cols(lane, sq == 0 ? s_ubt[0] : s_ubt[1], LDC);
+    }
+    if (CASTLE_BQ_WANT_G(k0)) {
+      pw.store_rows(lane, sq == 0 ? s_g[0] : s_g[1], LDK);
+      if constexpr (TC) pw.store_cols(lane, sq == 0 ? s_gt[0] : s_gt[1], LDC);
+    }
+    if (k0 + kCK < kend) CASTLE_BQ_LOAD(k0 + kCK);
     __syncthreads();
     const bool active = Kb <= Iw;
 

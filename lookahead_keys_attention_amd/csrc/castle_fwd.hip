@@ -236,7 +236,7 @@ __global__ __launch_bounds__(kThreads, (sizeof(T) == 2 && HD <= 64) ? 2 : 1) voi
   RowStage<T, TI, kNB, HD> pkc, pqu;
   ColStage<T, TI, kNB, HD> pvc;
   RowStage<T, T, kNB, HD> pub[NBLK_Q];
-  auto load_chunk = [&](int Kb) {
+  auto load_chunk = [&](int Kb) __attribute__((always_inline)) {
     pkc.load(kc, a.kc.sl, (int64_t)Kb * kNB, L);
     pvc.load(vc, a.vc.sl, (int64_t)Kb * kNB, L);
     pqu.load(qu, a.qu.sl, (int64_t)Kb * kNB, L);
@@ -246,7 +246,7 @@ __global__ __launch_bounds__(kThreads, (sizeof(T) == 2 && HD <= 64) ? 2 : 1) voi
       if (Kb < blk && blk < a.s.nblk) pub[q].load(snap + usnap_off(blk) * HD, HD, (int64_t)Kb * kNB, (int64_t)1 << 40);
     }
   };
-  auto store_chunk = [&](int Kb) {
+  auto store_chunk = [&](int Kb) __attribute__((always_inline)) {
     pkc.store(s_kc, LDK);
     pvc.store(s_vct, LDV);
     pqu.store(s_qu, LDK);
