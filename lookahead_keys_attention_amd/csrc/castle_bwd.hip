@@ -36,35 +36,6 @@ template <typename T> __device__ __forceinline__ T* head_ptr_mut(const View4& v,
   return reinterpret_cast<T*>(v.ptr) + (int64_t)b * v.sb + (int64_t)h * v.sh;
 }
 
-// Operand whose FREE index sits on lanes, read from data stored [contraction][free].
-// 16-bit types read a transposed LDS copy tc[free][contraction]; fp32 gathers from the
-// row-major tile rm[contraction][free] (free >= free_limit reads as zero).
-template <typename T>
-__device__ __forceinline__ frag<T> ld_tr_chain(const T* tc, int ldt, const T* rm, int ldr, int free_idx, int free_limit, int contr0, int g) {
-  if constexpr (sizeof(T) == 2) {
-    return ld_chain<T>(tc, ldt, free_idx, contr0, g);
-  } else {
-    frag<T> f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const int j = contr0 + 8 * (e >> 2) + 4 * g + (e & 3);
-      f[e] = free_idx < free_limit ? rm[j * ldr + free_idx] : (T)0.f;
-    }
-    return f;
-  }
-}
-template <typename T>
-__device__ __forceinline__ frag<T> ld_tr_nat(const T* tc, int ldt, const T* rm, int ldr, int free_idx, int free_limit, int contr0, int g) {
-  if constexpr (sizeof(T) == 2) {
-    return ld_nat<T>(tc, ldt, free_idx, contr0 + 8 * g);
-  } else {
-    frag<T> f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) f[e] = free_idx < free_limit ? rm[(contr0 + 8 * g + e) * ldr + free_idx] : (T)0.f;
-    return f;
-  }
-}
-
 struct Carver {
   unsigned char* p;
   template <typename U> __device__ __forceinline__ U* take(int count) {
@@ -115,17 +86,11 @@ __global__ __launch_bounds__(kThreads) void delta_kernel(BwdArgs a) {
 
 // ---------------------------------------------------------------------------
 template <typename T, int HD> constexpr int bwd_key_lds_bytes() {
-  constexpr int HDP = HD < 32 ? 32 : HD;
-  constexpr bool TC = sizeof(T) == 2;
   int b = 0;
   b += 3 * a16((int)sizeof(T) * kNB * lds_ld<T>(HD));           // qc, do, ku
   b += a16((int)sizeof(T) * kNB * lds_ld_chain<T>(HD));         // vu
   b += a16((int)sizeof(T) * kNB * lds_ld_chain<T>(kNB));        // T
-  if (TC) {
-    b += 3 * a16((int)sizeof(T) * HDP * lds_ld_chain<T>(kNB));  // qc^T, do^T, ku^T
-    b += a16((int)sizeof(T) * kNB * lds_ld_chain<T>(kNB));      // T^T
-  }
-  b += 2 * a16(4 * kNB);                                  // lse, delta
+  b += 2 * a16(4 * kNB);                                        // lse, delta
   return b;
 }
 
@@ -135,8 +100,7 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   constexpr int HDP = HD < 32 ? 32 : HD;
   constexpr int NT = HDP / 32;
   constexpr int BT = kNB / 32;   // 32-row sub-tiles per block
-  constexpr bool TC = sizeof(T) == 2;
-  constexpr int LDK = lds_ld<T>(HD), LDU = lds_ld_chain<T>(HD), LDV = lds_ld_chain<T>(kNB), LDT = lds_ld_chain<T>(kNB);
+  constexpr int LDK = lds_ld<T>(HD), LDU = lds_ld_chain<T>(HD), LDT = lds_ld_chain<T>(kNB);
 
   Carver cv{castle_smem};
   T* s_qc = cv.take<T>(kNB * LDK);
@@ -144,13 +108,6 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   T* s_ku = cv.take<T>(kNB * LDK);
   T* s_vu = cv.take<T>(kNB * LDU);
   T* s_t = cv.take<T>(kNB * LDT);
-  T* s_qct = s_qc; T* s_dot = s_do; T* s_kut = s_ku; T* s_tt = s_t;
-  if constexpr (TC) {
-    s_qct = cv.take<T>(HDP * LDV);
-    s_dot = cv.take<T>(HDP * LDV);
-    s_kut = cv.take<T>(HDP * LDV);
-    s_tt = cv.take<T>(kNB * LDT);
-  }
   float* s_lse = cv.take<float>(kNB);
   float* s_delta = cv.take<float>(kNB);
 
@@ -163,7 +120,6 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   const int kw0 = kb * 128 + 32 * wave;
   const int k = kw0 + c;
   const int Iw = kw0 / kNB;
-  const int sgroup = wave >> 1, slt = threadIdx.x & 127;   // staging group and index inside it
   const TI* qc = head_ptr<TI>(a.qc, b, h);
   const TI* kc = head_ptr<TI>(a.kc, b, h);
   const TI* vc = head_ptr<TI>(a.vc, b, h);
@@ -172,7 +128,6 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   const TI* vu = head_ptr<TI>(a.vu, b, h);
   const TI* dout = head_ptr<TI>(a.dout, b, h);
   const T* tb = reinterpret_cast<const T*>(a.ws.t_blk) + (int64_t)bh * a.s.Lp * kNB;
-  const T* ttb = reinterpret_cast<const T*>(a.ws.tt_blk) + (int64_t)bh * a.s.Lp * kNB;
   const T* usnap = reinterpret_cast<const T*>(a.ws.usnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
   T* gsnap = reinterpret_cast<T*>(a.gsnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
   const float* lse = a.ws.lse + (int64_t)bh * a.s.Lp;
@@ -189,43 +144,22 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   acc_t dvc[NT], dkc[NT], dqu[NT], G[NT];   // [n rows, k lanes]
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) { zero(dvc[nt]); zero(dkc[nt]); zero(dqu[nt]); zero(G[nt]); }
-  if (TC && HDP > HD) {
-    lds_zero(s_qct + HD * LDV, (HDP - HD) * LDV);
-    lds_zero(s_dot + HD * LDV, (HDP - HD) * LDV);
-    lds_zero(s_kut + HD * LDV, (HDP - HD) * LDV);
-  }
 
-  PatchStage<T, TI, kNB, HD, 128> pa, pb;
-  PatchStage<T, T, kNB, kNB, 128> pt;
-  auto stage_load = [&](int I) __attribute__((always_inline)) {
-    const int64_t r0 = (int64_t)I * kNB;
-    if (sgroup == 0) {
-      pa.load(slt, qc, a.qc.sl, r0, L);
-      pb.load(slt, ku, a.ku.sl, r0, L);
-      pt.load(slt, tb, kNB, r0, (int64_t)1 << 40);
-    } else {
-      pa.load(slt, dout, a.dout.sl, r0, L);
-      pb.load(slt, vu, a.vu.sl, r0, L);
-      if constexpr (TC) pt.load(slt, ttb, kNB, r0, (int64_t)1 << 40);
-    }
-  };
-  auto stage_store = [&]() __attribute__((always_inline)) {
-    if (sgroup == 0) {
-      pa.store_rows(slt, s_qc, LDK, c1);
-      if constexpr (TC) pa.store_cols(slt, s_qct, LDV, c1);
-      pb.store_rows(slt, s_ku, LDK);
-      if constexpr (TC) pb.store_cols(slt, s_kut, LDV);
-      pt.template store_rows<true>(slt, s_t, LDT);
-    } else {
-      pa.store_rows(slt, s_do, LDK);
-      if constexpr (TC) pa.store_cols(slt, s_dot, LDV);
-      pb.template store_rows<true>(slt, s_vu, LDU);
-      if constexpr (TC) pt.template store_rows<true>(slt, s_tt, LDT);
-    }
-  };
+  // every thread carries its 16-byte pieces of the five tiles of the next block
+  RowStage<T, TI, kNB, HD> pqc, pdo, pku, pvu;
+  RowStage<T, T, kNB, kNB> ptb;
+#define CASTLE_BK_LOAD(I_)                                   \
+  do {                                                       \
+    const int64_t r_ = (int64_t)(I_) * kNB;                  \
+    pqc.load(qc, a.qc.sl, r_, L);                            \
+    pdo.load(dout, a.dout.sl, r_, L);                        \
+    pku.load(ku, a.ku.sl, r_, L);                            \
+    pvu.load(vu, a.vu.sl, r_, L);                            \
+    ptb.load(tb, kNB, r_, (int64_t)1 << 40);                 \
+  } while (0)
 
   const int I0 = (kb * 128) / kNB;
-  stage_load(a.s.nblk - 1);
+  CASTLE_BK_LOAD(a.s.nblk - 1);
   for (int I = a.s.nblk - 1; I >= I0; --I) {
     const bool active = I >= Iw;
     if (active && I <= a.s.nblk - 2) {   // reverse state as of block I
@@ -244,10 +178,12 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
     }
     __syncthreads();
     const int64_t r0 = (int64_t)I * kNB;
-    // two thread groups (waves 0-1 / waves 2-3) stage three tiles each from the registers the
-    // previous iteration filled, then issue the loads of the next block
-    stage_store();
-    if (I > I0) stage_load(I - 1);
+    pqc.store_scaled(s_qc, LDK, c1);
+    pdo.store(s_do, LDK);
+    pku.store(s_ku, LDK);
+    pvu.store_halves(s_vu, LDU);
+    ptb.store_halves(s_t, LDT);
+    if (I > I0) CASTLE_BK_LOAD(I - 1);   // in flight while this block is processed
     if (threadIdx.x < kNB) {
       const int64_t i = r0 + threadIdx.x;
       s_lse[threadIdx.x] = i < L ? lse[i] * kLog2e : INFINITY;
@@ -262,8 +198,14 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
 #pragma unroll
     for (int jt = 0; jt < BT; ++jt) {
       zero(aT[jt]);
+      {
+        frag<T> oku[KS];
 #pragma unroll
-      for (int s = 0; s < KS; ++s) mma(aT[jt], ld_nat<T>(s_ku, LDK, 32 * jt + c, 16 * s + 8 * g), fqu[s]);
+        for (int s = 0; s < KS; ++s) oku[s] = ld_nat<T>(s_ku, LDK, 32 * jt + c, 16 * s + 8 * g);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < KS; ++s) mma(aT[jt], oku[s], fqu[s]);
+      }
       const int j0 = I * kNB + 32 * jt;
 #pragma unroll
       for (int r = 0; r < 16; ++r) aT[jt][r] = fast_rcp(1.f + fast_exp2(aT[jt][r]));
@@ -280,9 +222,14 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
 #pragma unroll
     for (int jt = 0; jt < BT; ++jt) {
       zero(dA[jt]);
+      {
+        frag<T> ovu[KS];
 #pragma unroll
-      for (int s = 0; s < KS; ++s)
-        mma(dA[jt], ld_chain<T>(s_vu, LDU, 32 * jt + c, 16 * s, g), chain<T>(G[s / 2], s % 2));
+        for (int s = 0; s < KS; ++s) ovu[s] = ld_chain<T>(s_vu, LDU, 32 * jt + c, 16 * s, g);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < KS; ++s) mma(dA[jt], ovu[s], chain<T>(G[s / 2], s % 2));
+      }
     }
     // (c) query sub-tiles of the block
 #pragma unroll
@@ -291,18 +238,33 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
       if (i0 + 31 < kw0) continue;   // every query precedes every key of this wave
       acc_t sc, su, dp;
       zero(sc); zero(su); zero(dp);
+      {
+        frag<T> oq[KS], od[KS], ot[BT][2];
 #pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        const frag<T> fq = ld_nat<T>(s_qc, LDK, 32 * it + c, 16 * s + 8 * g);
-        mma(sc, fq, fkc[s]);
-        if (I > Iw) mma(su, fq, fub[s]);
-        mma(dp, ld_nat<T>(s_do, LDK, 32 * it + c, 16 * s + 8 * g), fvc[s]);
-      }
+        for (int s = 0; s < KS; ++s) {
+          oq[s] = ld_nat<T>(s_qc, LDK, 32 * it + c, 16 * s + 8 * g);
+          od[s] = ld_nat<T>(s_do, LDK, 32 * it + c, 16 * s + 8 * g);
+        }
 #pragma unroll
-      for (int jt = 0; jt < BT; ++jt) {
-        if (jt > it) continue;
+        for (int jt = 0; jt < BT; ++jt)
 #pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2) mma(su, ld_chain<T>(s_t, LDT, 32 * it + c, 32 * jt + 16 * s2, g), fa[jt][s2]);
+          for (int s2 = 0; s2 < 2; ++s2)
+            if (jt <= it) ot[jt][s2] = ld_chain<T>(s_t, LDT, 32 * it + c, 32 * jt + 16 * s2, g);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+          mma(sc, oq[s], fkc[s]);
+          mma(dp, od[s], fvc[s]);
+        }
+        if (I > Iw) {
+#pragma unroll
+          for (int s = 0; s < KS; ++s) mma(su, oq[s], fub[s]);
+        }
+#pragma unroll
+        for (int jt = 0; jt < BT; ++jt)
+#pragma unroll
+          for (int s2 = 0; s2 < 2; ++s2)
+            if (jt <= it) mma(su, ot[jt][s2], fa[jt][s2]);
       }
       acc_t ds, dsu;
       const bool diag = i0 < kw0 + 31;   // tile touches the diagonal
@@ -321,22 +283,33 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
         ds[r] = dsv;
         dsu[r] = -dsv * sp;
       }
+      {
+        frag<T> odt[2][NT], oqt[2][NT], ott[2][BT];
 #pragma unroll
-      for (int s2 = 0; s2 < 2; ++s2) {
-        const frag<T> fp = chain<T>(sc, s2), fds = chain<T>(ds, s2), fdsu = chain<T>(dsu, s2);
-        const int ic = 32 * it + 16 * s2;
+        for (int s2 = 0; s2 < 2; ++s2) {
+          const int ic = 32 * it + 16 * s2;
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-          const frag<T> fdot = ld_tr_chain<T>(s_dot, LDV, s_do, LDK, 32 * nt + c, HD, ic, g);
-          const frag<T> fqct = ld_tr_chain<T>(s_qct, LDV, s_qc, LDK, 32 * nt + c, HD, ic, g);
-          mma(dvc[nt], fdot, fp);
-          mma(dkc[nt], fqct, fds);
-          mma(G[nt], fqct, fdsu);
+          for (int nt = 0; nt < NT; ++nt) {
+            odt[s2][nt] = ld_free<T, true>(s_do, LDK, 32 * nt, HD, ic, c, g);
+            oqt[s2][nt] = ld_free<T, true>(s_qc, LDK, 32 * nt, HD, ic, c, g);
+          }
+#pragma unroll
+          for (int jt = 0; jt < BT; ++jt)
+            if (jt <= it) ott[s2][jt] = ld_free<T, true>(s_t, LDT, 32 * jt, kNB, ic, c, g);
         }
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int jt = 0; jt < BT; ++jt) {
-          if (jt > it) continue;
-          mma(dA[jt], ld_tr_chain<T>(s_tt, LDT, s_t, LDT, 32 * jt + c, kNB, ic, g), fdsu);
+        for (int s2 = 0; s2 < 2; ++s2) {
+          const frag<T> fp = chain<T>(sc, s2), fds = chain<T>(ds, s2), fdsu = chain<T>(dsu, s2);
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) {
+            mma(dvc[nt], odt[s2][nt], fp);
+            mma(dkc[nt], oqt[s2][nt], fds);
+            mma(G[nt], oqt[s2][nt], fdsu);
+          }
+#pragma unroll
+          for (int jt = 0; jt < BT; ++jt)
+            if (jt <= it) mma(dA[jt], ott[s2][jt], fdsu);
         }
       }
     }
@@ -345,15 +318,23 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
     for (int jt = 0; jt < BT; ++jt) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) dA[jt][r] *= aT[jt][r] * (1.f - aT[jt][r]);
+      {
+        frag<T> okt[2][NT];
 #pragma unroll
-      for (int s2 = 0; s2 < 2; ++s2) {
-        const frag<T> fdz = chain<T>(dA[jt], s2);
+        for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-          mma(dqu[nt], ld_tr_chain<T>(s_kut, LDV, s_ku, LDK, 32 * nt + c, HD, 32 * jt + 16 * s2, g), fdz);
+          for (int nt = 0; nt < NT; ++nt) okt[s2][nt] = ld_free<T, true>(s_ku, LDK, 32 * nt, HD, 32 * jt + 16 * s2, c, g);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+          const frag<T> fdz = chain<T>(dA[jt], s2);
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) mma(dqu[nt], okt[s2][nt], fdz);
+        }
       }
     }
   }
+#undef CASTLE_BK_LOAD
   if (k < L) {
     store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dkc, b, h) + (int64_t)k * a.dkc.sl, dkc, kLn2, g);
     store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvc, b, h) + (int64_t)k * a.dvc.sl, dvc, 1.f, g);
@@ -365,18 +346,10 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
 constexpr int kCK = 32;   // keys per chunk in the query-stationary backward
 
 template <typename T, int HD> constexpr int bwd_query_lds_bytes() {
-  constexpr int HDP = HD < 32 ? 32 : HD;
-  constexpr bool TC = sizeof(T) == 2;
-  int b = 0;
-  b += 7 * a16((int)sizeof(T) * kCK * lds_ld<T>(HD));            // kc, vc, qu, ub[2], g[2]
-  if (TC) b += 6 * a16((int)sizeof(T) * HDP * lds_ld_chain<T>(kCK));   // kc^T, qu^T, ub^T[2], g^T[2]
-  b += 2 * a16((int)sizeof(T) * kCK * lds_ld<T>(128));                 // A, dSu
-  if (TC) b += a16((int)sizeof(T) * 128 * lds_ld_chain<T>(kCK));       // A^T
-  // epilogue (reuses the same memory): vu[2], qc[2], vu^T[2], qc^T[2], dT[2]
-  int e = 0;
-  e += 4 * a16((int)sizeof(T) * kNB * lds_ld<T>(HD));
-  if (TC) e += 2 * a16((int)sizeof(T) * HDP * lds_ld_chain<T>(kNB)) + 2 * a16((int)sizeof(T) * HDP * lds_ld<T>(kNB));
-  e += 2 * a16((int)sizeof(T) * kNB * lds_ld<T>(kNB));
+  int b = 7 * a16((int)sizeof(T) * kCK * lds_ld<T>(HD));           // kc, vc, qu, ub[2], g[2]
+  b += 2 * a16((int)sizeof(T) * 128 * lds_ld_chain<T>(kCK));       // A^T [j][k], dSu^T [i][k]
+  // epilogue (reuses the same memory): vu[2], qc[2], dT [i][j] for both blocks
+  int e = 4 * a16((int)sizeof(T) * kNB * lds_ld<T>(HD)) + 2 * a16((int)sizeof(T) * kNB * lds_ld_chain<T>(kNB));
   return b > e ? b : e;
 }
 
@@ -387,31 +360,21 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
   constexpr int NT = HDP / 32;
   constexpr int BT = kNB / 32;
   constexpr int TS = kNB / 16;   // 16-deep steps across a block
+  constexpr int CKT = kCK / 32;  // 32-key sub-tiles per chunk
   constexpr int QB = 128;
   constexpr int NQ = QB / kNB;
-  constexpr bool TC = sizeof(T) == 2;
-  constexpr int LDK = lds_ld<T>(HD), LDC = lds_ld_chain<T>(kCK), LDA = lds_ld<T>(QB);
-  constexpr int LDV = lds_ld_chain<T>(kNB), LDQ = lds_ld<T>(kNB), LDT = lds_ld<T>(kNB);
+  constexpr int LDK = lds_ld<T>(HD), LDC = lds_ld_chain<T>(kCK), LDT = lds_ld_chain<T>(kNB);
 
   Carver cv{castle_smem};
   T* s_kc = cv.take<T>(kCK * LDK);
   T* s_vc = cv.take<T>(kCK * LDK);
   T* s_qu = cv.take<T>(kCK * LDK);
-  T* s_ub[NQ]; T* s_g[NQ];
-  for (int q = 0; q < NQ; ++q) s_ub[q] = cv.take<T>(kCK * LDK);
-  for (int q = 0; q < NQ; ++q) s_g[q] = cv.take<T>(kCK * LDK);
-  T* s_kct = s_kc; T* s_qut = s_qu; T* s_ubt[NQ]; T* s_gt[NQ];
-  for (int q = 0; q < NQ; ++q) { s_ubt[q] = s_ub[q]; s_gt[q] = s_g[q]; }
-  if constexpr (TC) {
-    s_kct = cv.take<T>(HDP * LDC);
-    s_qut = cv.take<T>(HDP * LDC);
-    for (int q = 0; q < NQ; ++q) s_ubt[q] = cv.take<T>(HDP * LDC);
-    for (int q = 0; q < NQ; ++q) s_gt[q] = cv.take<T>(HDP * LDC);
-  }
-  T* s_a = cv.take<T>(kCK * LDA);
-  T* s_dsu = cv.take<T>(kCK * LDA);
-  T* s_at = s_a;
-  if constexpr (TC) s_at = cv.take<T>(QB * LDC);
+  T* s_ub0 = cv.take<T>(kCK * LDK);
+  T* s_ub1 = cv.take<T>(kCK * LDK);
+  T* s_g0 = cv.take<T>(kCK * LDK);
+  T* s_g1 = cv.take<T>(kCK * LDK);
+  T* s_at = cv.take<T>(QB * LDC);     // gate, [source j][key k]
+  T* s_dsut = cv.take<T>(QB * LDC);   // dSu,  [query i][key k]
 
   int rank, bh;
   work_item(a.s.B * a.s.H, rank, bh);
@@ -425,12 +388,14 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
   const int Ifirst = (qb * QB) / kNB;
   const int Iw = i0w / kNB;
   const int qw = Iw - Ifirst;                 // which of the workgroup's blocks
-  const int jw = 32 * wave;                   // columns of this wave inside the 128-wide tiles
-  const int cb = (jw / kNB) * kNB;            // first column of its block
+  const int jw = 32 * wave;                   // rows of this wave inside the 128-row exchange tiles
+  const int cb = (jw / kNB) * kNB;            // first row of its block there
   const int lw = jw % kNB;                    // offset of the wave inside its block
   const int nintra = (lw + 32) / 16;          // steps covering sources j <= i
   const int ifirst = lw / 16;                 // first step covering queries i >= j
   const bool has_g = Iw <= a.s.nblk - 2;
+  const T* s_ubw = qw == 0 ? s_ub0 : s_ub1;
+  const T* s_gw = qw == 0 ? s_g0 : s_g1;
 
   const TI* qc = head_ptr<TI>(a.qc, b, h);
   const TI* kc = head_ptr<TI>(a.kc, b, h);
@@ -466,29 +431,21 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
   for (int nt = 0; nt < NT; ++nt) { zero(dqc[nt]); zero(dku[nt]); zero(dvu[nt]); }
 #pragma unroll
   for (int jt = 0; jt < BT; ++jt) zero(dtacc[jt]);
-  if (TC && HDP > HD) {
-    lds_zero(s_kct + HD * LDC, (HDP - HD) * LDC);
-    lds_zero(s_qut + HD * LDC, (HDP - HD) * LDC);
-    for (int q = 0; q < NQ; ++q) {
-      lds_zero(s_ubt[q] + HD * LDC, (HDP - HD) * LDC);
-      lds_zero(s_gt[q] + HD * LDC, (HDP - HD) * LDC);
-    }
-  }
 
-  PatchStage<T, TI, kCK, HD, 64> pi;
-  PatchStage<T, T, kCK, HD, 64> pw;
-  const int sq = wave & 1;                          // which of the two row blocks the workspace tile serves
-  const int sblk = Ifirst + sq;
-  const TI* isrc = wave == 0 ? kc : (wave == 1 ? qu : vc);
-  const int64_t istride = wave == 0 ? a.kc.sl : (wave == 1 ? a.qu.sl : a.vc.sl);
-// issue the global loads of the chunk that starts at key K0 (each wave its own tiles)
-#define CASTLE_BQ_WANT_U(K0) (wave < 2 && sblk < a.s.nblk && (K0) / kNB < sblk)
-#define CASTLE_BQ_WANT_G(K0) (wave >= 2 && sblk <= a.s.nblk - 2 && (K0) / kNB <= sblk)
-#define CASTLE_BQ_LOAD(K0)                                                                          \
-  do {                                                                                              \
-    if (wave < 3) pi.load(lane, isrc, istride, (K0), L);                                            \
-    if (CASTLE_BQ_WANT_U(K0)) pw.load(lane, usnap + usnap_off(sblk) * HD, HD, (K0), (int64_t)1 << 40); \
-    if (CASTLE_BQ_WANT_G(K0)) pw.load(lane, gsnap + gsnap_off(sblk) * HD, HD, (K0), (int64_t)1 << 40); \
+  // staging: every thread carries one 16-byte piece of each of the 7 tiles of the next chunk
+  RowStage<T, TI, kCK, HD> pkc, pvc, pqu;
+  RowStage<T, T, kCK, HD> pu0, pu1, pg0, pg1;
+  const int blk0 = Ifirst, blk1 = Ifirst + 1;
+#define CASTLE_BQ_LOAD(K0)                                                                                      \
+  do {                                                                                                          \
+    const int kb_ = (K0) / kNB;                                                                                 \
+    pkc.load(kc, a.kc.sl, (K0), L);                                                                             \
+    pvc.load(vc, a.vc.sl, (K0), L);                                                                             \
+    pqu.load(qu, a.qu.sl, (K0), L);                                                                             \
+    if (kb_ < blk0) pu0.load(usnap + usnap_off(blk0) * HD, HD, (K0), (int64_t)1 << 40);                          \
+    if (kb_ < blk1 && blk1 < a.s.nblk) pu1.load(usnap + usnap_off(blk1) * HD, HD, (K0), (int64_t)1 << 40);        \
+    if (kb_ <= blk0 && blk0 <= a.s.nblk - 2) pg0.load(gsnap + gsnap_off(blk0) * HD, HD, (K0), (int64_t)1 << 40);  \
+    if (kb_ <= blk1 && blk1 <= a.s.nblk - 2) pg1.load(gsnap + gsnap_off(blk1) * HD, HD, (K0), (int64_t)1 << 40);  \
   } while (0)
 
   int kend = qb * QB + QB;
@@ -497,156 +454,195 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
   for (int k0 = 0; k0 < kend; k0 += kCK) {
     const int Kb = k0 / kNB;
     __syncthreads();
-    // one wave per tile (wave 0: kc + ub[0], wave 1: qu + ub[1], wave 2: vc + g[0], wave 3: g[1]),
-    // written from the registers the previous iteration filled; then the next chunk's loads go out
-    if (wave < 3) {
-      pi.store_rows(lane, wave == 0 ? s_kc : (wave == 1 ? s_qu : s_vc), LDK);
-      if constexpr (TC) {
-        if (wave < 2) pi.store_cols(lane, wave == 0 ? s_kct : s_qut, LDC);
-      }
-    }
-    if (CASTLE_BQ_WANT_U(k0)) {
-      pw.store_rows(lane, sq == 0 ? s_ub[0] : s_ub[1], LDK);
-      if constexpr (TC) pw.store_cols(lane, sq == 0 ? s_ubt[0] : s_ubt[1], LDC);
-    }
-    if (CASTLE_BQ_WANT_G(k0)) {
-      pw.store_rows(lane, sq == 0 ? s_g[0] : s_g[1], LDK);
-      if constexpr (TC) pw.store_cols(lane, sq == 0 ? s_gt[0] : s_gt[1], LDC);
-    }
-    if (k0 + kCK < kend) CASTLE_BQ_LOAD(k0 + kCK);
+    pkc.store(s_kc, LDK);
+    pvc.store(s_vc, LDK);
+    pqu.store(s_qu, LDK);
+    if (Kb < blk0) pu0.store(s_ub0, LDK);
+    if (Kb < blk1 && blk1 < a.s.nblk) pu1.store(s_ub1, LDK);
+    if (Kb <= blk0 && blk0 <= a.s.nblk - 2) pg0.store(s_g0, LDK);
+    if (Kb <= blk1 && blk1 <= a.s.nblk - 2) pg1.store(s_g1, LDK);
+    if (k0 + kCK < kend) CASTLE_BQ_LOAD(k0 + kCK);   // in flight while this chunk is processed
     __syncthreads();
     const bool active = Kb <= Iw;
 
-    // phase 0: gate tile A[k rows, j lanes] for this wave's 32 source rows
-    acc_t aK;
-    zero(aK);
-    if (active) {
+    // phase 0: gate tiles A[k rows, j lanes] for this wave's 32 source rows, shared as A^T[j][k]
+    acc_t aK[CKT];
 #pragma unroll
-      for (int s = 0; s < KS; ++s) mma(aK, ld_nat<T>(s_qu, LDK, c, 16 * s + 8 * g), fku[s]);
+    for (int kt = 0; kt < CKT; ++kt) {
+      zero(aK[kt]);
+      if (!active) continue;
+      {
+        frag<T> oqu[KS];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) aK[r] = fast_rcp(1.f + fast_exp2(aK[r]));
-      if (k0 + 31 >= i0w) {   // chunk reaches the diagonal: keep j > k only
+        for (int s = 0; s < KS; ++s) oqu[s] = ld_nat<T>(s_qu, LDK, 32 * kt + c, 16 * s + 8 * g);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < KS; ++s) mma(aK[kt], oqu[s], fku[s]);
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) aK[kt][r] = fast_rcp(1.f + fast_exp2(aK[kt][r]));
+      if (k0 + 32 * kt + 31 >= i0w) {   // sub-tile reaches the diagonal: keep j > k only
 #pragma unroll
         for (int r = 0; r < 16; ++r)
-          if (i <= k0 + acc_row(r, g)) aK[r] = 0.f;
+          if (i <= k0 + 32 * kt + acc_row(r, g)) aK[kt][r] = 0.f;
       }
 #pragma unroll
-      for (int r = 0; r < 16; ++r) s_a[acc_row(r, g) * LDA + jw + c] = (T)aK[r];
-      if constexpr (TC) {
-#pragma unroll
-        for (int q = 0; q < 4; ++q) st4<T>(s_at + (jw + c) * LDC + 8 * q + 4 * g, pack4<T>(aK, q));
-      }
+      for (int q = 0; q < 4; ++q) st4<T>(s_at + (jw + c) * LDC + 32 * kt + 8 * q + 4 * g, pack4<T>(aK[kt], q));
     }
     __syncthreads();
 
     // phase 1: this lane's row is a query
-    if (active && k0 <= i0w + 31) {
+#pragma unroll
+    for (int kt = 0; kt < CKT; ++kt) {
+      const int ks = k0 + 32 * kt;
+      if (!(active && ks <= i0w + 31)) continue;
       acc_t sc, su, dp;
       zero(sc); zero(su); zero(dp);
+      {
+        // all operand fragments of this group are requested before the first MFMA
+        frag<T> okc[KS], oub[KS], ovc[KS], oat[TS];
 #pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        mma(sc, ld_nat<T>(s_kc, LDK, c, 16 * s + 8 * g), fqc[s]);
-        if (Kb < Iw) mma(su, ld_nat<T>(s_ub[qw], LDK, c, 16 * s + 8 * g), fqc[s]);
-        mma(dp, ld_nat<T>(s_vc, LDK, c, 16 * s + 8 * g), fdo[s]);
+        for (int s = 0; s < KS; ++s) {
+          okc[s] = ld_nat<T>(s_kc, LDK, 32 * kt + c, 16 * s + 8 * g);
+          ovc[s] = ld_nat<T>(s_vc, LDK, 32 * kt + c, 16 * s + 8 * g);
+          oub[s] = ld_nat<T>(s_ubw, LDK, 32 * kt + c, 16 * s + 8 * g);
+        }
+#pragma unroll
+        for (int s = 0; s < TS; ++s) oat[s] = ld_free<T, false>(s_at + cb * LDC, LDC, 32 * kt, kCK, 16 * s, c, g);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+          mma(sc, okc[s], fqc[s]);
+          mma(dp, ovc[s], fdo[s]);
+        }
+        if (Kb < Iw) {
+#pragma unroll
+          for (int s = 0; s < KS; ++s) mma(su, oub[s], fqc[s]);
+        }
+#pragma unroll
+        for (int s = 0; s < TS; ++s)
+          if (s < nintra) mma(su, oat[s], ft[s]);
       }
-#pragma unroll
-      for (int s = 0; s < TS; ++s)
-        if (s < nintra) mma(su, ld_nat<T>(s_a, LDA, c, cb + 16 * s + 8 * g), ft[s]);
       acc_t ds, dsu;
-      const bool diag = k0 + 31 > i0w;   // chunk reaches the diagonal
+      const bool diag = ks + 31 > i0w;   // sub-tile reaches the diagonal
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const float sg = fast_rcp(1.f + fast_exp2(-su[r]));
         const float x = __builtin_fmaf(-su[r], sg, sc[r]);
         float p = fast_exp2(x - lse2);
-        if (diag && k0 + acc_row(r, g) > i) p = 0.f;
+        if (diag && ks + acc_row(r, g) > i) p = 0.f;
         const float dsv = p * (dp[r] - dlt);
         const float y = su[r] * kLn2;                     // true Su
         const float t = __builtin_fmaf(-y, sg, y);
         const float sp = __builtin_fmaf(sg, t, sg);
         ds[r] = dsv;
         dsu[r] = -dsv * sp;
-        s_dsu[acc_row(r, g) * LDA + jw + c] = (T)dsu[r];
       }
 #pragma unroll
-      for (int s2 = 0; s2 < 2; ++s2) {
-        const frag<T> fds = chain<T>(ds, s2), fdsu = chain<T>(dsu, s2);
+      for (int q = 0; q < 4; ++q) st4<T>(s_dsut + (jw + c) * LDC + 32 * kt + 8 * q + 4 * g, pack4<T>(dsu, q));
+      {
+        frag<T> okt[2][NT], out[2][NT], oat[2][BT];
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-          mma(dqc[nt], ld_tr_chain<T>(s_kct, LDC, s_kc, LDK, 32 * nt + c, HD, 16 * s2, g), fds);
-          if (Kb < Iw) mma(dqc[nt], ld_tr_chain<T>(s_ubt[qw], LDC, s_ub[qw], LDK, 32 * nt + c, HD, 16 * s2, g), fdsu);
+        for (int s2 = 0; s2 < 2; ++s2) {
+          const int kc0 = 32 * kt + 16 * s2;
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) {
+            okt[s2][nt] = ld_free<T, true>(s_kc, LDK, 32 * nt, HD, kc0, c, g);
+            out[s2][nt] = ld_free<T, true>(s_ubw, LDK, 32 * nt, HD, kc0, c, g);
+          }
+#pragma unroll
+          for (int jt = 0; jt < BT; ++jt) oat[s2][jt] = ld_chain<T>(s_at, LDC, cb + 32 * jt + c, kc0, g);
         }
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int jt = 0; jt < BT; ++jt)
-          if (32 * jt < lw + 32)
-            mma(dtacc[jt], ld_tr_chain<T>(s_at, LDC, s_a, LDA, cb + 32 * jt + c, QB, 16 * s2, g), fdsu);
+        for (int s2 = 0; s2 < 2; ++s2) {
+          const frag<T> fds = chain<T>(ds, s2), fdsu = chain<T>(dsu, s2);
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) {
+            mma(dqc[nt], okt[s2][nt], fds);
+            if (Kb < Iw) mma(dqc[nt], out[s2][nt], fdsu);
+          }
+#pragma unroll
+          for (int jt = 0; jt < BT; ++jt)
+            if (32 * jt < lw + 32) mma(dtacc[jt], oat[s2][jt], fdsu);
+        }
       }
     }
     __syncthreads();
 
     // phase 2: this lane's row is a lookahead source j; needs some key k < j
-    if (active && k0 < i0w + 31) {
+#pragma unroll
+    for (int kt = 0; kt < CKT; ++kt) {
+      const int ks = k0 + 32 * kt;
+      if (!(active && ks < i0w + 31)) continue;
       acc_t dA;
       zero(dA);
+      frag<T> oqt[2][NT], ogt[2][NT];
+      {
+        frag<T> ods[TS], og[KS];
 #pragma unroll
-      for (int s = 0; s < TS; ++s)
-        if (s >= ifirst) mma(dA, ld_nat<T>(s_dsu, LDA, c, cb + 16 * s + 8 * g), ftt[s]);
-      if (has_g) {
+        for (int s = 0; s < TS; ++s) ods[s] = ld_free<T, false>(s_dsut + cb * LDC, LDC, 32 * kt, kCK, 16 * s, c, g);
 #pragma unroll
-        for (int s = 0; s < KS; ++s) mma(dA, ld_nat<T>(s_g[qw], LDK, c, 16 * s + 8 * g), fvu[s]);
+        for (int s = 0; s < KS; ++s) og[s] = ld_nat<T>(s_gw, LDK, 32 * kt + c, 16 * s + 8 * g);
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) {
+            oqt[s2][nt] = ld_free<T, true>(s_qu, LDK, 32 * nt, HD, 32 * kt + 16 * s2, c, g);
+            ogt[s2][nt] = ld_free<T, true>(s_gw, LDK, 32 * nt, HD, 32 * kt + 16 * s2, c, g);
+          }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < TS; ++s)
+          if (s >= ifirst) mma(dA, ods[s], ftt[s]);
+        if (has_g) {
+#pragma unroll
+          for (int s = 0; s < KS; ++s) mma(dA, og[s], fvu[s]);
+        }
       }
       acc_t dz;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) dz[r] = dA[r] * aK[r] * (1.f - aK[r]);
+      for (int r = 0; r < 16; ++r) dz[r] = dA[r] * aK[kt][r] * (1.f - aK[kt][r]);
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
-        const frag<T> fdz = chain<T>(dz, s2), fa = chain<T>(aK, s2);
+        const frag<T> fdz = chain<T>(dz, s2), fa = chain<T>(aK[kt], s2);
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
-          mma(dku[nt], ld_tr_chain<T>(s_qut, LDC, s_qu, LDK, 32 * nt + c, HD, 16 * s2, g), fdz);
-          if (has_g) mma(dvu[nt], ld_tr_chain<T>(s_gt[qw], LDC, s_g[qw], LDK, 32 * nt + c, HD, 16 * s2, g), fa);
+          mma(dku[nt], oqt[s2][nt], fdz);
+          if (has_g) mma(dvu[nt], ogt[s2][nt], fa);
         }
       }
     }
   }
+#undef CASTLE_BQ_LOAD
 
-  // ---- epilogue: in-block terms dT = tril(dTacc):  dqc += dT Vu,  dvu += dT^T Qc -------------
+  // ---- epilogue: in-block terms dT = tril(dTacc):  dqc += dT Vu,  dvu += dT^T Qc' ------------
   __syncthreads();
   Carver ce{castle_smem};
-  T* e_vu[NQ]; T* e_qc[NQ]; T* e_vut[NQ]; T* e_qct[NQ]; T* e_dt[NQ];
-  for (int q = 0; q < NQ; ++q) e_vu[q] = ce.take<T>(kNB * LDK);
-  for (int q = 0; q < NQ; ++q) e_qc[q] = ce.take<T>(kNB * LDK);
-  for (int q = 0; q < NQ; ++q) { e_vut[q] = e_vu[q]; e_qct[q] = e_qc[q]; }
-  if constexpr (TC) {
-    for (int q = 0; q < NQ; ++q) e_vut[q] = ce.take<T>(HDP * LDV);
-    for (int q = 0; q < NQ; ++q) e_qct[q] = ce.take<T>(HDP * LDQ);
-  }
-  for (int q = 0; q < NQ; ++q) e_dt[q] = ce.take<T>(kNB * LDT);
-#pragma unroll
-  for (int q = 0; q < NQ; ++q) {
-    const int64_t r0 = (int64_t)(Ifirst + q) * kNB;
+  T* e_vu0 = ce.take<T>(kNB * LDK);
+  T* e_vu1 = ce.take<T>(kNB * LDK);
+  T* e_qc0 = ce.take<T>(kNB * LDK);
+  T* e_qc1 = ce.take<T>(kNB * LDK);
+  T* e_dt0 = ce.take<T>(kNB * LDT);   // dT, [query i][source j] (block local)
+  T* e_dt1 = ce.take<T>(kNB * LDT);
+  {
     RowStage<T, TI, kNB, HD> st;
-    st.load(vu, a.vu.sl, r0, L); st.store(e_vu[q], LDK);
-    st.load(qc, a.qc.sl, r0, L); st.store_scaled(e_qc[q], LDK, c1);
-    if constexpr (TC) {
-      if (HDP > HD) {
-        lds_zero(e_vut[q] + HD * LDV, (HDP - HD) * LDV);
-        lds_zero(e_qct[q] + HD * LDQ, (HDP - HD) * LDQ);
-      }
-      ColStage<T, TI, kNB, HD> ct;
-      ct.load(vu, a.vu.sl, r0, L); ct.store(e_vut[q], LDV);
-      ct.load(qc, a.qc.sl, r0, L); ct.store(e_qct[q], LDQ, c1);
-    }
+    st.load(vu, a.vu.sl, (int64_t)blk0 * kNB, L); st.store(e_vu0, LDK);
+    st.load(vu, a.vu.sl, (int64_t)blk1 * kNB, L); st.store(e_vu1, LDK);
+    st.load(qc, a.qc.sl, (int64_t)blk0 * kNB, L); st.store_scaled(e_qc0, LDK, c1);
+    st.load(qc, a.qc.sl, (int64_t)blk1 * kNB, L); st.store_scaled(e_qc1, LDK, c1);
   }
-  // dT^T[j rows, i lanes] masked to j <= i, shared as e_dt[j][i] for the source-side product
+  const T* e_vuw = qw == 0 ? e_vu0 : e_vu1;
+  const T* e_qcw = qw == 0 ? e_qc0 : e_qc1;
+  T* e_dtw = qw == 0 ? e_dt0 : e_dt1;
+  // dT^T[j rows, i lanes] masked to j <= i, shared as dT[i][j] for the source-side product
 #pragma unroll
   for (int jt = 0; jt < BT; ++jt) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int jl = 32 * jt + acc_row(r, g);
-      if (jl > lw + c) dtacc[jt][r] = 0.f;
-      e_dt[qw][jl * LDT + lw + c] = (T)dtacc[jt][r];
-    }
+    for (int r = 0; r < 16; ++r)
+      if (32 * jt + acc_row(r, g) > lw + c) dtacc[jt][r] = 0.f;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) st4<T>(e_dtw + (lw + c) * LDT + 32 * jt + 8 * q + 4 * g, pack4<T>(dtacc[jt], q));
   }
   __syncthreads();
 #pragma unroll
@@ -657,16 +653,17 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
       const frag<T> fdt = chain<T>(dtacc[jt], s2);
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt)
-        mma(dqc[nt], ld_tr_chain<T>(e_vut[qw], LDV, e_vu[qw], LDK, 32 * nt + c, HD, 32 * jt + 16 * s2, g), fdt);
+        mma(dqc[nt], ld_free<T, true>(e_vuw, LDK, 32 * nt, HD, 32 * jt + 16 * s2, c, g), fdt);
     }
   }
 #pragma unroll
   for (int s = 0; s < TS; ++s) {
     if (s < ifirst) continue;
-    const frag<T> fdt = ld_nat<T>(e_dt[qw], LDT, lw + c, 16 * s + 8 * g);   // (source j, queries i)
+    // B operand: source j = lw + c on lanes, queries i = 16 s .. natural order, from dT[i][j]
+    const frag<T> fdt = ld_free<T, false>(e_dtw, LDT, lw, kNB, 16 * s, c, g);
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
-      mma(dvu[nt], ld_tr_nat<T>(e_qct[qw], LDQ, e_qc[qw], LDK, 32 * nt + c, HD, 16 * s, g), fdt);
+      mma(dvu[nt], ld_free<T, false>(e_qcw, LDK, 32 * nt, HD, 16 * s, c, g), fdt);
   }
   if (i < L) {
     store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqc, b, h) + (int64_t)i * a.dqc.sl, dqc, c0, g);

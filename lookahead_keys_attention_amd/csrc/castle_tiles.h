@@ -111,6 +111,43 @@ template <typename T, typename TI, int N> __device__ __forceinline__ vec<T, N> c
   }
 }
 
+// ---- transposed operand fragments straight from a row-major LDS tile ---------------------
+// ds_read_b64_tr_b16: inside each group of 16 lanes, lane i slot e receives element (i % 4) of
+// the 4-element row whose address lane (4e + i/4) supplied.  If lanes 4e..4e+3 of a group point
+// at columns n .. n+15 of contraction row rho(e), lane i ends up with rows rho(0..3) of its own
+// column n + i.  Two such reads build an operand fragment whose FREE index (n0 + c) sits on
+// lanes from data stored [contraction][free], in natural or chained contraction order.
+typedef short v4i16_t __attribute__((ext_vector_type(4)));
+template <typename T> __device__ __forceinline__ vec<T, 4> lds_tr4(const T* p) {
+  static_assert(sizeof(T) == 2, "transpose reads exist for 16-bit elements");
+  typedef v4i16_t __attribute__((address_space(3))) * lds_ptr;
+  return __builtin_bit_cast(vec<T, 4>, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)p));
+}
+// rm: row-major tile [contraction][free], ld multiple of 4.  Returns the fragment for free
+// index n0 + c (n0 multiple of 32) and the 16 contraction rows starting at contr0.
+// 16-bit types use transpose reads; fp32 gathers.  Lanes whose free index is >= free_limit
+// (only possible when the tile has fewer than 32 payload columns) get zeros.
+template <typename T, bool CHAINED>
+__device__ __forceinline__ frag<T> ld_free(const T* rm, int ld, int n0, int free_limit, int contr0, int c, int g) {
+  frag<T> f;
+  if constexpr (sizeof(T) == 2) {
+    const int lp = c & 15;
+    const T* p = rm + (contr0 + (CHAINED ? 4 : 8) * g + (lp >> 2)) * ld + n0 + 16 * (c >> 4) + 4 * (lp & 3);
+    const vec<T, 4> lo = lds_tr4<T>(p);
+    const vec<T, 4> hi = lds_tr4<T>(p + (CHAINED ? 8 : 4) * ld);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { f[e] = lo[e]; f[4 + e] = hi[e]; }
+    if (free_limit < n0 + 32 && n0 + c >= free_limit) f = zero_frag<T>();
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int j = contr0 + (CHAINED ? 8 * (e >> 2) + 4 * g + (e & 3) : 8 * g + e);
+      f[e] = n0 + c < free_limit ? rm[j * ld + n0 + c] : (T)0.f;
+    }
+  }
+  return f;
+}
+
 // natural fragment straight from global memory (row-major, unit inner stride); zeros when !ok
 template <typename T, typename TI = T>
 __device__ __forceinline__ frag<T> ldg_nat(const TI* base, int64_t row_stride, int64_t row, int col, bool ok) {
