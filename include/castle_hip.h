@@ -79,7 +79,8 @@ int64_t castle_bwd_workspace_bytes(int B, int H, int L, int d, int dtype);
 /* Parallel backward.  Same operands as castle_fwd plus the forward output `out`, the
  * upstream gradient `dout` and the forward workspace as castle_fwd left it.  Writes the six
  * gradients (all (B,H,L,d) views; every element is written, nothing is accumulated).
- * U carries no gradient (lookahead_keys_attention_triton.py:513-515).  d in {16,32,64}. */
+ * U carries no gradient (lookahead_keys_attention_triton.py:513-515).  d in {16,32,64}, and 128 for
+ * the 16-bit element types (there every kernel runs twice, each pass keeping half of the outputs). */
 int castle_bwd(const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
                const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
                const castle_view4* out, const castle_view4* dout,

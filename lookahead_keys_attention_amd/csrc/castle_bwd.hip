@@ -94,8 +94,12 @@ template <typename T, int HD> constexpr int bwd_key_lds_bytes() {
   return b;
 }
 
-template <typename T, typename TI, int HD>
+// PART selects the outputs of a launch: 0 = all (d <= 64); 1 = dVc, dKc; 2 = dQu and the reverse
+// state (gsnap).  At d = 128 the four accumulator sets do not fit the register file together, so
+// the kernel runs once with PART 1 and once with PART 2 (the score tiles are recomputed).
+template <typename T, typename TI, int HD, int PART>
 __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
+  constexpr bool DO_KV = PART != 2, DO_QG = PART != 1;
   constexpr int KS = HD / 16;
   constexpr int HDP = HD < 32 ? 32 : HD;
   constexpr int NT = HDP / 32;
@@ -159,10 +163,11 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   } while (0)
 
   const int I0 = (kb * 128) / kNB;
-  CASTLE_BK_LOAD(a.s.nblk - 1);
+  constexpr bool PF = HD <= 64;   // d = 128 has no registers to spare for a block in flight
+  if (PF) CASTLE_BK_LOAD(a.s.nblk - 1);
   for (int I = a.s.nblk - 1; I >= I0; --I) {
     const bool active = I >= Iw;
-    if (active && I <= a.s.nblk - 2) {   // reverse state as of block I
+    if (DO_QG && active && I <= a.s.nblk - 2) {   // reverse state as of block I
       T* dst = gsnap + (gsnap_off(I) + k) * HD;
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt)
@@ -178,12 +183,13 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
     }
     __syncthreads();
     const int64_t r0 = (int64_t)I * kNB;
+    if (!PF) CASTLE_BK_LOAD(I);
     pqc.store_scaled(s_qc, LDK, c1);
     pdo.store(s_do, LDK);
     pku.store(s_ku, LDK);
     pvu.store_halves(s_vu, LDU);
     ptb.store_halves(s_t, LDT);
-    if (I > I0) CASTLE_BK_LOAD(I - 1);   // in flight while this block is processed
+    if (PF && I > I0) CASTLE_BK_LOAD(I - 1);   // in flight while this block is processed
     if (threadIdx.x < kNB) {
       const int64_t i = r0 + threadIdx.x;
       s_lse[threadIdx.x] = i < L ? lse[i] * kLog2e : INFINITY;
@@ -222,7 +228,7 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
 #pragma unroll
     for (int jt = 0; jt < BT; ++jt) {
       zero(dA[jt]);
-      {
+      if constexpr (DO_QG) {
         frag<T> ovu[KS];
 #pragma unroll
         for (int s = 0; s < KS; ++s) ovu[s] = ld_chain<T>(s_vu, LDU, 32 * jt + c, 16 * s, g);
@@ -290,12 +296,14 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
           const int ic = 32 * it + 16 * s2;
 #pragma unroll
           for (int nt = 0; nt < NT; ++nt) {
-            odt[s2][nt] = ld_free<T, true>(s_do, LDK, 32 * nt, HD, ic, c, g);
+            if constexpr (DO_KV) odt[s2][nt] = ld_free<T, true>(s_do, LDK, 32 * nt, HD, ic, c, g);
             oqt[s2][nt] = ld_free<T, true>(s_qc, LDK, 32 * nt, HD, ic, c, g);
           }
+          if constexpr (DO_QG) {
 #pragma unroll
-          for (int jt = 0; jt < BT; ++jt)
-            if (jt <= it) ott[s2][jt] = ld_free<T, true>(s_t, LDT, 32 * jt, kNB, ic, c, g);
+            for (int jt = 0; jt < BT; ++jt)
+              if (jt <= it) ott[s2][jt] = ld_free<T, true>(s_t, LDT, 32 * jt, kNB, ic, c, g);
+          }
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -303,19 +311,23 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
           const frag<T> fp = chain<T>(sc, s2), fds = chain<T>(ds, s2), fdsu = chain<T>(dsu, s2);
 #pragma unroll
           for (int nt = 0; nt < NT; ++nt) {
-            mma(dvc[nt], odt[s2][nt], fp);
-            mma(dkc[nt], oqt[s2][nt], fds);
-            mma(G[nt], oqt[s2][nt], fdsu);
+            if constexpr (DO_KV) {
+              mma(dvc[nt], odt[s2][nt], fp);
+              mma(dkc[nt], oqt[s2][nt], fds);
+            }
+            if constexpr (DO_QG) mma(G[nt], oqt[s2][nt], fdsu);
           }
+          if constexpr (DO_QG) {
 #pragma unroll
-          for (int jt = 0; jt < BT; ++jt)
-            if (jt <= it) mma(dA[jt], ott[s2][jt], fdsu);
+            for (int jt = 0; jt < BT; ++jt)
+              if (jt <= it) mma(dA[jt], ott[s2][jt], fdsu);
+          }
         }
       }
     }
     // (d) dZ^T = dA^T * A (1 - A)  ->  dQu
 #pragma unroll
-    for (int jt = 0; jt < BT; ++jt) {
+    for (int jt = 0; jt < (DO_QG ? BT : 0); ++jt) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) dA[jt][r] *= aT[jt][r] * (1.f - aT[jt][r]);
       {
@@ -336,9 +348,11 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   }
 #undef CASTLE_BK_LOAD
   if (k < L) {
-    store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dkc, b, h) + (int64_t)k * a.dkc.sl, dkc, kLn2, g);
-    store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvc, b, h) + (int64_t)k * a.dvc.sl, dvc, 1.f, g);
-    store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqu, b, h) + (int64_t)k * a.dqu.sl, dqu, c0 * kLn2, g);
+    if constexpr (DO_KV) {
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dkc, b, h) + (int64_t)k * a.dkc.sl, dkc, kLn2, g);
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvc, b, h) + (int64_t)k * a.dvc.sl, dvc, 1.f, g);
+    }
+    if constexpr (DO_QG) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqu, b, h) + (int64_t)k * a.dqu.sl, dqu, c0 * kLn2, g);
   }
 }
 
@@ -353,8 +367,10 @@ template <typename T, int HD> constexpr int bwd_query_lds_bytes() {
   return b > e ? b : e;
 }
 
-template <typename T, typename TI, int HD>
+// PART: 0 = all outputs (d <= 64); 1 = dQc; 2 = dKu, dVu (see bwd_key_kernel).
+template <typename T, typename TI, int HD, int PART>
 __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
+  constexpr bool DO_Q = PART != 2, DO_S = PART != 1;
   constexpr int KS = HD / 16;
   constexpr int HDP = HD < 32 ? 32 : HD;
   constexpr int NT = HDP / 32;
@@ -444,24 +460,26 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
     pqu.load(qu, a.qu.sl, (K0), L);                                                                             \
     if (kb_ < blk0) pu0.load(usnap + usnap_off(blk0) * HD, HD, (K0), (int64_t)1 << 40);                          \
     if (kb_ < blk1 && blk1 < a.s.nblk) pu1.load(usnap + usnap_off(blk1) * HD, HD, (K0), (int64_t)1 << 40);        \
-    if (kb_ <= blk0 && blk0 <= a.s.nblk - 2) pg0.load(gsnap + gsnap_off(blk0) * HD, HD, (K0), (int64_t)1 << 40);  \
-    if (kb_ <= blk1 && blk1 <= a.s.nblk - 2) pg1.load(gsnap + gsnap_off(blk1) * HD, HD, (K0), (int64_t)1 << 40);  \
+    if (DO_S && kb_ <= blk0 && blk0 <= a.s.nblk - 2) pg0.load(gsnap + gsnap_off(blk0) * HD, HD, (K0), (int64_t)1 << 40);  \
+    if (DO_S && kb_ <= blk1 && blk1 <= a.s.nblk - 2) pg1.load(gsnap + gsnap_off(blk1) * HD, HD, (K0), (int64_t)1 << 40);  \
   } while (0)
 
   int kend = qb * QB + QB;
   if (kend > a.s.Lp) kend = a.s.Lp;
-  CASTLE_BQ_LOAD(0);
+  constexpr bool PF = HD <= 64;   // d = 128 has no registers to spare for a chunk in flight
+  if (PF) CASTLE_BQ_LOAD(0);
   for (int k0 = 0; k0 < kend; k0 += kCK) {
     const int Kb = k0 / kNB;
     __syncthreads();
+    if (!PF) CASTLE_BQ_LOAD(k0);
     pkc.store(s_kc, LDK);
     pvc.store(s_vc, LDK);
     pqu.store(s_qu, LDK);
     if (Kb < blk0) pu0.store(s_ub0, LDK);
     if (Kb < blk1 && blk1 < a.s.nblk) pu1.store(s_ub1, LDK);
-    if (Kb <= blk0 && blk0 <= a.s.nblk - 2) pg0.store(s_g0, LDK);
-    if (Kb <= blk1 && blk1 <= a.s.nblk - 2) pg1.store(s_g1, LDK);
-    if (k0 + kCK < kend) CASTLE_BQ_LOAD(k0 + kCK);   // in flight while this chunk is processed
+    if (DO_S && Kb <= blk0 && blk0 <= a.s.nblk - 2) pg0.store(s_g0, LDK);
+    if (DO_S && Kb <= blk1 && blk1 <= a.s.nblk - 2) pg1.store(s_g1, LDK);
+    if (PF && k0 + kCK < kend) CASTLE_BQ_LOAD(k0 + kCK);   // in flight while this chunk is processed
     __syncthreads();
     const bool active = Kb <= Iw;
 
@@ -538,17 +556,21 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
         ds[r] = dsv;
         dsu[r] = -dsv * sp;
       }
+      if constexpr (DO_S) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) st4<T>(s_dsut + (jw + c) * LDC + 32 * kt + 8 * q + 4 * g, pack4<T>(dsu, q));
+        for (int q = 0; q < 4; ++q) st4<T>(s_dsut + (jw + c) * LDC + 32 * kt + 8 * q + 4 * g, pack4<T>(dsu, q));
+      }
       {
         frag<T> okt[2][NT], out[2][NT], oat[2][BT];
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
           const int kc0 = 32 * kt + 16 * s2;
+          if constexpr (DO_Q) {
 #pragma unroll
-          for (int nt = 0; nt < NT; ++nt) {
-            okt[s2][nt] = ld_free<T, true>(s_kc, LDK, 32 * nt, HD, kc0, c, g);
-            out[s2][nt] = ld_free<T, true>(s_ubw, LDK, 32 * nt, HD, kc0, c, g);
+            for (int nt = 0; nt < NT; ++nt) {
+              okt[s2][nt] = ld_free<T, true>(s_kc, LDK, 32 * nt, HD, kc0, c, g);
+              out[s2][nt] = ld_free<T, true>(s_ubw, LDK, 32 * nt, HD, kc0, c, g);
+            }
           }
 #pragma unroll
           for (int jt = 0; jt < BT; ++jt) oat[s2][jt] = ld_chain<T>(s_at, LDC, cb + 32 * jt + c, kc0, g);
@@ -557,10 +579,12 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
           const frag<T> fds = chain<T>(ds, s2), fdsu = chain<T>(dsu, s2);
+          if constexpr (DO_Q) {
 #pragma unroll
-          for (int nt = 0; nt < NT; ++nt) {
-            mma(dqc[nt], okt[s2][nt], fds);
-            if (Kb < Iw) mma(dqc[nt], out[s2][nt], fdsu);
+            for (int nt = 0; nt < NT; ++nt) {
+              mma(dqc[nt], okt[s2][nt], fds);
+              if (Kb < Iw) mma(dqc[nt], out[s2][nt], fdsu);
+            }
           }
 #pragma unroll
           for (int jt = 0; jt < BT; ++jt)
@@ -572,7 +596,7 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
 
     // phase 2: this lane's row is a lookahead source j; needs some key k < j
 #pragma unroll
-    for (int kt = 0; kt < CKT; ++kt) {
+    for (int kt = 0; kt < (DO_S ? CKT : 0); ++kt) {
       const int ks = k0 + 32 * kt;
       if (!(active && ks < i0w + 31)) continue;
       acc_t dA;
@@ -646,7 +670,7 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
   }
   __syncthreads();
 #pragma unroll
-  for (int jt = 0; jt < BT; ++jt) {
+  for (int jt = 0; jt < (DO_Q ? BT : 0); ++jt) {
     if (32 * jt >= lw + 32) continue;
 #pragma unroll
     for (int s2 = 0; s2 < 2; ++s2) {
@@ -657,7 +681,7 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
     }
   }
 #pragma unroll
-  for (int s = 0; s < TS; ++s) {
+  for (int s = 0; s < (DO_S ? TS : 0); ++s) {
     if (s < ifirst) continue;
     // B operand: source j = lw + c on lanes, queries i = 16 s .. natural order, from dT[i][j]
     const frag<T> fdt = ld_free<T, false>(e_dtw, LDT, lw, kNB, 16 * s, c, g);
@@ -666,35 +690,63 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
       mma(dvu[nt], ld_free<T, false>(e_qcw, LDK, 32 * nt, HD, 16 * s, c, g), fdt);
   }
   if (i < L) {
-    store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqc, b, h) + (int64_t)i * a.dqc.sl, dqc, c0, g);
-    store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dku, b, h) + (int64_t)i * a.dku.sl, dku, c0 * kLn2, g);
-    store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvu, b, h) + (int64_t)i * a.dvu.sl, dvu, kLn2, g);
+    if constexpr (DO_Q) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqc, b, h) + (int64_t)i * a.dqc.sl, dqc, c0, g);
+    if constexpr (DO_S) {
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dku, b, h) + (int64_t)i * a.dku.sl, dku, c0 * kLn2, g);
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvu, b, h) + (int64_t)i * a.dvu.sl, dvu, kLn2, g);
+    }
   }
 }
 
 // ---------------------------------------------------------------------------
+template <typename T, typename TI, int HD, int PART> static int launch_bwd_part(const BwdArgs& a, hipStream_t stream) {
+  const int BH = a.s.B * a.s.H;
+  constexpr int key_lds = bwd_key_lds_bytes<T, HD>(), query_lds = bwd_query_lds_bytes<T, HD>();
+  static bool configured = false;   // raising the dynamic-LDS limit is idempotent, so a race is harmless
+  if (!configured) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_key_kernel<T, TI, HD, PART>), hipFuncAttributeMaxDynamicSharedMemorySize, key_lds) != hipSuccess) return -3;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_query_kernel<T, TI, HD, PART>), hipFuncAttributeMaxDynamicSharedMemorySize, query_lds) != hipSuccess) return -3;
+    configured = true;
+  }
+  return 0;
+}
+
 template <typename T, typename TI, int HD> static int launch_bwd_t(const BwdArgs& a, hipStream_t stream) {
   const int BH = a.s.B * a.s.H;
   constexpr int key_lds = bwd_key_lds_bytes<T, HD>(), query_lds = bwd_query_lds_bytes<T, HD>();
   if (key_lds > kMaxLds || query_lds > kMaxLds) return -2;
-  static bool configured = false;   // raising the dynamic-LDS limit is idempotent, so a race is harmless
-  if (!configured) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_key_kernel<T, TI, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, key_lds) != hipSuccess) return -3;
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_query_kernel<T, TI, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, query_lds) != hipSuccess) return -3;
-    configured = true;
+  constexpr bool SPLIT = HD > 64;   // two passes per kernel, half of the outputs each
+  int rc = 0;
+  if constexpr (SPLIT) {
+    rc = launch_bwd_part<T, TI, HD, 1>(a, stream);
+    if (rc == 0) rc = launch_bwd_part<T, TI, HD, 2>(a, stream);
+  } else {
+    rc = launch_bwd_part<T, TI, HD, 0>(a, stream);
   }
+  if (rc != 0) return rc;
   constexpr int RPB = kThreads / (HD / elem_traits<T>::vec16);
+  const dim3 grid(a.s.Lp / 128 * BH), block(kThreads);
   {
     ProfScope ps(kSlotDelta, stream);
-    hipLaunchKernelGGL((delta_kernel<TI, HD>), dim3((a.s.Lp + RPB - 1) / RPB, BH), dim3(kThreads), 0, stream, a);
+    hipLaunchKernelGGL((delta_kernel<TI, HD>), dim3((a.s.Lp + RPB - 1) / RPB, BH), block, 0, stream, a);
   }
   {
     ProfScope ps(kSlotBwdKey, stream);
-    hipLaunchKernelGGL((bwd_key_kernel<T, TI, HD>), dim3(a.s.Lp / 128 * BH), dim3(kThreads), key_lds, stream, a);
+    if constexpr (SPLIT) {
+      hipLaunchKernelGGL((bwd_key_kernel<T, TI, HD, 2>), grid, block, key_lds, stream, a);
+      hipLaunchKernelGGL((bwd_key_kernel<T, TI, HD, 1>), grid, block, key_lds, stream, a);
+    } else {
+      hipLaunchKernelGGL((bwd_key_kernel<T, TI, HD, 0>), grid, block, key_lds, stream, a);
+    }
   }
   {
     ProfScope ps(kSlotBwdQuery, stream);
-    hipLaunchKernelGGL((bwd_query_kernel<T, TI, HD>), dim3(a.s.Lp / 128 * BH), dim3(kThreads), query_lds, stream, a);
+    if constexpr (SPLIT) {
+      hipLaunchKernelGGL((bwd_query_kernel<T, TI, HD, 1>), grid, block, query_lds, stream, a);
+      hipLaunchKernelGGL((bwd_query_kernel<T, TI, HD, 2>), grid, block, query_lds, stream, a);
+    } else {
+      hipLaunchKernelGGL((bwd_query_kernel<T, TI, HD, 0>), grid, block, query_lds, stream, a);
+    }
   }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
@@ -704,7 +756,10 @@ template <typename T, typename TI> static int launch_bwd_d(const BwdArgs& a, hip
     case 16: return launch_bwd_t<T, TI, 16>(a, stream);
     case 32: return launch_bwd_t<T, TI, 32>(a, stream);
     case 64: return launch_bwd_t<T, TI, 64>(a, stream);
-    default: return -2;   // d = 128: the register budget of the key-stationary kernel is exceeded
+    case 128:
+      if constexpr (sizeof(T) == 2) return launch_bwd_t<T, TI, 128>(a, stream);
+      return -2;
+    default: return -2;
   }
 }
 

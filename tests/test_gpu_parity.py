@@ -65,6 +65,7 @@ BWD_CASES = [
     (1, 1, 1, 64, torch.float32), (1, 2, 9, 16, torch.float32), (2, 2, 64, 64, torch.float32),
     (1, 2, 200, 32, torch.float32), (1, 2, 321, 64, torch.float32), (2, 2, 384, 64, torch.bfloat16),
     (1, 2, 300, 32, torch.bfloat16), (1, 2, 256, 16, torch.bfloat16), (1, 2, 256, 64, torch.float16),
+    (1, 2, 300, 128, torch.bfloat16), (1, 1, 130, 128, torch.float16),
 ]
 
 
