@@ -30,6 +30,10 @@ if ROOT not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16/fp16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 1 GiB copy
+# (profiles/castle_cfg2_cfg4_pmc_hbm_traffic.txt).  Recorded values, not measured by this script.
+MEASURED_TRAFFIC_BYTES = {"bwd_key": 1613.2e6, "bwd_query": 1434.1e6, "decode_stream": 378.9e6}
+
 # algorithmic contractions (unit: B*H*L^2*d flop = 2*d flop per causal pair) attributed to each kernel
 KERNEL_UNITS = {"tqv": 0.0, "scan": 2.0, "attn": 3.0, "delta": 0.0, "bwd_key": 9.0, "bwd_query": 4.0}
 
@@ -90,7 +94,8 @@ def bench_layer(steps, warmup):
         "core": {"flop": core, "ms": round(core_ms, 4), "tflops": round(core / (core_ms * 1e-3) / 1e12, 2),
                  "frac_of_peak": round(core / (core_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4), "kernels": table},
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None},
+                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(dom)},
         "global_batch": B, "seq_len": L,
     }
 
@@ -137,7 +142,8 @@ def bench_decode(n_steps=512, prefill=2048):
     out["kernel_ms_per_step"] = round(kern_s * 1e3 / max(1, len(stream_ms)), 4)
     out["kernel_tokens_per_s"] = round(B * len(stream_ms) / kern_s, 1)
     out["roofline"] = {"bound": "hbm", "kernel": "decode_stream", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
-                       "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None}
+                       "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4),
+                       "traffic": MEASURED_TRAFFIC_BYTES["decode_stream"]}
     out["workload"] = f"config 4: B{B} H{H} d{d} bf16, prefill {prefill}, {n_steps} cached steps"
     for k in ("prefill_tokens_per_s", "tokens_per_s", "ms_per_decode_step"):
         out[k] = round(out[k], 3)
