@@ -168,18 +168,11 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   for (int I = a.s.nblk - 1; I >= I0; --I) {
     const bool active = I >= Iw;
     if (DO_QG && active && I <= a.s.nblk - 2) {   // reverse state as of block I
-      T* dst = gsnap + (gsnap_off(I) + k) * HD;
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int n = 32 * nt + 8 * q + 4 * g;
-          if (n < HD) st4<T>(dst + n, pack4<T>(G[nt], q));
-        }
+      store_snap_tile<T, HD, NT>(gsnap + (gsnap_off(I) + kw0) * HD, G, c, g);
     }
     if (I > Iw) {
 #pragma unroll
-      for (int s = 0; s < KS; ++s) fub[s] = ldg_nat<T>(usnap + usnap_off(I) * HD, HD, k, 16 * s + 8 * g, true);
+      for (int s = 0; s < KS; ++s) fub[s] = ldg_snap_nat<T>(usnap + (usnap_off(I) + kw0) * HD, c, 16 * s + 8 * g);
     }
     __syncthreads();
     const int64_t r0 = (int64_t)I * kNB;
@@ -450,7 +443,7 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
 
   // staging: every thread carries one 16-byte piece of each of the 7 tiles of the next chunk
   RowStage<T, TI, kCK, HD> pkc, pvc, pqu;
-  RowStage<T, T, kCK, HD> pu0, pu1, pg0, pg1;
+  SnapStage<T, kCK, HD> pu0, pu1, pg0, pg1;
   const int blk0 = Ifirst, blk1 = Ifirst + 1;
 #define CASTLE_BQ_LOAD(K0)                                                                                      \
   do {                                                                                                          \
@@ -458,10 +451,10 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
     pkc.load(kc, a.kc.sl, (K0), L);                                                                             \
     pvc.load(vc, a.vc.sl, (K0), L);                                                                             \
     pqu.load(qu, a.qu.sl, (K0), L);                                                                             \
-    if (kb_ < blk0) pu0.load(usnap + usnap_off(blk0) * HD, HD, (K0), (int64_t)1 << 40);                          \
-    if (kb_ < blk1 && blk1 < a.s.nblk) pu1.load(usnap + usnap_off(blk1) * HD, HD, (K0), (int64_t)1 << 40);        \
-    if (DO_S && kb_ <= blk0 && blk0 <= a.s.nblk - 2) pg0.load(gsnap + gsnap_off(blk0) * HD, HD, (K0), (int64_t)1 << 40);  \
-    if (DO_S && kb_ <= blk1 && blk1 <= a.s.nblk - 2) pg1.load(gsnap + gsnap_off(blk1) * HD, HD, (K0), (int64_t)1 << 40);  \
+    if (kb_ < blk0) pu0.load(usnap + (usnap_off(blk0) + (K0)) * HD);                          \
+    if (kb_ < blk1 && blk1 < a.s.nblk) pu1.load(usnap + (usnap_off(blk1) + (K0)) * HD);        \
+    if (DO_S && kb_ <= blk0 && blk0 <= a.s.nblk - 2) pg0.load(gsnap + (gsnap_off(blk0) + (K0)) * HD);  \
+    if (DO_S && kb_ <= blk1 && blk1 <= a.s.nblk - 2) pg1.load(gsnap + (gsnap_off(blk1) + (K0)) * HD);  \
   } while (0)
 
   int kend = qb * QB + QB;

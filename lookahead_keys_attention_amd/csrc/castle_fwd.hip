@@ -119,14 +119,7 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(FwdArgs a) {
   }
   for (int I = I0; I < a.s.nblk; ++I) {
     if (I * kNB >= kw0 + 32) {   // all keys of this wave precede block I: snapshot
-      T* dst = snap + (usnap_off(I) + k) * HD;
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int n = 32 * nt + 8 * q + 4 * g;
-          if (n < HD) st4<T>(dst + n, pack4<T>(st[nt], q));
-        }
+      store_snap_tile<T, HD, NT>(snap + (usnap_off(I) + kw0) * HD, st, c, g);
     }
     __syncthreads();
     if (!PF) {
@@ -235,7 +228,7 @@ __global__ __launch_bounds__(kThreads, (sizeof(T) == 2 && HD <= 64) ? 2 : 1) voi
 
   RowStage<T, TI, kNB, HD> pkc, pqu;
   ColStage<T, TI, kNB, HD> pvc;
-  RowStage<T, T, kNB, HD> pub[NBLK_Q];
+  SnapStage<T, kNB, HD> pub[NBLK_Q];
   auto load_chunk = [&](int Kb) __attribute__((always_inline)) {
     pkc.load(kc, a.kc.sl, (int64_t)Kb * kNB, L);
     pvc.load(vc, a.vc.sl, (int64_t)Kb * kNB, L);
@@ -243,7 +236,7 @@ __global__ __launch_bounds__(kThreads, (sizeof(T) == 2 && HD <= 64) ? 2 : 1) voi
 #pragma unroll
     for (int q = 0; q < NBLK_Q; ++q) {
       const int blk = Ifirst + q;
-      if (Kb < blk && blk < a.s.nblk) pub[q].load(snap + usnap_off(blk) * HD, HD, (int64_t)Kb * kNB, (int64_t)1 << 40);
+      if (Kb < blk && blk < a.s.nblk) pub[q].load(snap + (usnap_off(blk) + (int64_t)Kb * kNB) * HD);
     }
   };
   auto store_chunk = [&](int Kb) __attribute__((always_inline)) {

@@ -447,6 +447,76 @@ __device__ __forceinline__ void work_item(int BH, int& rank, int& bh) {
   bh = blockIdx.x % BH;
 }
 
+// ---- state snapshots -------------------------------------------------------------------
+// A snapshot holds one state row (HD values) per key.  Keys are grouped by 32 ("snapshot
+// tile", 32*HD elements, tiles in key order); inside a tile the 16-byte pieces (V values of one
+// key) are stored piece-column major: element (key c, column n) sits at
+//   (n / V) * 32 * V + c * V + n % V.
+// The producers hold the state transposed in MFMA accumulators (rows n, one key per lane), so
+// each of their store instructions covers 512 contiguous bytes; consumers read whole tiles as
+// one contiguous run of pieces.
+template <typename T> __device__ __forceinline__ int snap_elem(int c, int n) {
+  constexpr int V = elem_traits<T>::vec16;
+  return (n / V) * 32 * V + c * V + n % V;
+}
+
+// Stores acc tiles st[nt] (rows n = 32 nt + .., lane (c, g) = key c of the tile) into one snapshot tile.
+template <typename T, int HD, int NT>
+__device__ __forceinline__ void store_snap_tile(T* tile, const acc_t (&st)[NT], int c, int g) {
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int n = 32 * nt + 8 * q + 4 * g;
+      if (n < HD) st4<T>(tile + snap_elem<T>(c, n), pack4<T>(st[nt], q));
+    }
+}
+
+// The natural-order operand fragment (columns 16 s + 8 g .. + 7 of key c) straight from a snapshot tile.
+template <typename T> __device__ __forceinline__ frag<T> ldg_snap_nat(const T* tile, int c, int col) {
+  constexpr int V = elem_traits<T>::vec16;
+  if constexpr (V == 8) {
+    return *reinterpret_cast<const frag_mem<T>*>(tile + snap_elem<T>(c, col));
+  } else {
+    frag<T> f;
+    const vec<T, 4> lo = *reinterpret_cast<const vec<T, 4>*>(tile + snap_elem<T>(c, col));
+    const vec<T, 4> hi = *reinterpret_cast<const vec<T, 4>*>(tile + snap_elem<T>(c, col + 4));
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { f[e] = lo[e]; f[4 + e] = hi[e]; }
+    return f;
+  }
+}
+
+// Two-phase staging of ROWS (a multiple of 32) snapshot rows into a row-major LDS tile.
+template <typename T, int ROWS, int COLS>
+struct SnapStage {
+  static constexpr int V = elem_traits<T>::vec16;
+  static constexpr int VPR = COLS / V;
+  static constexpr int TOTAL = ROWS * VPR;
+  static constexpr int N = (TOTAL + kThreads - 1) / kThreads;
+  static_assert(ROWS % 32 == 0, "whole snapshot tiles only");
+  vec<T, V> r[N];
+
+  // src: first element of the first tile (the tiles of consecutive key groups are contiguous)
+  __device__ __forceinline__ void load(const T* src) {
+#pragma unroll
+    for (int n = 0; n < N; ++n) {
+      const int v = threadIdx.x + n * kThreads;
+      if (v < TOTAL) r[n] = *reinterpret_cast<const vec<T, V>*>(src + (int64_t)v * V);
+    }
+  }
+  __device__ __forceinline__ void store(T* dst, int ld) const {
+#pragma unroll
+    for (int n = 0; n < N; ++n) {
+      const int v = threadIdx.x + n * kThreads;
+      if (v < TOTAL) {
+        const int tile = v / (32 * VPR), piece = (v / 32) % VPR, c = v % 32;
+        *reinterpret_cast<vec<T, V>*>(dst + (32 * tile + c) * ld + piece * V) = r[n];
+      }
+    }
+  }
+};
+
 // offsets (in rows) of block I inside the snapshot arrays
 __host__ __device__ inline int64_t usnap_off(int64_t I) { return (int64_t)kNB * I * (I - 1) / 2; }   // I >= 1, I*kNB rows
 __host__ __device__ inline int64_t gsnap_off(int64_t I) { return (int64_t)kNB * I * (I + 1) / 2; }   // I <= nblk-2, (I+1)*kNB rows
