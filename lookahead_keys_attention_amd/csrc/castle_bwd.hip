@@ -350,6 +350,328 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
 }
 
 // ---------------------------------------------------------------------------
+// Key-stationary backward with two wave roles (16-bit compute types, d <= 64): 512 threads,
+// waves 0-3 "score" waves, waves 4-7 "gradient" waves; pair (w, w + 4) owns keys
+// kb*128 + 32 w .. + 31 and is expected to share a SIMD, so the element-wise chain of one role
+// overlaps the MFMAs of the other.  Per 64-query block I (swept from the last one down):
+//   score wave:    gate A_KI (-> A(1-A) for the partner), then per 32-query sub-tile the scores,
+//                  P, dS, dSu, handed over through LDS as [key][query] tiles
+//   gradient wave: reverse state G (snapshot, G Vu^T), dVc, dKc, G, dA from the handed tiles,
+//                  then dZ and dQu
+// The gradient wave runs one sub-tile behind the score wave; four barriers per block.
+template <typename T, int HD> constexpr int bwd_key2_lds_bytes() {
+  int b = bwd_key_lds_bytes<T, HD>();
+  b += 4 * 3 * a16((int)sizeof(T) * 32 * lds_ld<T>(kNB));   // P, dS, dSu per wave pair
+  b += 4 * a16((int)sizeof(T) * 32 * lds_ld<T>(kNB));       // A (1 - A) per wave pair
+  return b;
+}
+
+template <typename T, typename TI, int HD>
+__global__ __launch_bounds__(2 * kThreads, 1) void bwd_key2_kernel(BwdArgs a) {
+  static_assert(sizeof(T) == 2 && HD <= 64, "two-role kernel: 16-bit operands, d <= 64");
+  constexpr int KS = HD / 16;
+  constexpr int HDP = HD < 32 ? 32 : HD;
+  constexpr int NT = HDP / 32;
+  constexpr int BT = kNB / 32;
+  constexpr int LDK = lds_ld<T>(HD), LDU = lds_ld_chain<T>(HD), LDT = lds_ld_chain<T>(kNB);
+  constexpr int LDX = lds_ld<T>(kNB);
+
+  Carver cv{castle_smem};
+  T* s_qc = cv.take<T>(kNB * LDK);
+  T* s_do = cv.take<T>(kNB * LDK);
+  T* s_ku = cv.take<T>(kNB * LDK);
+  T* s_vu = cv.take<T>(kNB * LDU);
+  T* s_t = cv.take<T>(kNB * LDT);
+  float* s_lse = cv.take<float>(kNB);
+  float* s_delta = cv.take<float>(kNB);
+  T* s_x = cv.take<T>(4 * 3 * 32 * LDX);
+  T* s_w = cv.take<T>(4 * 32 * LDX);
+
+  int kb, bh;
+  work_item(a.s.B * a.s.H, kb, bh);
+  const int b = bh / a.s.H, h = bh % a.s.H;
+  const int lane = lane_id(), wave = wave_id(), c = lane & 31, g = lane >> 5;
+  const bool scorer = wave < 4;
+  const int pw = wave & 3;
+  const int L = a.s.L;
+  const float c0 = a.s.scale, c1 = a.s.scale * kLog2e;
+  const int kw0 = kb * 128 + 32 * pw;
+  const int k = kw0 + c;
+  const int Iw = kw0 / kNB;
+  const int I0 = (kb * 128) / kNB;
+  T* x_p = s_x + pw * 3 * 32 * LDX;   // [key][query of the block]
+  T* x_ds = x_p + 32 * LDX;
+  T* x_dsu = x_ds + 32 * LDX;
+  T* x_w = s_w + pw * 32 * LDX;       // [key][source of the block]
+
+  const TI* qc = head_ptr<TI>(a.qc, b, h);
+  const TI* ku = head_ptr<TI>(a.ku, b, h);
+  const TI* vu = head_ptr<TI>(a.vu, b, h);
+  const TI* dout = head_ptr<TI>(a.dout, b, h);
+  const T* tb = reinterpret_cast<const T*>(a.ws.t_blk) + (int64_t)bh * a.s.Lp * kNB;
+  // All 512 threads stage the five tiles of a block: the loads of block I - 1 are issued right
+  // after the tiles of block I have been written and stay in flight for the whole block.
+#define CASTLE_BK2_STAGE_DECL                                \
+  RowStage<T, TI, kNB, HD, 2 * kThreads> pqc, pdo, pku, pvu; \
+  RowStage<T, T, kNB, kNB, 2 * kThreads> ptb
+#define CASTLE_BK2_STAGE_LOAD(I_)                            \
+  do {                                                       \
+    const int64_t r_ = (int64_t)(I_) * kNB;                  \
+    pqc.load(qc, a.qc.sl, r_, L);                            \
+    pdo.load(dout, a.dout.sl, r_, L);                        \
+    pku.load(ku, a.ku.sl, r_, L);                            \
+    pvu.load(vu, a.vu.sl, r_, L);                            \
+    ptb.load(tb, kNB, r_, (int64_t)1 << 40);                 \
+  } while (0)
+#define CASTLE_BK2_STAGE_STORE()                             \
+  do {                                                       \
+    pqc.store_scaled(s_qc, LDK, c1);                         \
+    pdo.store(s_do, LDK);                                    \
+    pku.store(s_ku, LDK);                                    \
+    pvu.store_halves(s_vu, LDU);                             \
+    ptb.store_halves(s_t, LDT);                              \
+  } while (0)
+
+  if (scorer) {
+    const TI* kc = head_ptr<TI>(a.kc, b, h);
+    const TI* vc = head_ptr<TI>(a.vc, b, h);
+    const TI* qu = head_ptr<TI>(a.qu, b, h);
+    const T* usnap = reinterpret_cast<const T*>(a.ws.usnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
+    const float* lse = a.ws.lse + (int64_t)bh * a.s.Lp;
+    const float* delta = a.delta + (int64_t)bh * a.s.Lp;
+
+    frag<T> fkc[KS], fvc[KS], fqu[KS], fub[KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      fkc[s] = ldg_nat<T, TI>(kc, a.kc.sl, k, 16 * s + 8 * g, k < L);
+      fvc[s] = ldg_nat<T, TI>(vc, a.vc.sl, k, 16 * s + 8 * g, k < L);
+      fqu[s] = ldg_nat_scaled<T, TI>(qu, a.qu.sl, k, 16 * s + 8 * g, k < L, -c1);
+      fub[s] = zero_frag<T>();
+    }
+    CASTLE_BK2_STAGE_DECL;
+#define CASTLE_BK2_LOAD(I_)                                                                        \
+  do {                                                                                             \
+    CASTLE_BK2_STAGE_LOAD(I_);                                                                     \
+    if ((I_) > Iw) {                                                                               \
+      _Pragma("unroll") for (int s = 0; s < KS; ++s)                                               \
+        fub[s] = ldg_snap_nat<T>(usnap + (usnap_off(I_) + kw0) * HD, c, 16 * s + 8 * g);           \
+    }                                                                                              \
+  } while (0)
+
+    CASTLE_BK2_LOAD(a.s.nblk - 1);
+    frag<T> fa[BT][2];
+    for (int I = a.s.nblk - 1; I >= I0; --I) {
+      const bool active = I >= Iw;
+      const bool inter = I > Iw;   // lookahead state from earlier blocks exists
+      CASTLE_BK2_STAGE_STORE();
+      if (threadIdx.x < kNB) {
+        const int64_t i = (int64_t)I * kNB + threadIdx.x;
+        s_lse[threadIdx.x] = i < L ? lse[i] * kLog2e : INFINITY;
+        s_delta[threadIdx.x] = i < L ? delta[i] : 0.f;
+      }
+      __syncthreads();   // 1: tiles staged
+      if (I > I0) CASTLE_BK2_STAGE_LOAD(I - 1);   // in flight for the whole block
+#pragma unroll
+      for (int it = 0; it < BT; ++it) {
+        if (it == 0 && active) {
+          // gate tiles A^T[j rows, k lanes] of the whole source block
+#pragma unroll
+          for (int jt = 0; jt < BT; ++jt) {
+            acc_t aT;
+            zero(aT);
+            {
+              frag<T> oku[KS];
+#pragma unroll
+              for (int s = 0; s < KS; ++s) oku[s] = ld_nat<T>(s_ku, LDK, 32 * jt + c, 16 * s + 8 * g);
+              __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+              for (int s = 0; s < KS; ++s) mma(aT, oku[s], fqu[s]);
+            }
+            const int j0 = I * kNB + 32 * jt;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) aT[r] = fast_rcp(1.f + fast_exp2(aT[r]));
+            if (j0 <= kw0 + 31) {   // tile touches the diagonal: keep j > k only
+#pragma unroll
+              for (int r = 0; r < 16; ++r)
+                if (j0 + acc_row(r, g) <= k) aT[r] = 0.f;
+            }
+            fa[jt][0] = chain<T>(aT, 0);
+            fa[jt][1] = chain<T>(aT, 1);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) aT[r] = aT[r] * (1.f - aT[r]);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) st4<T>(x_w + c * LDX + 32 * jt + 8 * q + 4 * g, pack4<T>(aT, q));
+          }
+        }
+        const int i0 = I * kNB + 32 * it;
+        if (active && i0 + 31 >= kw0) {   // else every query precedes every key of this wave
+          acc_t sc, su, dp;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int il = 32 * it + acc_row(r, g);
+            sc[r] = -s_lse[il];
+            dp[r] = -s_delta[il];
+            su[r] = 0.f;
+          }
+          {
+            frag<T> oq[KS], od[KS], ot[BT][2];
+#pragma unroll
+            for (int s = 0; s < KS; ++s) {
+              oq[s] = ld_nat<T>(s_qc, LDK, 32 * it + c, 16 * s + 8 * g);
+              od[s] = ld_nat<T>(s_do, LDK, 32 * it + c, 16 * s + 8 * g);
+            }
+#pragma unroll
+            for (int jt = 0; jt < BT; ++jt)
+#pragma unroll
+              for (int s2 = 0; s2 < 2; ++s2)
+                if (jt <= it) ot[jt][s2] = ld_chain<T>(s_t, LDT, 32 * it + c, 32 * jt + 16 * s2, g);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int s = 0; s < KS; ++s) {
+              mma(sc, oq[s], fkc[s]);
+              mma(dp, od[s], fvc[s]);
+            }
+            if (inter) {
+#pragma unroll
+              for (int s = 0; s < KS; ++s) mma(su, oq[s], fub[s]);
+            }
+#pragma unroll
+            for (int jt = 0; jt < BT; ++jt)
+#pragma unroll
+              for (int s2 = 0; s2 < 2; ++s2)
+                if (jt <= it) mma(su, ot[jt][s2], fa[jt][s2]);
+          }
+          acc_t ds, dsu;
+          const bool diag = i0 < kw0 + 31;   // tile touches the diagonal
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float sg = fast_rcp(1.f + fast_exp2(-su[r]));
+            float p = fast_exp2(__builtin_fmaf(-su[r], sg, sc[r]));   // sc carries -lse
+            if (diag && i0 + acc_row(r, g) < k) p = 0.f;
+            const float dsv = p * dp[r];                      // dp carries -delta
+            const float y = su[r] * kLn2;                     // true Su
+            const float t = __builtin_fmaf(-y, sg, y);        // y (1 - sigmoid)
+            const float sp = __builtin_fmaf(sg, t, sg);       // silu'(y)
+            sc[r] = p;
+            ds[r] = dsv;
+            dsu[r] = -dsv * sp;
+          }
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int o = c * LDX + 32 * it + 8 * q + 4 * g;
+            st4<T>(x_p + o, pack4<T>(sc, q));
+            st4<T>(x_ds + o, pack4<T>(ds, q));
+            st4<T>(x_dsu + o, pack4<T>(dsu, q));
+          }
+        }
+        __syncthreads();   // 2, 3: sub-tile handed over
+      }
+      if (I - 1 > Iw && I > I0) {   // lookahead state as of the next block
+#pragma unroll
+        for (int s = 0; s < KS; ++s) fub[s] = ldg_snap_nat<T>(usnap + (usnap_off(I - 1) + kw0) * HD, c, 16 * s + 8 * g);
+      }
+      __syncthreads();   // 4: tiles free
+    }
+#undef CASTLE_BK2_LOAD
+  } else {
+    T* gsnap = reinterpret_cast<T*>(a.gsnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
+    acc_t dvc[NT], dkc[NT], dqu[NT], G[NT];   // [n rows, k lanes]
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) { zero(dvc[nt]); zero(dkc[nt]); zero(dqu[nt]); zero(G[nt]); }
+    CASTLE_BK2_STAGE_DECL;
+    CASTLE_BK2_STAGE_LOAD(a.s.nblk - 1);
+    for (int I = a.s.nblk - 1; I >= I0; --I) {
+      const bool active = I >= Iw;
+      CASTLE_BK2_STAGE_STORE();
+      if (active && I <= a.s.nblk - 2)   // reverse state as of block I
+        store_snap_tile<T, HD, NT>(gsnap + (gsnap_off(I) + kw0) * HD, G, c, g);
+      __syncthreads();   // 1
+      if (I > I0) CASTLE_BK2_STAGE_LOAD(I - 1);
+      // dA^T[j rows, k lanes], second term first: G (before this block) times Vu^T
+      acc_t dA[BT];
+#pragma unroll
+      for (int jt = 0; jt < BT; ++jt) {
+        zero(dA[jt]);
+        if (active) {
+          frag<T> ovu[KS];
+#pragma unroll
+          for (int s = 0; s < KS; ++s) ovu[s] = ld_chain<T>(s_vu, LDU, 32 * jt + c, 16 * s, g);
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int s = 0; s < KS; ++s) mma(dA[jt], ovu[s], chain<T>(G[s / 2], s % 2));
+        }
+      }
+#pragma unroll
+      for (int it = 0; it < BT; ++it) {
+        __syncthreads();   // 2, 3: sub-tile `it` is there
+        const int i0 = I * kNB + 32 * it;
+        if (active && i0 + 31 >= kw0) {
+#pragma unroll
+          for (int s2 = 0; s2 < 2; ++s2) {
+            const int ic = 32 * it + 16 * s2;
+            frag<T> odt[NT], oqt[NT], ott[BT];
+            const frag<T> fp = ld_nat<T>(x_p, LDX, c, ic + 8 * g);
+            const frag<T> fds = ld_nat<T>(x_ds, LDX, c, ic + 8 * g);
+            const frag<T> fdsu = ld_nat<T>(x_dsu, LDX, c, ic + 8 * g);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+              odt[nt] = ld_free<T, false>(s_do, LDK, 32 * nt, HD, ic, c, g);
+              oqt[nt] = ld_free<T, false>(s_qc, LDK, 32 * nt, HD, ic, c, g);
+            }
+#pragma unroll
+            for (int jt = 0; jt < BT; ++jt)
+              if (jt <= it) ott[jt] = ld_free<T, false>(s_t, LDT, 32 * jt, kNB, ic, c, g);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+              mma(dvc[nt], odt[nt], fp);
+              mma(dkc[nt], oqt[nt], fds);
+              mma(G[nt], oqt[nt], fdsu);
+            }
+#pragma unroll
+            for (int jt = 0; jt < BT; ++jt)
+              if (jt <= it) mma(dA[jt], ott[jt], fdsu);
+          }
+        }
+      }
+      // dZ^T = dA^T * A (1 - A)  ->  dQu
+      if (active) {
+#pragma unroll
+        for (int jt = 0; jt < BT; ++jt) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const vec<T, 4> w = *reinterpret_cast<const vec4_mem<T>*>(x_w + c * LDX + 32 * jt + 8 * q + 4 * g);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) dA[jt][4 * q + e] *= (float)w[e];
+          }
+          frag<T> okt[2][NT];
+#pragma unroll
+          for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) okt[s2][nt] = ld_free<T, true>(s_ku, LDK, 32 * nt, HD, 32 * jt + 16 * s2, c, g);
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int s2 = 0; s2 < 2; ++s2) {
+            const frag<T> fdz = chain<T>(dA[jt], s2);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) mma(dqu[nt], okt[s2][nt], fdz);
+          }
+        }
+      }
+      __syncthreads();   // 4
+    }
+    if (k < L) {
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dkc, b, h) + (int64_t)k * a.dkc.sl, dkc, kLn2, g);
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvc, b, h) + (int64_t)k * a.dvc.sl, dvc, 1.f, g);
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqu, b, h) + (int64_t)k * a.dqu.sl, dqu, c0 * kLn2, g);
+    }
+  }
+#undef CASTLE_BK2_STAGE_DECL
+#undef CASTLE_BK2_STAGE_LOAD
+#undef CASTLE_BK2_STAGE_STORE
+}
+
+// ---------------------------------------------------------------------------
 constexpr int kCK = 32;   // keys per chunk in the query-stationary backward
 
 template <typename T, int HD> constexpr int bwd_query_lds_bytes() {
@@ -709,6 +1031,14 @@ template <typename T, typename TI, int HD> static int launch_bwd_t(const BwdArgs
   constexpr int key_lds = bwd_key_lds_bytes<T, HD>(), query_lds = bwd_query_lds_bytes<T, HD>();
   if (key_lds > kMaxLds || query_lds > kMaxLds) return -2;
   constexpr bool SPLIT = HD > 64;   // two passes per kernel, half of the outputs each
+  constexpr bool TWO_ROLE = sizeof(T) == 2 && HD <= 64;
+  if constexpr (TWO_ROLE) {
+    static bool configured2 = false;
+    if (!configured2) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_key2_kernel<T, TI, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_key2_lds_bytes<T, HD>()) != hipSuccess) return -3;
+      configured2 = true;
+    }
+  }
   int rc = 0;
   if constexpr (SPLIT) {
     rc = launch_bwd_part<T, TI, HD, 1>(a, stream);
@@ -728,6 +1058,9 @@ template <typename T, typename TI, int HD> static int launch_bwd_t(const BwdArgs
     if constexpr (SPLIT) {
       hipLaunchKernelGGL((bwd_key_kernel<T, TI, HD, 2>), grid, block, key_lds, stream, a);
       hipLaunchKernelGGL((bwd_key_kernel<T, TI, HD, 1>), grid, block, key_lds, stream, a);
+    } else if constexpr (TWO_ROLE) {
+      constexpr int key2_lds = bwd_key2_lds_bytes<T, HD>();
+      hipLaunchKernelGGL((bwd_key2_kernel<T, TI, HD>), grid, dim3(2 * kThreads), key2_lds, stream, a);
     } else {
       hipLaunchKernelGGL((bwd_key_kernel<T, TI, HD, 0>), grid, block, key_lds, stream, a);
     }

@@ -240,18 +240,18 @@ template <typename T> __host__ __device__ constexpr int lds_ld_chain(int cols) {
 // registers (zeros beyond row_end), store() converts them to T and writes the row-major LDS tile.
 // Splitting the phases lets a kernel issue the loads of the next tile before computing on the
 // current one.
-template <typename T, typename TI, int ROWS, int COLS>
+template <typename T, typename TI, int ROWS, int COLS, int THREADS = kThreads>
 struct RowStage {
   static constexpr int V = elem_traits<T>::vec16;
   static constexpr int VPR = COLS / V;
   static constexpr int TOTAL = ROWS * VPR;
-  static constexpr int N = (TOTAL + kThreads - 1) / kThreads;
+  static constexpr int N = (TOTAL + THREADS - 1) / THREADS;
   vec<TI, V> r[N];
 
   __device__ __forceinline__ void load(const TI* src, int64_t row_stride, int64_t row0, int64_t row_end) {
 #pragma unroll
     for (int n = 0; n < N; ++n) {
-      const int v = threadIdx.x + n * kThreads;
+      const int v = threadIdx.x + n * THREADS;
 #pragma unroll
       for (int e = 0; e < V; ++e) r[n][e] = (TI)0.f;
       if (v < TOTAL && row0 + v / VPR < row_end)
@@ -261,7 +261,7 @@ struct RowStage {
   __device__ __forceinline__ void store(T* dst, int ld) const {
 #pragma unroll
     for (int n = 0; n < N; ++n) {
-      const int v = threadIdx.x + n * kThreads;
+      const int v = threadIdx.x + n * THREADS;
       if (v < TOTAL) *reinterpret_cast<vec<T, V>*>(dst + (v / VPR) * ld + (v % VPR) * V) = cvt_vec<T, TI, V>(r[n]);
     }
   }
@@ -270,7 +270,7 @@ struct RowStage {
     constexpr int HV = V / 2;
 #pragma unroll
     for (int n = 0; n < N; ++n) {
-      const int v = threadIdx.x + n * kThreads;
+      const int v = threadIdx.x + n * THREADS;
       if (v < TOTAL) {
         const vec<T, V> x = cvt_vec<T, TI, V>(r[n]);
         typedef vec<T, HV> __attribute__((aligned(8))) half_mem;
@@ -286,7 +286,7 @@ struct RowStage {
   __device__ __forceinline__ void store_scaled(T* dst, int ld, float mul) const {
 #pragma unroll
     for (int n = 0; n < N; ++n) {
-      const int v = threadIdx.x + n * kThreads;
+      const int v = threadIdx.x + n * THREADS;
       if (v < TOTAL) {
         vec<float, V> f = __builtin_convertvector(r[n], vec<float, V>);
 #pragma unroll
