@@ -73,7 +73,9 @@ int castle_fwd(const castle_view4* qc, const castle_view4* kc, const castle_view
                const castle_view4* out, const castle_view4* U,
                void* workspace, int64_t workspace_bytes, void* stream);
 
-/* Bytes of extra device workspace castle_bwd needs (reverse state snapshots, delta). */
+/* Bytes of extra device workspace castle_bwd needs: reverse state snapshots, delta and, for the
+ * 16-bit element types at d <= 64, the dS / dSu score-gradient tiles its first kernel hands to its
+ * second (2 * B * H * Lp * Lp elements, Lp = L rounded up to 128). */
 int64_t castle_bwd_workspace_bytes(int B, int H, int L, int d, int dtype);
 
 /* Parallel backward.  Same operands as castle_fwd plus the forward output `out`, the

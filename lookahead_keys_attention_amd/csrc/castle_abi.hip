@@ -34,7 +34,7 @@ int64_t align_up(int64_t x, int64_t a) { return (x + a - 1) / a * a; }
 
 struct Geometry {
   int Lp, nblk;
-  int64_t lse_bytes, tblk_bytes, snap_bytes;
+  int64_t lse_bytes, tblk_bytes, snap_bytes, mat_bytes;
   int64_t off_lse, off_t, off_tt, off_snap, total;
 };
 
@@ -46,6 +46,8 @@ Geometry geometry(int B, int H, int L, int d, int es) {
   g.lse_bytes = align_up(BH * g.Lp * 4, 256);
   g.tblk_bytes = align_up(BH * g.Lp * kNB * es, 256);
   g.snap_bytes = align_up(BH * castle::snap_rows(g.nblk) * d * es, 256);
+  // dS / dSu tiles between the two backward kernels: only the 16-bit, d <= 64 path uses them
+  g.mat_bytes = (es == 2 && d <= 64) ? align_up(BH * g.Lp * g.Lp * es, 256) : 0;
   g.off_lse = 0;
   g.off_t = g.off_lse + g.lse_bytes;
   g.off_tt = g.off_t + g.tblk_bytes;
@@ -148,7 +150,7 @@ int64_t castle_bwd_workspace_bytes(int B, int H, int L, int d, int dtype) {
   const int rc = check_core(B, H, L, d, dtype);
   if (rc != CASTLE_OK) return rc;
   const Geometry g = geometry(B, H, L, d, elem_size(dtype));
-  return g.snap_bytes + g.lse_bytes;   // reverse-state snapshots + delta
+  return g.snap_bytes + g.lse_bytes + 2 * g.mat_bytes;   // reverse-state snapshots + delta + dS, dSu tiles
 }
 
 int castle_bwd(const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
@@ -169,7 +171,7 @@ int castle_bwd(const castle_view4* qc, const castle_view4* kc, const castle_view
   if (fwd_workspace == nullptr || reinterpret_cast<uintptr_t>(fwd_workspace) % 256 != 0 || fwd_workspace_bytes < g.total)
     return CASTLE_ERR_WORKSPACE;
   if (bwd_workspace == nullptr || reinterpret_cast<uintptr_t>(bwd_workspace) % 256 != 0 ||
-      bwd_workspace_bytes < g.snap_bytes + g.lse_bytes)
+      bwd_workspace_bytes < g.snap_bytes + g.lse_bytes + 2 * g.mat_bytes)
     return CASTLE_ERR_WORKSPACE;
 
   castle::BwdArgs a;
@@ -182,6 +184,8 @@ int castle_bwd(const castle_view4* qc, const castle_view4* kc, const castle_view
   a.ws = carve(const_cast<void*>(fwd_workspace), g);
   a.gsnap = bwd_workspace;
   a.delta = reinterpret_cast<float*>(static_cast<char*>(bwd_workspace) + g.snap_bytes);
+  a.ds_mat = g.mat_bytes ? static_cast<char*>(bwd_workspace) + g.snap_bytes + g.lse_bytes : nullptr;
+  a.dsu_mat = g.mat_bytes ? static_cast<char*>(bwd_workspace) + g.snap_bytes + g.lse_bytes + g.mat_bytes : nullptr;
   return castle::launch_bwd(a, dtype, (flags & CASTLE_FLAG_BF16_OPERANDS) != 0, static_cast<hipStream_t>(stream));
 }
 

@@ -575,6 +575,8 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_key2_kernel(BwdArgs a) {
 #undef CASTLE_BK2_LOAD
   } else {
     T* gsnap = reinterpret_cast<T*>(a.gsnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
+    T* ds_mat = reinterpret_cast<T*>(a.ds_mat) + (int64_t)bh * a.s.Lp * a.s.Lp;
+    T* dsu_mat = reinterpret_cast<T*>(a.dsu_mat) + (int64_t)bh * a.s.Lp * a.s.Lp;
     acc_t dvc[NT], dkc[NT], dqu[NT], G[NT];   // [n rows, k lanes]
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) { zero(dvc[nt]); zero(dkc[nt]); zero(dqu[nt]); zero(G[nt]); }
@@ -613,6 +615,11 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_key2_kernel(BwdArgs a) {
             const frag<T> fp = ld_nat<T>(x_p, LDX, c, ic + 8 * g);
             const frag<T> fds = ld_nat<T>(x_ds, LDX, c, ic + 8 * g);
             const frag<T> fdsu = ld_nat<T>(x_dsu, LDX, c, ic + 8 * g);
+            {   // hand the tile to the query-stationary kernel: 1 KB contiguous per store
+              const int64_t tile = ((int64_t)(kw0 / 32) * (a.s.Lp / 32) + i0 / 32) * 1024 + s2 * 512 + c * 16 + g * 8;
+              *reinterpret_cast<frag_mem<T>*>(ds_mat + tile) = fds;
+              *reinterpret_cast<frag_mem<T>*>(dsu_mat + tile) = fdsu;
+            }
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
               odt[nt] = ld_free<T, false>(s_do, LDK, 32 * nt, HD, ic, c, g);
@@ -1014,6 +1021,304 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
 }
 
 // ---------------------------------------------------------------------------
+// Query-stationary backward that consumes the dS / dSu tiles written by bwd_key2_kernel
+// (16-bit compute types, d <= 64): no score recomputation, only the gate.
+//   row = query i:   dQc += dS Kc + dSu U_I,  dT^T += A^T dSu^T
+//   row = source j:  dA = dSu^T T' + G' Vu^T,  dZ = dA A (1 - A),  dKu += dZ^T Qu,  dVu += A^T G'
+template <typename T> constexpr int kLdD = 128 + 8;   // dS / dSu tiles [key][128 queries]
+template <typename T> constexpr int kLdA = kCK + 8;   // gate tile [128 sources][key]
+template <typename T, int HD> constexpr int bwd_query2_lds_bytes() {
+  int b = 6 * a16((int)sizeof(T) * kCK * lds_ld<T>(HD));          // kc, qu, ub[2], g[2]
+  b += a16((int)sizeof(T) * 128 * kLdA<T>);                       // A^T [j][k]
+  b += 2 * a16((int)sizeof(T) * kCK * kLdD<T>);                   // dS, dSu [k][i]
+  int e = 4 * a16((int)sizeof(T) * kNB * lds_ld<T>(HD)) + 2 * a16((int)sizeof(T) * kNB * lds_ld_chain<T>(kNB));
+  return b > e ? b : e;
+}
+
+// Staging of the 4 consecutive 32x32 tiles (8 KB) that one chunk of 32 keys shares with the 128
+// queries of a workgroup.  Every wave instruction reads 1 KB contiguous; within 16 lanes the LDS
+// rows differ, which keeps the 16-byte stores conflict free.
+template <typename T>
+struct TileStage {
+  vec<T, 8> r[2];
+  __device__ __forceinline__ void load(const T* src) {
+#pragma unroll
+    for (int n = 0; n < 2; ++n) {
+      const int v = threadIdx.x + n * kThreads;
+      const int slab = v >> 6, l = v & 63;                       // slab = 2 * tile + s2
+      const int g = (l >> 4) & 1, k = (l & 15) + 16 * (l >> 5);
+      r[n] = *reinterpret_cast<const frag_mem<T>*>(src + slab * 512 + k * 16 + g * 8);
+    }
+  }
+  __device__ __forceinline__ void store(T* dst) const {
+#pragma unroll
+    for (int n = 0; n < 2; ++n) {
+      const int v = threadIdx.x + n * kThreads;
+      const int slab = v >> 6, l = v & 63;
+      const int g = (l >> 4) & 1, k = (l & 15) + 16 * (l >> 5);
+      *reinterpret_cast<frag_mem<T>*>(dst + k * kLdD<T> + 16 * slab + 8 * g) = r[n];
+    }
+  }
+};
+
+template <typename T, typename TI, int HD>
+__global__ __launch_bounds__(kThreads, 1) void bwd_query2_kernel(BwdArgs a) {
+  static_assert(sizeof(T) == 2 && HD <= 64 && kCK == 32, "tile consumer: 16-bit operands, d <= 64");
+  constexpr int KS = HD / 16;
+  constexpr int HDP = HD < 32 ? 32 : HD;
+  constexpr int NT = HDP / 32;
+  constexpr int BT = kNB / 32;
+  constexpr int TS = kNB / 16;   // 16-deep steps across a block
+  constexpr int QB = 128;
+  constexpr int LDK = lds_ld<T>(HD), LDT = lds_ld_chain<T>(kNB), LDA = kLdA<T>, LDD = kLdD<T>;
+
+  Carver cv{castle_smem};
+  T* s_kc = cv.take<T>(kCK * LDK);
+  T* s_qu = cv.take<T>(kCK * LDK);
+  T* s_ub0 = cv.take<T>(kCK * LDK);
+  T* s_ub1 = cv.take<T>(kCK * LDK);
+  T* s_g0 = cv.take<T>(kCK * LDK);
+  T* s_g1 = cv.take<T>(kCK * LDK);
+  T* s_at = cv.take<T>(QB * LDA);    // gate, [source j][key k]
+  T* s_ds = cv.take<T>(kCK * LDD);   // dS,  [key k][query i]
+  T* s_dsu = cv.take<T>(kCK * LDD);  // dSu, [key k][query i]
+
+  int rank, bh;
+  work_item(a.s.B * a.s.H, rank, bh);
+  const int qb = a.s.Lp / 128 - 1 - rank;   // the last row block meets the most keys
+  const int b = bh / a.s.H, h = bh % a.s.H;
+  const int lane = lane_id(), wave = wave_id(), c = lane & 31, g = lane >> 5;
+  const int L = a.s.L;
+  const float c0 = a.s.scale, c1 = a.s.scale * kLog2e;
+  const int i0w = qb * QB + 32 * wave;
+  const int i = i0w + c;                      // this lane's row: a query or a lookahead source
+  const int Ifirst = (qb * QB) / kNB;
+  const int Iw = i0w / kNB;
+  const int qw = Iw - Ifirst;                 // which of the workgroup's blocks
+  const int jw = 32 * wave;                   // rows of this wave inside the 128-row exchange tiles
+  const int cb = (jw / kNB) * kNB;            // first row of its block there
+  const int lw = jw % kNB;                    // offset of the wave inside its block
+  const int ifirst = lw / 16;                 // first step covering queries i >= j
+  const bool has_g = Iw <= a.s.nblk - 2;
+  const T* s_ubw = qw == 0 ? s_ub0 : s_ub1;
+  const T* s_gw = qw == 0 ? s_g0 : s_g1;
+
+  const TI* qc = head_ptr<TI>(a.qc, b, h);
+  const TI* kc = head_ptr<TI>(a.kc, b, h);
+  const TI* qu = head_ptr<TI>(a.qu, b, h);
+  const TI* ku = head_ptr<TI>(a.ku, b, h);
+  const TI* vu = head_ptr<TI>(a.vu, b, h);
+  const T* ttb = reinterpret_cast<const T*>(a.ws.tt_blk) + (int64_t)bh * a.s.Lp * kNB;
+  const T* usnap = reinterpret_cast<const T*>(a.ws.usnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
+  const T* gsnap = reinterpret_cast<const T*>(a.gsnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
+  const int64_t tiles_per_row = a.s.Lp / 32;
+  const T* dsm = reinterpret_cast<const T*>(a.ds_mat) + (int64_t)bh * a.s.Lp * a.s.Lp + (int64_t)qb * 4 * 1024;
+  const T* dsum = reinterpret_cast<const T*>(a.dsu_mat) + (int64_t)bh * a.s.Lp * a.s.Lp + (int64_t)qb * 4 * 1024;
+
+  frag<T> fku[KS], fvu[KS], ftt[TS];
+#pragma unroll
+  for (int s = 0; s < KS; ++s) {
+    fku[s] = ldg_nat_scaled<T, TI>(ku, a.ku.sl, i, 16 * s + 8 * g, i < L, -c1);
+    fvu[s] = ldg_nat<T, TI>(vu, a.vu.sl, i, 16 * s + 8 * g, i < L);
+  }
+#pragma unroll
+  for (int s = 0; s < TS; ++s) ftt[s] = ldg_nat<T>(ttb, kNB, i, 16 * s + 8 * g, s >= ifirst);
+
+  acc_t dqc[NT], dku[NT], dvu[NT];   // [n rows, row-of-this-lane]
+  acc_t dtacc[BT];                   // [j rows (block local), i lanes]
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) { zero(dqc[nt]); zero(dku[nt]); zero(dvu[nt]); }
+#pragma unroll
+  for (int jt = 0; jt < BT; ++jt) zero(dtacc[jt]);
+
+  RowStage<T, TI, kCK, HD> pkc, pqu;
+  SnapStage<T, kCK, HD> pu0, pu1, pg0, pg1;
+  TileStage<T> pds, pdsu;
+  const int blk0 = Ifirst, blk1 = Ifirst + 1;
+#define CASTLE_BQ2_LOAD(K0)                                                                          \
+  do {                                                                                               \
+    const int kb_ = (K0) / kNB;                                                                      \
+    pkc.load(kc, a.kc.sl, (K0), L);                                                                  \
+    pqu.load(qu, a.qu.sl, (K0), L);                                                                  \
+    if (kb_ < blk0) pu0.load(usnap + (usnap_off(blk0) + (K0)) * HD);                                 \
+    if (kb_ < blk1 && blk1 < a.s.nblk) pu1.load(usnap + (usnap_off(blk1) + (K0)) * HD);              \
+    if (kb_ <= blk0 && blk0 <= a.s.nblk - 2) pg0.load(gsnap + (gsnap_off(blk0) + (K0)) * HD);        \
+    if (kb_ <= blk1 && blk1 <= a.s.nblk - 2) pg1.load(gsnap + (gsnap_off(blk1) + (K0)) * HD);        \
+    pds.load(dsm + (int64_t)((K0) / 32) * tiles_per_row * 1024);                                     \
+    pdsu.load(dsum + (int64_t)((K0) / 32) * tiles_per_row * 1024);                                   \
+  } while (0)
+
+  int kend = qb * QB + QB;
+  if (kend > a.s.Lp) kend = a.s.Lp;
+  CASTLE_BQ2_LOAD(0);
+  for (int k0 = 0; k0 < kend; k0 += kCK) {
+    const int Kb = k0 / kNB;
+    __syncthreads();
+    pkc.store(s_kc, LDK);
+    pqu.store(s_qu, LDK);
+    if (Kb < blk0) pu0.store(s_ub0, LDK);
+    if (Kb < blk1 && blk1 < a.s.nblk) pu1.store(s_ub1, LDK);
+    if (Kb <= blk0 && blk0 <= a.s.nblk - 2) pg0.store(s_g0, LDK);
+    if (Kb <= blk1 && blk1 <= a.s.nblk - 2) pg1.store(s_g1, LDK);
+    pds.store(s_ds);
+    pdsu.store(s_dsu);
+    if (k0 + kCK < kend) CASTLE_BQ2_LOAD(k0 + kCK);   // in flight while this chunk is processed
+    __syncthreads();
+    const bool live = k0 <= i0w;   // the chunk's keys do not lie beyond this wave's rows
+
+    // gate tile A[k rows, j lanes] for this wave's 32 source rows, shared as A^T[j][k]
+    acc_t aK;
+    zero(aK);
+    if (live) {
+      {
+        frag<T> oqu[KS];
+#pragma unroll
+        for (int s = 0; s < KS; ++s) oqu[s] = ld_nat<T>(s_qu, LDK, c, 16 * s + 8 * g);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < KS; ++s) mma(aK, oqu[s], fku[s]);
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) aK[r] = fast_rcp(1.f + fast_exp2(aK[r]));
+      if (k0 + 31 >= i0w) {   // the tile reaches the diagonal: keep j > k only
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if (i <= k0 + acc_row(r, g)) aK[r] = 0.f;
+      }
+    }
+    if (Kb <= Iw) {   // a wave the chunk has passed still owes zeros to the other wave of its block
+#pragma unroll
+      for (int q = 0; q < 4; ++q) st4<T>(s_at + (jw + c) * LDA + 8 * q + 4 * g, pack4<T>(aK, q));
+    }
+    __syncthreads();
+    if (!live) continue;
+
+    {   // row = query
+      frag<T> bds[2], bdsu[2], okt[2][NT], out[2][NT], oat[2][BT];
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        bds[s2] = ld_free<T, false>(s_ds, LDD, jw, 1 << 30, 16 * s2, c, g);
+        bdsu[s2] = ld_free<T, false>(s_dsu, LDD, jw, 1 << 30, 16 * s2, c, g);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          okt[s2][nt] = ld_free<T, false>(s_kc, LDK, 32 * nt, HD, 16 * s2, c, g);
+          out[s2][nt] = ld_free<T, false>(s_ubw, LDK, 32 * nt, HD, 16 * s2, c, g);
+        }
+#pragma unroll
+        for (int jt = 0; jt < BT; ++jt) oat[s2][jt] = ld_nat<T>(s_at, LDA, cb + 32 * jt + c, 16 * s2 + 8 * g);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          mma(dqc[nt], okt[s2][nt], bds[s2]);
+          if (Kb < Iw) mma(dqc[nt], out[s2][nt], bdsu[s2]);
+        }
+#pragma unroll
+        for (int jt = 0; jt < BT; ++jt)
+          if (32 * jt < lw + 32) mma(dtacc[jt], oat[s2][jt], bdsu[s2]);
+      }
+    }
+    {   // row = lookahead source
+      acc_t dA;
+      zero(dA);
+      frag<T> oqt[2][NT], ogt[2][NT];
+      {
+        frag<T> ods[TS], og[KS];
+#pragma unroll
+        for (int s = 0; s < TS; ++s) ods[s] = ld_nat<T>(s_dsu, LDD, c, cb + 16 * s + 8 * g);
+#pragma unroll
+        for (int s = 0; s < KS; ++s) og[s] = ld_nat<T>(s_gw, LDK, c, 16 * s + 8 * g);
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) {
+            oqt[s2][nt] = ld_free<T, true>(s_qu, LDK, 32 * nt, HD, 16 * s2, c, g);
+            ogt[s2][nt] = ld_free<T, true>(s_gw, LDK, 32 * nt, HD, 16 * s2, c, g);
+          }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < TS; ++s)
+          if (s >= ifirst) mma(dA, ods[s], ftt[s]);
+        if (has_g) {
+#pragma unroll
+          for (int s = 0; s < KS; ++s) mma(dA, og[s], fvu[s]);
+        }
+      }
+      acc_t dz;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dz[r] = dA[r] * aK[r] * (1.f - aK[r]);
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        const frag<T> fdz = chain<T>(dz, s2), fa = chain<T>(aK, s2);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          mma(dku[nt], oqt[s2][nt], fdz);
+          if (has_g) mma(dvu[nt], ogt[s2][nt], fa);
+        }
+      }
+    }
+  }
+#undef CASTLE_BQ2_LOAD
+
+  // ---- epilogue: in-block terms dT = tril(dTacc):  dqc += dT Vu,  dvu += dT^T Qc' ------------
+  __syncthreads();
+  Carver ce{castle_smem};
+  T* e_vu0 = ce.take<T>(kNB * LDK);
+  T* e_vu1 = ce.take<T>(kNB * LDK);
+  T* e_qc0 = ce.take<T>(kNB * LDK);
+  T* e_qc1 = ce.take<T>(kNB * LDK);
+  T* e_dt0 = ce.take<T>(kNB * LDT);   // dT, [query i][source j] (block local)
+  T* e_dt1 = ce.take<T>(kNB * LDT);
+  {
+    RowStage<T, TI, kNB, HD> st;
+    st.load(vu, a.vu.sl, (int64_t)blk0 * kNB, L); st.store(e_vu0, LDK);
+    st.load(vu, a.vu.sl, (int64_t)blk1 * kNB, L); st.store(e_vu1, LDK);
+    st.load(qc, a.qc.sl, (int64_t)blk0 * kNB, L); st.store_scaled(e_qc0, LDK, c1);
+    st.load(qc, a.qc.sl, (int64_t)blk1 * kNB, L); st.store_scaled(e_qc1, LDK, c1);
+  }
+  const T* e_vuw = qw == 0 ? e_vu0 : e_vu1;
+  const T* e_qcw = qw == 0 ? e_qc0 : e_qc1;
+  T* e_dtw = qw == 0 ? e_dt0 : e_dt1;
+  // dT^T[j rows, i lanes] masked to j <= i, shared as dT[i][j] for the source-side product
+#pragma unroll
+  for (int jt = 0; jt < BT; ++jt) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+      if (32 * jt + acc_row(r, g) > lw + c) dtacc[jt][r] = 0.f;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) st4<T>(e_dtw + (lw + c) * LDT + 32 * jt + 8 * q + 4 * g, pack4<T>(dtacc[jt], q));
+  }
+  __syncthreads();
+#pragma unroll
+  for (int jt = 0; jt < BT; ++jt) {
+    if (32 * jt >= lw + 32) continue;
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) {
+      const frag<T> fdt = chain<T>(dtacc[jt], s2);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+        mma(dqc[nt], ld_free<T, true>(e_vuw, LDK, 32 * nt, HD, 32 * jt + 16 * s2, c, g), fdt);
+    }
+  }
+#pragma unroll
+  for (int s = 0; s < TS; ++s) {
+    if (s < ifirst) continue;
+    // B operand: source j = lw + c on lanes, queries i = 16 s .. in natural order, from dT[i][j]
+    const frag<T> fdt = ld_free<T, false>(e_dtw, LDT, lw, kNB, 16 * s, c, g);
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+      mma(dvu[nt], ld_free<T, false>(e_qcw, LDK, 32 * nt, HD, 16 * s, c, g), fdt);
+  }
+  if (i < L) {
+    store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqc, b, h) + (int64_t)i * a.dqc.sl, dqc, c0, g);
+    store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dku, b, h) + (int64_t)i * a.dku.sl, dku, c0 * kLn2, g);
+    store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvu, b, h) + (int64_t)i * a.dvu.sl, dvu, kLn2, g);
+  }
+}
+
+// ---------------------------------------------------------------------------
 template <typename T, typename TI, int HD, int PART> static int launch_bwd_part(const BwdArgs& a, hipStream_t stream) {
   const int BH = a.s.B * a.s.H;
   constexpr int key_lds = bwd_key_lds_bytes<T, HD>(), query_lds = bwd_query_lds_bytes<T, HD>();
@@ -1036,6 +1341,7 @@ template <typename T, typename TI, int HD> static int launch_bwd_t(const BwdArgs
     static bool configured2 = false;
     if (!configured2) {
       if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_key2_kernel<T, TI, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_key2_lds_bytes<T, HD>()) != hipSuccess) return -3;
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_query2_kernel<T, TI, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_query2_lds_bytes<T, HD>()) != hipSuccess) return -3;
       configured2 = true;
     }
   }
@@ -1070,6 +1376,9 @@ template <typename T, typename TI, int HD> static int launch_bwd_t(const BwdArgs
     if constexpr (SPLIT) {
       hipLaunchKernelGGL((bwd_query_kernel<T, TI, HD, 1>), grid, block, query_lds, stream, a);
       hipLaunchKernelGGL((bwd_query_kernel<T, TI, HD, 2>), grid, block, query_lds, stream, a);
+    } else if constexpr (TWO_ROLE) {
+      constexpr int query2_lds = bwd_query2_lds_bytes<T, HD>();
+      hipLaunchKernelGGL((bwd_query2_kernel<T, TI, HD>), grid, block, query2_lds, stream, a);
     } else {
       hipLaunchKernelGGL((bwd_query_kernel<T, TI, HD, 0>), grid, block, query_lds, stream, a);
     }

@@ -40,6 +40,12 @@ struct BwdArgs {
   FwdWorkspace ws;
   void* gsnap;    // [B*H][snap_rows(nblk)][d]  reverse state at block ends
   float* delta;   // [B*H][Lp]  rowsum(dO * O)
+  // Score-gradient tiles handed from the key-stationary to the query-stationary kernel (16-bit
+  // operands, d <= 64 only, else nullptr): per head (Lp/32)^2 tiles of 32 keys x 32 queries,
+  // tile (kt, it) at ((kt * (Lp/32) + it) * 1024 elements; only tiles with kt <= it are written.
+  // Inside a tile, element (key k, query i) sits at (i / 16) * 512 + k * 16 + i % 16.
+  void* ds_mat;   // dS
+  void* dsu_mat;  // dSu
 };
 
 struct DecodeArgs {
