@@ -1036,33 +1036,29 @@ template <typename T, int HD> constexpr int bwd_query2_lds_bytes() {
 }
 
 // Staging of the 4 consecutive 32x32 tiles (8 KB) that one chunk of 32 keys shares with the 128
-// queries of a workgroup.  Every wave instruction reads 1 KB contiguous; within 16 lanes the LDS
-// rows differ, which keeps the 16-byte stores conflict free.
+// queries of a workgroup, one 16-byte piece per thread (512 threads).  Every wave instruction
+// reads 1 KB contiguous; within 16 lanes the LDS rows differ, which keeps the stores conflict free.
 template <typename T>
 struct TileStage {
-  vec<T, 8> r[2];
+  vec<T, 8> r;
   __device__ __forceinline__ void load(const T* src) {
-#pragma unroll
-    for (int n = 0; n < 2; ++n) {
-      const int v = threadIdx.x + n * kThreads;
-      const int slab = v >> 6, l = v & 63;                       // slab = 2 * tile + s2
-      const int g = (l >> 4) & 1, k = (l & 15) + 16 * (l >> 5);
-      r[n] = *reinterpret_cast<const frag_mem<T>*>(src + slab * 512 + k * 16 + g * 8);
-    }
+    const int slab = threadIdx.x >> 6, l = threadIdx.x & 63;       // slab = 2 * tile + s2
+    const int g = (l >> 4) & 1, k = (l & 15) + 16 * (l >> 5);
+    r = *reinterpret_cast<const frag_mem<T>*>(src + slab * 512 + k * 16 + g * 8);
   }
   __device__ __forceinline__ void store(T* dst) const {
-#pragma unroll
-    for (int n = 0; n < 2; ++n) {
-      const int v = threadIdx.x + n * kThreads;
-      const int slab = v >> 6, l = v & 63;
-      const int g = (l >> 4) & 1, k = (l & 15) + 16 * (l >> 5);
-      *reinterpret_cast<frag_mem<T>*>(dst + k * kLdD<T> + 16 * slab + 8 * g) = r[n];
-    }
+    const int slab = threadIdx.x >> 6, l = threadIdx.x & 63;
+    const int g = (l >> 4) & 1, k = (l & 15) + 16 * (l >> 5);
+    *reinterpret_cast<frag_mem<T>*>(dst + k * kLdD<T> + 16 * slab + 8 * g) = r;
   }
 };
 
+// 512 threads, two wave roles over the same 128 rows (wave pair (w, w + 4) owns rows 32 w ..):
+//   waves 0-3, row = lookahead source j:  gate A, dA, dZ, dKu, dVu
+//   waves 4-7, row = query i:             dQc, dT
+// Keys are streamed in chunks of 32 (three barriers per chunk); two waves share a SIMD.
 template <typename T, typename TI, int HD>
-__global__ __launch_bounds__(kThreads, 1) void bwd_query2_kernel(BwdArgs a) {
+__global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) {
   static_assert(sizeof(T) == 2 && HD <= 64 && kCK == 32, "tile consumer: 16-bit operands, d <= 64");
   constexpr int KS = HD / 16;
   constexpr int HDP = HD < 32 ? 32 : HD;
@@ -1082,145 +1078,119 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query2_kernel(BwdArgs a) {
   T* s_at = cv.take<T>(QB * LDA);    // gate, [source j][key k]
   T* s_ds = cv.take<T>(kCK * LDD);   // dS,  [key k][query i]
   T* s_dsu = cv.take<T>(kCK * LDD);  // dSu, [key k][query i]
+  // the epilogue reuses the same memory
+  Carver ce{castle_smem};
+  T* e_vu0 = ce.take<T>(kNB * LDK);
+  T* e_vu1 = ce.take<T>(kNB * LDK);
+  T* e_qc0 = ce.take<T>(kNB * LDK);
+  T* e_qc1 = ce.take<T>(kNB * LDK);
+  T* e_dt0 = ce.take<T>(kNB * LDT);   // dT, [query i][source j] (block local)
+  T* e_dt1 = ce.take<T>(kNB * LDT);
 
   int rank, bh;
   work_item(a.s.B * a.s.H, rank, bh);
   const int qb = a.s.Lp / 128 - 1 - rank;   // the last row block meets the most keys
   const int b = bh / a.s.H, h = bh % a.s.H;
   const int lane = lane_id(), wave = wave_id(), c = lane & 31, g = lane >> 5;
+  const bool source_role = wave < 4;
+  const int pw = wave & 3;
+  const int tid = threadIdx.x & (kThreads - 1);   // thread index inside the role
   const int L = a.s.L;
   const float c0 = a.s.scale, c1 = a.s.scale * kLog2e;
-  const int i0w = qb * QB + 32 * wave;
-  const int i = i0w + c;                      // this lane's row: a query or a lookahead source
+  const int i0w = qb * QB + 32 * pw;
+  const int i = i0w + c;                      // this lane's row
   const int Ifirst = (qb * QB) / kNB;
   const int Iw = i0w / kNB;
   const int qw = Iw - Ifirst;                 // which of the workgroup's blocks
-  const int jw = 32 * wave;                   // rows of this wave inside the 128-row exchange tiles
+  const int jw = 32 * pw;                     // rows of this wave pair inside the 128-row exchange tiles
   const int cb = (jw / kNB) * kNB;            // first row of its block there
-  const int lw = jw % kNB;                    // offset of the wave inside its block
+  const int lw = jw % kNB;                    // offset of the wave pair inside its block
   const int ifirst = lw / 16;                 // first step covering queries i >= j
   const bool has_g = Iw <= a.s.nblk - 2;
   const T* s_ubw = qw == 0 ? s_ub0 : s_ub1;
   const T* s_gw = qw == 0 ? s_g0 : s_g1;
+  const T* e_vuw = qw == 0 ? e_vu0 : e_vu1;
+  const T* e_qcw = qw == 0 ? e_qc0 : e_qc1;
+  T* e_dtw = qw == 0 ? e_dt0 : e_dt1;
+  const int blk0 = Ifirst, blk1 = Ifirst + 1;
 
   const TI* qc = head_ptr<TI>(a.qc, b, h);
-  const TI* kc = head_ptr<TI>(a.kc, b, h);
-  const TI* qu = head_ptr<TI>(a.qu, b, h);
-  const TI* ku = head_ptr<TI>(a.ku, b, h);
   const TI* vu = head_ptr<TI>(a.vu, b, h);
-  const T* ttb = reinterpret_cast<const T*>(a.ws.tt_blk) + (int64_t)bh * a.s.Lp * kNB;
   const T* usnap = reinterpret_cast<const T*>(a.ws.usnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
   const T* gsnap = reinterpret_cast<const T*>(a.gsnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
-  const int64_t tiles_per_row = a.s.Lp / 32;
+  const int64_t tile_row = (int64_t)(a.s.Lp / 32) * 1024;   // elements between the tiles of consecutive key groups
   const T* dsm = reinterpret_cast<const T*>(a.ds_mat) + (int64_t)bh * a.s.Lp * a.s.Lp + (int64_t)qb * 4 * 1024;
   const T* dsum = reinterpret_cast<const T*>(a.dsu_mat) + (int64_t)bh * a.s.Lp * a.s.Lp + (int64_t)qb * 4 * 1024;
-
-  frag<T> fku[KS], fvu[KS], ftt[TS];
-#pragma unroll
-  for (int s = 0; s < KS; ++s) {
-    fku[s] = ldg_nat_scaled<T, TI>(ku, a.ku.sl, i, 16 * s + 8 * g, i < L, -c1);
-    fvu[s] = ldg_nat<T, TI>(vu, a.vu.sl, i, 16 * s + 8 * g, i < L);
-  }
-#pragma unroll
-  for (int s = 0; s < TS; ++s) ftt[s] = ldg_nat<T>(ttb, kNB, i, 16 * s + 8 * g, s >= ifirst);
-
-  acc_t dqc[NT], dku[NT], dvu[NT];   // [n rows, row-of-this-lane]
-  acc_t dtacc[BT];                   // [j rows (block local), i lanes]
-#pragma unroll
-  for (int nt = 0; nt < NT; ++nt) { zero(dqc[nt]); zero(dku[nt]); zero(dvu[nt]); }
-#pragma unroll
-  for (int jt = 0; jt < BT; ++jt) zero(dtacc[jt]);
-
-  RowStage<T, TI, kCK, HD> pkc, pqu;
-  SnapStage<T, kCK, HD> pu0, pu1, pg0, pg1;
-  TileStage<T> pds, pdsu;
-  const int blk0 = Ifirst, blk1 = Ifirst + 1;
-#define CASTLE_BQ2_LOAD(K0)                                                                          \
-  do {                                                                                               \
-    const int kb_ = (K0) / kNB;                                                                      \
-    pkc.load(kc, a.kc.sl, (K0), L);                                                                  \
-    pqu.load(qu, a.qu.sl, (K0), L);                                                                  \
-    if (kb_ < blk0) pu0.load(usnap + (usnap_off(blk0) + (K0)) * HD);                                 \
-    if (kb_ < blk1 && blk1 < a.s.nblk) pu1.load(usnap + (usnap_off(blk1) + (K0)) * HD);              \
-    if (kb_ <= blk0 && blk0 <= a.s.nblk - 2) pg0.load(gsnap + (gsnap_off(blk0) + (K0)) * HD);        \
-    if (kb_ <= blk1 && blk1 <= a.s.nblk - 2) pg1.load(gsnap + (gsnap_off(blk1) + (K0)) * HD);        \
-    pds.load(dsm + (int64_t)((K0) / 32) * tiles_per_row * 1024);                                     \
-    pdsu.load(dsum + (int64_t)((K0) / 32) * tiles_per_row * 1024);                                   \
-  } while (0)
-
   int kend = qb * QB + QB;
   if (kend > a.s.Lp) kend = a.s.Lp;
-  CASTLE_BQ2_LOAD(0);
-  for (int k0 = 0; k0 < kend; k0 += kCK) {
-    const int Kb = k0 / kNB;
-    __syncthreads();
-    pkc.store(s_kc, LDK);
-    pqu.store(s_qu, LDK);
-    if (Kb < blk0) pu0.store(s_ub0, LDK);
-    if (Kb < blk1 && blk1 < a.s.nblk) pu1.store(s_ub1, LDK);
-    if (Kb <= blk0 && blk0 <= a.s.nblk - 2) pg0.store(s_g0, LDK);
-    if (Kb <= blk1 && blk1 <= a.s.nblk - 2) pg1.store(s_g1, LDK);
-    pds.store(s_ds);
-    pdsu.store(s_dsu);
-    if (k0 + kCK < kend) CASTLE_BQ2_LOAD(k0 + kCK);   // in flight while this chunk is processed
-    __syncthreads();
-    const bool live = k0 <= i0w;   // the chunk's keys do not lie beyond this wave's rows
+  TileStage<T> pds, pdsu;   // every thread: one piece of each
 
-    // gate tile A[k rows, j lanes] for this wave's 32 source rows, shared as A^T[j][k]
-    acc_t aK;
-    zero(aK);
-    if (live) {
-      {
-        frag<T> oqu[KS];
+  if (source_role) {
+    const TI* kc = head_ptr<TI>(a.kc, b, h);
+    const TI* qu = head_ptr<TI>(a.qu, b, h);
+    const TI* ku = head_ptr<TI>(a.ku, b, h);
+    const T* ttb = reinterpret_cast<const T*>(a.ws.tt_blk) + (int64_t)bh * a.s.Lp * kNB;
+    frag<T> fku[KS], fvu[KS], ftt[TS];
 #pragma unroll
-        for (int s = 0; s < KS; ++s) oqu[s] = ld_nat<T>(s_qu, LDK, c, 16 * s + 8 * g);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int s = 0; s < KS; ++s) mma(aK, oqu[s], fku[s]);
-      }
-#pragma unroll
-      for (int r = 0; r < 16; ++r) aK[r] = fast_rcp(1.f + fast_exp2(aK[r]));
-      if (k0 + 31 >= i0w) {   // the tile reaches the diagonal: keep j > k only
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-          if (i <= k0 + acc_row(r, g)) aK[r] = 0.f;
-      }
+    for (int s = 0; s < KS; ++s) {
+      fku[s] = ldg_nat_scaled<T, TI>(ku, a.ku.sl, i, 16 * s + 8 * g, i < L, -c1);
+      fvu[s] = ldg_nat<T, TI>(vu, a.vu.sl, i, 16 * s + 8 * g, i < L);
     }
-    if (Kb <= Iw) {   // a wave the chunk has passed still owes zeros to the other wave of its block
 #pragma unroll
-      for (int q = 0; q < 4; ++q) st4<T>(s_at + (jw + c) * LDA + 8 * q + 4 * g, pack4<T>(aK, q));
-    }
-    __syncthreads();
-    if (!live) continue;
+    for (int s = 0; s < TS; ++s) ftt[s] = ldg_nat<T>(ttb, kNB, i, 16 * s + 8 * g, s >= ifirst);
+    acc_t dku[NT], dvu[NT];   // [n rows, j lanes]
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) { zero(dku[nt]); zero(dvu[nt]); }
 
-    {   // row = query
-      frag<T> bds[2], bdsu[2], okt[2][NT], out[2][NT], oat[2][BT];
+    // this role stages kc, qu and the lookahead state of the first block
+    RowStage<T, TI, kCK, HD> pkc, pqu;
+    SnapStage<T, kCK, HD> pu0;
+#define CASTLE_BQ2_LOAD_A(K0)                                                            \
+  do {                                                                                   \
+    pkc.load(kc, a.kc.sl, (K0), L, tid);                                                 \
+    pqu.load(qu, a.qu.sl, (K0), L, tid);                                                 \
+    if ((K0) / kNB < blk0) pu0.load(usnap + (usnap_off(blk0) + (K0)) * HD, tid);         \
+    pds.load(dsm + (int64_t)((K0) / 32) * tile_row);                                     \
+    pdsu.load(dsum + (int64_t)((K0) / 32) * tile_row);                                   \
+  } while (0)
+    CASTLE_BQ2_LOAD_A(0);
+    for (int k0 = 0; k0 < kend; k0 += kCK) {
+      const int Kb = k0 / kNB;
+      __syncthreads();   // 1: tiles free
+      pkc.store(s_kc, LDK, tid);
+      pqu.store(s_qu, LDK, tid);
+      if (Kb < blk0) pu0.store(s_ub0, LDK, tid);
+      pds.store(s_ds);
+      pdsu.store(s_dsu);
+      if (k0 + kCK < kend) CASTLE_BQ2_LOAD_A(k0 + kCK);   // in flight while this chunk is processed
+      __syncthreads();   // 2: tiles staged
+      const bool live = k0 <= i0w;   // the chunk's keys do not lie beyond this wave's rows
+      // gate tile A[k rows, j lanes] for this wave's 32 source rows, shared as A^T[j][k]
+      acc_t aK;
+      zero(aK);
+      if (live) {
+        {
+          frag<T> oqu[KS];
 #pragma unroll
-      for (int s2 = 0; s2 < 2; ++s2) {
-        bds[s2] = ld_free<T, false>(s_ds, LDD, jw, 1 << 30, 16 * s2, c, g);
-        bdsu[s2] = ld_free<T, false>(s_dsu, LDD, jw, 1 << 30, 16 * s2, c, g);
+          for (int s = 0; s < KS; ++s) oqu[s] = ld_nat<T>(s_qu, LDK, c, 16 * s + 8 * g);
+          __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-          okt[s2][nt] = ld_free<T, false>(s_kc, LDK, 32 * nt, HD, 16 * s2, c, g);
-          out[s2][nt] = ld_free<T, false>(s_ubw, LDK, 32 * nt, HD, 16 * s2, c, g);
+          for (int s = 0; s < KS; ++s) mma(aK, oqu[s], fku[s]);
         }
 #pragma unroll
-        for (int jt = 0; jt < BT; ++jt) oat[s2][jt] = ld_nat<T>(s_at, LDA, cb + 32 * jt + c, 16 * s2 + 8 * g);
-      }
-      __builtin_amdgcn_sched_barrier(0);
+        for (int r = 0; r < 16; ++r) aK[r] = fast_rcp(1.f + fast_exp2(aK[r]));
+        if (k0 + 31 >= i0w) {   // the tile reaches the diagonal: keep j > k only
 #pragma unroll
-      for (int s2 = 0; s2 < 2; ++s2) {
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-          mma(dqc[nt], okt[s2][nt], bds[s2]);
-          if (Kb < Iw) mma(dqc[nt], out[s2][nt], bdsu[s2]);
+          for (int r = 0; r < 16; ++r)
+            if (i <= k0 + acc_row(r, g)) aK[r] = 0.f;
         }
-#pragma unroll
-        for (int jt = 0; jt < BT; ++jt)
-          if (32 * jt < lw + 32) mma(dtacc[jt], oat[s2][jt], bdsu[s2]);
       }
-    }
-    {   // row = lookahead source
+      if (Kb <= Iw) {   // a wave the chunk has passed still owes zeros to the other rows of its block
+#pragma unroll
+        for (int q = 0; q < 4; ++q) st4<T>(s_at + (jw + c) * LDA + 8 * q + 4 * g, pack4<T>(aK, q));
+      }
+      __syncthreads();   // 3: gate shared
+      if (!live) continue;
       acc_t dA;
       zero(dA);
       frag<T> oqt[2][NT], ogt[2][NT];
@@ -1259,62 +1229,130 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query2_kernel(BwdArgs a) {
         }
       }
     }
-  }
-#undef CASTLE_BQ2_LOAD
-
-  // ---- epilogue: in-block terms dT = tril(dTacc):  dqc += dT Vu,  dvu += dT^T Qc' ------------
-  __syncthreads();
-  Carver ce{castle_smem};
-  T* e_vu0 = ce.take<T>(kNB * LDK);
-  T* e_vu1 = ce.take<T>(kNB * LDK);
-  T* e_qc0 = ce.take<T>(kNB * LDK);
-  T* e_qc1 = ce.take<T>(kNB * LDK);
-  T* e_dt0 = ce.take<T>(kNB * LDT);   // dT, [query i][source j] (block local)
-  T* e_dt1 = ce.take<T>(kNB * LDT);
-  {
-    RowStage<T, TI, kNB, HD> st;
-    st.load(vu, a.vu.sl, (int64_t)blk0 * kNB, L); st.store(e_vu0, LDK);
-    st.load(vu, a.vu.sl, (int64_t)blk1 * kNB, L); st.store(e_vu1, LDK);
-    st.load(qc, a.qc.sl, (int64_t)blk0 * kNB, L); st.store_scaled(e_qc0, LDK, c1);
-    st.load(qc, a.qc.sl, (int64_t)blk1 * kNB, L); st.store_scaled(e_qc1, LDK, c1);
-  }
-  const T* e_vuw = qw == 0 ? e_vu0 : e_vu1;
-  const T* e_qcw = qw == 0 ? e_qc0 : e_qc1;
-  T* e_dtw = qw == 0 ? e_dt0 : e_dt1;
-  // dT^T[j rows, i lanes] masked to j <= i, shared as dT[i][j] for the source-side product
+#undef CASTLE_BQ2_LOAD_A
+    // ---- epilogue: in-block term dvu += dT^T Qc' --------------------------------------------
+    __syncthreads();   // e1: chunk tiles dead
+    {
+      RowStage<T, TI, kNB, HD, 2 * kThreads> st;
+      st.load(vu, a.vu.sl, (int64_t)blk0 * kNB, L); st.store(e_vu0, LDK);
+      st.load(vu, a.vu.sl, (int64_t)blk1 * kNB, L); st.store(e_vu1, LDK);
+      st.load(qc, a.qc.sl, (int64_t)blk0 * kNB, L); st.store_scaled(e_qc0, LDK, c1);
+      st.load(qc, a.qc.sl, (int64_t)blk1 * kNB, L); st.store_scaled(e_qc1, LDK, c1);
+    }
+    __syncthreads();   // e2: epilogue tiles and dT shared
 #pragma unroll
-  for (int jt = 0; jt < BT; ++jt) {
-#pragma unroll
-    for (int r = 0; r < 16; ++r)
-      if (32 * jt + acc_row(r, g) > lw + c) dtacc[jt][r] = 0.f;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) st4<T>(e_dtw + (lw + c) * LDT + 32 * jt + 8 * q + 4 * g, pack4<T>(dtacc[jt], q));
-  }
-  __syncthreads();
-#pragma unroll
-  for (int jt = 0; jt < BT; ++jt) {
-    if (32 * jt >= lw + 32) continue;
-#pragma unroll
-    for (int s2 = 0; s2 < 2; ++s2) {
-      const frag<T> fdt = chain<T>(dtacc[jt], s2);
+    for (int s = 0; s < TS; ++s) {
+      if (s < ifirst) continue;
+      // B operand: source j = lw + c on lanes, queries i = 16 s .. in natural order, from dT[i][j]
+      const frag<T> fdt = ld_free<T, false>(e_dtw, LDT, lw, kNB, 16 * s, c, g);
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt)
-        mma(dqc[nt], ld_free<T, true>(e_vuw, LDK, 32 * nt, HD, 32 * jt + 16 * s2, c, g), fdt);
+        mma(dvu[nt], ld_free<T, false>(e_qcw, LDK, 32 * nt, HD, 16 * s, c, g), fdt);
     }
-  }
+    if (i < L) {
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dku, b, h) + (int64_t)i * a.dku.sl, dku, c0 * kLn2, g);
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvu, b, h) + (int64_t)i * a.dvu.sl, dvu, kLn2, g);
+    }
+  } else {
+    acc_t dqc[NT];     // [n rows, i lanes]
+    acc_t dtacc[BT];   // [j rows (block local), i lanes]
 #pragma unroll
-  for (int s = 0; s < TS; ++s) {
-    if (s < ifirst) continue;
-    // B operand: source j = lw + c on lanes, queries i = 16 s .. in natural order, from dT[i][j]
-    const frag<T> fdt = ld_free<T, false>(e_dtw, LDT, lw, kNB, 16 * s, c, g);
+    for (int nt = 0; nt < NT; ++nt) zero(dqc[nt]);
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
-      mma(dvu[nt], ld_free<T, false>(e_qcw, LDK, 32 * nt, HD, 16 * s, c, g), fdt);
-  }
-  if (i < L) {
-    store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqc, b, h) + (int64_t)i * a.dqc.sl, dqc, c0, g);
-    store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dku, b, h) + (int64_t)i * a.dku.sl, dku, c0 * kLn2, g);
-    store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvu, b, h) + (int64_t)i * a.dvu.sl, dvu, kLn2, g);
+    for (int jt = 0; jt < BT; ++jt) zero(dtacc[jt]);
+    // this role stages the lookahead state of the second block and both reverse states
+    SnapStage<T, kCK, HD> pu1, pg0, pg1;
+#define CASTLE_BQ2_LOAD_B(K0)                                                                             \
+  do {                                                                                                    \
+    const int kb_ = (K0) / kNB;                                                                           \
+    if (kb_ < blk1 && blk1 < a.s.nblk) pu1.load(usnap + (usnap_off(blk1) + (K0)) * HD, tid);              \
+    if (kb_ <= blk0 && blk0 <= a.s.nblk - 2) pg0.load(gsnap + (gsnap_off(blk0) + (K0)) * HD, tid);        \
+    if (kb_ <= blk1 && blk1 <= a.s.nblk - 2) pg1.load(gsnap + (gsnap_off(blk1) + (K0)) * HD, tid);        \
+    pds.load(dsm + (int64_t)((K0) / 32) * tile_row);                                                      \
+    pdsu.load(dsum + (int64_t)((K0) / 32) * tile_row);                                                    \
+  } while (0)
+    CASTLE_BQ2_LOAD_B(0);
+    for (int k0 = 0; k0 < kend; k0 += kCK) {
+      const int Kb = k0 / kNB;
+      __syncthreads();   // 1
+      if (Kb < blk1 && blk1 < a.s.nblk) pu1.store(s_ub1, LDK, tid);
+      if (Kb <= blk0 && blk0 <= a.s.nblk - 2) pg0.store(s_g0, LDK, tid);
+      if (Kb <= blk1 && blk1 <= a.s.nblk - 2) pg1.store(s_g1, LDK, tid);
+      pds.store(s_ds);
+      pdsu.store(s_dsu);
+      if (k0 + kCK < kend) CASTLE_BQ2_LOAD_B(k0 + kCK);
+      __syncthreads();   // 2
+      const bool live = k0 <= i0w;
+      frag<T> bdsu[2];
+      if (live) {
+        frag<T> bds[2], okt[2][NT], out[2][NT];
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+          bds[s2] = ld_free<T, false>(s_ds, LDD, jw, 1 << 30, 16 * s2, c, g);
+          bdsu[s2] = ld_free<T, false>(s_dsu, LDD, jw, 1 << 30, 16 * s2, c, g);
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) {
+            okt[s2][nt] = ld_free<T, false>(s_kc, LDK, 32 * nt, HD, 16 * s2, c, g);
+            out[s2][nt] = ld_free<T, false>(s_ubw, LDK, 32 * nt, HD, 16 * s2, c, g);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) {
+            mma(dqc[nt], okt[s2][nt], bds[s2]);
+            if (Kb < Iw) mma(dqc[nt], out[s2][nt], bdsu[s2]);
+          }
+      }
+      __syncthreads();   // 3
+      if (!live) continue;
+      {
+        frag<T> oat[2][BT];
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+          for (int jt = 0; jt < BT; ++jt) oat[s2][jt] = ld_nat<T>(s_at, LDA, cb + 32 * jt + c, 16 * s2 + 8 * g);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+          for (int jt = 0; jt < BT; ++jt)
+            if (32 * jt < lw + 32) mma(dtacc[jt], oat[s2][jt], bdsu[s2]);
+      }
+    }
+#undef CASTLE_BQ2_LOAD_B
+    // ---- epilogue: dT = tril(dTacc):  dqc += dT Vu -------------------------------------------
+    __syncthreads();   // e1
+    {
+      RowStage<T, TI, kNB, HD, 2 * kThreads> st;
+      st.load(vu, a.vu.sl, (int64_t)blk0 * kNB, L); st.store(e_vu0, LDK);
+      st.load(vu, a.vu.sl, (int64_t)blk1 * kNB, L); st.store(e_vu1, LDK);
+      st.load(qc, a.qc.sl, (int64_t)blk0 * kNB, L); st.store_scaled(e_qc0, LDK, c1);
+      st.load(qc, a.qc.sl, (int64_t)blk1 * kNB, L); st.store_scaled(e_qc1, LDK, c1);
+    }
+    // dT^T[j rows, i lanes] masked to j <= i, shared as dT[i][j] for the source-side product
+#pragma unroll
+    for (int jt = 0; jt < BT; ++jt) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        if (32 * jt + acc_row(r, g) > lw + c) dtacc[jt][r] = 0.f;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) st4<T>(e_dtw + (lw + c) * LDT + 32 * jt + 8 * q + 4 * g, pack4<T>(dtacc[jt], q));
+    }
+    __syncthreads();   // e2
+#pragma unroll
+    for (int jt = 0; jt < BT; ++jt) {
+      if (32 * jt >= lw + 32) continue;
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        const frag<T> fdt = chain<T>(dtacc[jt], s2);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+          mma(dqc[nt], ld_free<T, true>(e_vuw, LDK, 32 * nt, HD, 32 * jt + 16 * s2, c, g), fdt);
+      }
+    }
+    if (i < L) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqc, b, h) + (int64_t)i * a.dqc.sl, dqc, c0, g);
   }
 }
 
@@ -1378,7 +1416,7 @@ template <typename T, typename TI, int HD> static int launch_bwd_t(const BwdArgs
       hipLaunchKernelGGL((bwd_query_kernel<T, TI, HD, 2>), grid, block, query_lds, stream, a);
     } else if constexpr (TWO_ROLE) {
       constexpr int query2_lds = bwd_query2_lds_bytes<T, HD>();
-      hipLaunchKernelGGL((bwd_query2_kernel<T, TI, HD>), grid, block, query2_lds, stream, a);
+      hipLaunchKernelGGL((bwd_query2_kernel<T, TI, HD>), grid, dim3(2 * kThreads), query2_lds, stream, a);
     } else {
       hipLaunchKernelGGL((bwd_query_kernel<T, TI, HD, 0>), grid, block, query_lds, stream, a);
     }

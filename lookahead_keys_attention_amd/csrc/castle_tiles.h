@@ -248,29 +248,29 @@ struct RowStage {
   static constexpr int N = (TOTAL + THREADS - 1) / THREADS;
   vec<TI, V> r[N];
 
-  __device__ __forceinline__ void load(const TI* src, int64_t row_stride, int64_t row0, int64_t row_end) {
+  __device__ __forceinline__ void load(const TI* src, int64_t row_stride, int64_t row0, int64_t row_end, int tid = threadIdx.x) {
 #pragma unroll
     for (int n = 0; n < N; ++n) {
-      const int v = threadIdx.x + n * THREADS;
+      const int v = tid + n * THREADS;
 #pragma unroll
       for (int e = 0; e < V; ++e) r[n][e] = (TI)0.f;
       if (v < TOTAL && row0 + v / VPR < row_end)
         r[n] = *reinterpret_cast<const vec<TI, V>*>(src + (row0 + v / VPR) * row_stride + (v % VPR) * V);
     }
   }
-  __device__ __forceinline__ void store(T* dst, int ld) const {
+  __device__ __forceinline__ void store(T* dst, int ld, int tid = threadIdx.x) const {
 #pragma unroll
     for (int n = 0; n < N; ++n) {
-      const int v = threadIdx.x + n * THREADS;
+      const int v = tid + n * THREADS;
       if (v < TOTAL) *reinterpret_cast<vec<T, V>*>(dst + (v / VPR) * ld + (v % VPR) * V) = cvt_vec<T, TI, V>(r[n]);
     }
   }
   // for tiles whose rows are only 8-byte aligned (leading dimension from lds_ld_chain)
-  __device__ __forceinline__ void store_halves(T* dst, int ld) const {
+  __device__ __forceinline__ void store_halves(T* dst, int ld, int tid = threadIdx.x) const {
     constexpr int HV = V / 2;
 #pragma unroll
     for (int n = 0; n < N; ++n) {
-      const int v = threadIdx.x + n * THREADS;
+      const int v = tid + n * THREADS;
       if (v < TOTAL) {
         const vec<T, V> x = cvt_vec<T, TI, V>(r[n]);
         typedef vec<T, HV> __attribute__((aligned(8))) half_mem;
@@ -283,10 +283,10 @@ struct RowStage {
       }
     }
   }
-  __device__ __forceinline__ void store_scaled(T* dst, int ld, float mul) const {
+  __device__ __forceinline__ void store_scaled(T* dst, int ld, float mul, int tid = threadIdx.x) const {
 #pragma unroll
     for (int n = 0; n < N; ++n) {
-      const int v = threadIdx.x + n * THREADS;
+      const int v = tid + n * THREADS;
       if (v < TOTAL) {
         vec<float, V> f = __builtin_convertvector(r[n], vec<float, V>);
 #pragma unroll
@@ -498,17 +498,17 @@ struct SnapStage {
   vec<T, V> r[N];
 
   // src: first element of the first tile (the tiles of consecutive key groups are contiguous)
-  __device__ __forceinline__ void load(const T* src) {
+  __device__ __forceinline__ void load(const T* src, int tid = threadIdx.x) {
 #pragma unroll
     for (int n = 0; n < N; ++n) {
-      const int v = threadIdx.x + n * kThreads;
+      const int v = tid + n * kThreads;
       if (v < TOTAL) r[n] = *reinterpret_cast<const vec<T, V>*>(src + (int64_t)v * V);
     }
   }
-  __device__ __forceinline__ void store(T* dst, int ld) const {
+  __device__ __forceinline__ void store(T* dst, int ld, int tid = threadIdx.x) const {
 #pragma unroll
     for (int n = 0; n < N; ++n) {
-      const int v = threadIdx.x + n * kThreads;
+      const int v = tid + n * kThreads;
       if (v < TOTAL) {
         const int tile = v / (32 * VPR), piece = (v / 32) % VPR, c = v % 32;
         *reinterpret_cast<vec<T, V>*>(dst + (32 * tile + c) * ld + piece * V) = r[n];
