@@ -57,7 +57,8 @@ int castle_abi_version(void);
 const char* castle_error_string(int code);
 
 /* Bytes of device workspace castle_fwd needs.  The forward pass leaves there what the
- * backward pass reads again (per-block T tiles, forward state snapshots, log-sum-exp);
+ * backward pass reads again (operand copies in the compute type, per-block T tiles, forward state
+ * snapshots, log-sum-exp);
  * keep the buffer alive and unmodified until castle_bwd has run.  < 0 on error. */
 int64_t castle_fwd_workspace_bytes(int B, int H, int L, int d, int dtype);
 
@@ -73,7 +74,8 @@ int castle_fwd(const castle_view4* qc, const castle_view4* kc, const castle_view
                const castle_view4* out, const castle_view4* U,
                void* workspace, int64_t workspace_bytes, void* stream);
 
-/* Bytes of extra device workspace castle_bwd needs: reverse state snapshots, delta and, for the
+/* Bytes of extra device workspace castle_bwd needs: reverse state snapshots, delta, a copy of dout in
+ * the compute type and, for the
  * 16-bit element types at d <= 64, the dS / dSu score-gradient tiles its first kernel hands to its
  * second (2 * B * H * Lp * Lp elements, Lp = L rounded up to 128). */
 int64_t castle_bwd_workspace_bytes(int B, int H, int L, int d, int dtype);

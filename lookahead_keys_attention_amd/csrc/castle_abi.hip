@@ -34,8 +34,8 @@ int64_t align_up(int64_t x, int64_t a) { return (x + a - 1) / a * a; }
 
 struct Geometry {
   int Lp, nblk;
-  int64_t lse_bytes, tblk_bytes, snap_bytes, mat_bytes;
-  int64_t off_lse, off_t, off_tt, off_snap, total;
+  int64_t lse_bytes, tblk_bytes, snap_bytes, mat_bytes, op_bytes;
+  int64_t off_lse, off_t, off_tt, off_snap, off_ops, total;
 };
 
 Geometry geometry(int B, int H, int L, int d, int es) {
@@ -52,7 +52,9 @@ Geometry geometry(int B, int H, int L, int d, int es) {
   g.off_t = g.off_lse + g.lse_bytes;
   g.off_tt = g.off_t + g.tblk_bytes;
   g.off_snap = g.off_tt + g.tblk_bytes;
-  g.total = g.off_snap + g.snap_bytes;
+  g.op_bytes = align_up(BH * g.Lp * d * es, 256);   // one operand in the compute type, padded to Lp rows
+  g.off_ops = g.off_snap + g.snap_bytes;
+  g.total = g.off_ops + 6 * g.op_bytes;
   return g;
 }
 
@@ -92,6 +94,12 @@ castle::FwdWorkspace carve(void* base, const Geometry& g) {
   w.t_blk = p + g.off_t;
   w.tt_blk = p + g.off_tt;
   w.usnap = p + g.off_snap;
+  w.qc_p = p + g.off_ops;
+  w.kc_p = p + g.off_ops + g.op_bytes;
+  w.vc_p = p + g.off_ops + 2 * g.op_bytes;
+  w.qu_p = p + g.off_ops + 3 * g.op_bytes;
+  w.ku_p = p + g.off_ops + 4 * g.op_bytes;
+  w.vu_p = p + g.off_ops + 5 * g.op_bytes;
   return w;
 }
 
@@ -150,7 +158,7 @@ int64_t castle_bwd_workspace_bytes(int B, int H, int L, int d, int dtype) {
   const int rc = check_core(B, H, L, d, dtype);
   if (rc != CASTLE_OK) return rc;
   const Geometry g = geometry(B, H, L, d, elem_size(dtype));
-  return g.snap_bytes + g.lse_bytes + 2 * g.mat_bytes;   // reverse-state snapshots + delta + dS, dSu tiles
+  return g.snap_bytes + g.lse_bytes + g.op_bytes + 2 * g.mat_bytes;   // reverse-state snapshots, delta, dO copy, dS / dSu tiles
 }
 
 int castle_bwd(const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
@@ -171,7 +179,7 @@ int castle_bwd(const castle_view4* qc, const castle_view4* kc, const castle_view
   if (fwd_workspace == nullptr || reinterpret_cast<uintptr_t>(fwd_workspace) % 256 != 0 || fwd_workspace_bytes < g.total)
     return CASTLE_ERR_WORKSPACE;
   if (bwd_workspace == nullptr || reinterpret_cast<uintptr_t>(bwd_workspace) % 256 != 0 ||
-      bwd_workspace_bytes < g.snap_bytes + g.lse_bytes + 2 * g.mat_bytes)
+      bwd_workspace_bytes < g.snap_bytes + g.lse_bytes + g.op_bytes + 2 * g.mat_bytes)
     return CASTLE_ERR_WORKSPACE;
 
   castle::BwdArgs a;
@@ -184,8 +192,9 @@ int castle_bwd(const castle_view4* qc, const castle_view4* kc, const castle_view
   a.ws = carve(const_cast<void*>(fwd_workspace), g);
   a.gsnap = bwd_workspace;
   a.delta = reinterpret_cast<float*>(static_cast<char*>(bwd_workspace) + g.snap_bytes);
-  a.ds_mat = g.mat_bytes ? static_cast<char*>(bwd_workspace) + g.snap_bytes + g.lse_bytes : nullptr;
-  a.dsu_mat = g.mat_bytes ? static_cast<char*>(bwd_workspace) + g.snap_bytes + g.lse_bytes + g.mat_bytes : nullptr;
+  a.dout_p = static_cast<char*>(bwd_workspace) + g.snap_bytes + g.lse_bytes;
+  a.ds_mat = g.mat_bytes ? static_cast<char*>(bwd_workspace) + g.snap_bytes + g.lse_bytes + g.op_bytes : nullptr;
+  a.dsu_mat = g.mat_bytes ? static_cast<char*>(bwd_workspace) + g.snap_bytes + g.lse_bytes + g.op_bytes + g.mat_bytes : nullptr;
   return castle::launch_bwd(a, dtype, (flags & CASTLE_FLAG_BF16_OPERANDS) != 0, static_cast<hipStream_t>(stream));
 }
 

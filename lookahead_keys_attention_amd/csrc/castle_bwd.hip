@@ -62,23 +62,28 @@ __device__ __forceinline__ void store_rows(T* dst_row, acc_t (&acc)[NT], float m
 }
 
 // ---------------------------------------------------------------------------
-template <typename T, int HD>
+// delta = rowsum(dO * O); also leaves dO in the compute type, padded to Lp rows, for the other kernels
+template <typename T, typename TI, int HD>
 __global__ __launch_bounds__(kThreads) void delta_kernel(BwdArgs a) {
-  constexpr int V = elem_traits<T>::vec16;
+  constexpr int V = elem_traits<TI>::vec16;
   constexpr int LPR = HD / V;
   constexpr int RPB = kThreads / LPR;
-  typedef vec<T, V> vt;
+  typedef vec<TI, V> vt;
   const int bh = blockIdx.y, b = bh / a.s.H, h = bh % a.s.H;
   const int grp = threadIdx.x / LPR, sub = threadIdx.x % LPR;
   const int64_t i = (int64_t)blockIdx.x * RPB + grp;
   if (i >= a.s.Lp) return;
   float acc = 0.f;
+  vt d;
+#pragma unroll
+  for (int e = 0; e < V; ++e) d[e] = (TI)0.f;
   if (i < a.s.L) {
-    vt o = *reinterpret_cast<const vt*>(head_ptr<T>(a.out, b, h) + i * a.out.sl + sub * V);
-    vt d = *reinterpret_cast<const vt*>(head_ptr<T>(a.dout, b, h) + i * a.dout.sl + sub * V);
+    vt o = *reinterpret_cast<const vt*>(head_ptr<TI>(a.out, b, h) + i * a.out.sl + sub * V);
+    d = *reinterpret_cast<const vt*>(head_ptr<TI>(a.dout, b, h) + i * a.dout.sl + sub * V);
 #pragma unroll
     for (int e = 0; e < V; ++e) acc = __builtin_fmaf((float)o[e], (float)d[e], acc);
   }
+  *reinterpret_cast<vec<T, V>*>(reinterpret_cast<T*>(a.dout_p) + ((int64_t)bh * a.s.Lp + i) * HD + sub * V) = cvt_vec<T, TI, V>(d);
 #pragma unroll
   for (int o = 1; o < LPR; o <<= 1) acc += __shfl_xor(acc, o);
   if (sub == 0) a.delta[(int64_t)bh * a.s.Lp + i] = acc;
@@ -124,13 +129,13 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   const int kw0 = kb * 128 + 32 * wave;
   const int k = kw0 + c;
   const int Iw = kw0 / kNB;
-  const TI* qc = head_ptr<TI>(a.qc, b, h);
-  const TI* kc = head_ptr<TI>(a.kc, b, h);
-  const TI* vc = head_ptr<TI>(a.vc, b, h);
-  const TI* qu = head_ptr<TI>(a.qu, b, h);
-  const TI* ku = head_ptr<TI>(a.ku, b, h);
-  const TI* vu = head_ptr<TI>(a.vu, b, h);
-  const TI* dout = head_ptr<TI>(a.dout, b, h);
+  const T* qc = prep_ptr<T>(a.ws.qc_p, bh, a.s.Lp, HD);
+  const T* kc = prep_ptr<T>(a.ws.kc_p, bh, a.s.Lp, HD);
+  const T* vc = prep_ptr<T>(a.ws.vc_p, bh, a.s.Lp, HD);
+  const T* qu = prep_ptr<T>(a.ws.qu_p, bh, a.s.Lp, HD);
+  const T* ku = prep_ptr<T>(a.ws.ku_p, bh, a.s.Lp, HD);
+  const T* vu = prep_ptr<T>(a.ws.vu_p, bh, a.s.Lp, HD);
+  const T* dout = prep_ptr<T>(a.dout_p, bh, a.s.Lp, HD);
   const T* tb = reinterpret_cast<const T*>(a.ws.t_blk) + (int64_t)bh * a.s.Lp * kNB;
   const T* usnap = reinterpret_cast<const T*>(a.ws.usnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
   T* gsnap = reinterpret_cast<T*>(a.gsnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
@@ -140,9 +145,9 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   frag<T> fkc[KS], fvc[KS], fqu[KS], fub[KS];
 #pragma unroll
   for (int s = 0; s < KS; ++s) {
-    fkc[s] = ldg_nat<T, TI>(kc, a.kc.sl, k, 16 * s + 8 * g, k < L);
-    fvc[s] = ldg_nat<T, TI>(vc, a.vc.sl, k, 16 * s + 8 * g, k < L);
-    fqu[s] = ldg_nat_scaled<T, TI>(qu, a.qu.sl, k, 16 * s + 8 * g, k < L, -c1);
+    fkc[s] = ldg_nat<T>(kc, HD, k, 16 * s + 8 * g, true);
+    fvc[s] = ldg_nat<T>(vc, HD, k, 16 * s + 8 * g, true);
+    fqu[s] = ldg_nat_scaled<T, T>(qu, HD, k, 16 * s + 8 * g, true, -c1);
     fub[s] = zero_frag<T>();
   }
   acc_t dvc[NT], dkc[NT], dqu[NT], G[NT];   // [n rows, k lanes]
@@ -150,15 +155,15 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   for (int nt = 0; nt < NT; ++nt) { zero(dvc[nt]); zero(dkc[nt]); zero(dqu[nt]); zero(G[nt]); }
 
   // every thread carries its 16-byte pieces of the five tiles of the next block
-  RowStage<T, TI, kNB, HD> pqc, pdo, pku, pvu;
+  RowStage<T, T, kNB, HD> pqc, pdo, pku, pvu;
   RowStage<T, T, kNB, kNB> ptb;
 #define CASTLE_BK_LOAD(I_)                                   \
   do {                                                       \
     const int64_t r_ = (int64_t)(I_) * kNB;                  \
-    pqc.load(qc, a.qc.sl, r_, L);                            \
-    pdo.load(dout, a.dout.sl, r_, L);                        \
-    pku.load(ku, a.ku.sl, r_, L);                            \
-    pvu.load(vu, a.vu.sl, r_, L);                            \
+    pqc.load(qc, HD, r_, kNoRowLimit);                            \
+    pdo.load(dout, HD, r_, kNoRowLimit);                        \
+    pku.load(ku, HD, r_, kNoRowLimit);                            \
+    pvu.load(vu, HD, r_, kNoRowLimit);                            \
     ptb.load(tb, kNB, r_, (int64_t)1 << 40);                 \
   } while (0)
 
@@ -177,7 +182,7 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
     __syncthreads();
     const int64_t r0 = (int64_t)I * kNB;
     if (!PF) CASTLE_BK_LOAD(I);
-    pqc.store_scaled(s_qc, LDK, c1);
+    pqc.store(s_qc, LDK);
     pdo.store(s_do, LDK);
     pku.store(s_ku, LDK);
     pvu.store_halves(s_vu, LDU);
@@ -354,15 +359,19 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
 // waves 0-3 "score" waves, waves 4-7 "gradient" waves; pair (w, w + 4) owns keys
 // kb*128 + 32 w .. + 31 and is expected to share a SIMD, so the element-wise chain of one role
 // overlaps the MFMAs of the other.  Per 64-query block I (swept from the last one down):
-//   score wave:    gate A_KI (-> A(1-A) for the partner), then per 32-query sub-tile the scores,
-//                  P, dS, dSu, handed over through LDS as [key][query] tiles
-//   gradient wave: reverse state G (snapshot, G Vu^T), dVc, dKc, G, dA from the handed tiles,
-//                  then dZ and dQu
-// The gradient wave runs one sub-tile behind the score wave; four barriers per block.
+//   score wave:    per 32-query sub-tile the scores, P, dS, dSu, handed over through LDS as
+//                  [key][query] tiles; then the gate A of the NEXT block (-> A(1-A) for the partner)
+//   gradient wave: dZ and dQu of the PREVIOUS block, reverse state G (snapshot, G Vu^T), then
+//                  dVc, dKc, G, dA from the handed tiles; it also stores the dS / dSu tiles for
+//                  the query-stationary kernel
+// The gradient wave runs one sub-tile behind the score wave; four barriers per block, and in each
+// of the three compute slots between them both roles have about the same amount of work.
+// The Ku tile and the A(1-A) tiles are double buffered because they outlive their block.
 template <typename T, int HD> constexpr int bwd_key2_lds_bytes() {
   int b = bwd_key_lds_bytes<T, HD>();
+  b += a16((int)sizeof(T) * kNB * lds_ld<T>(HD));           // second Ku tile
   b += 4 * 3 * a16((int)sizeof(T) * 32 * lds_ld<T>(kNB));   // P, dS, dSu per wave pair
-  b += 4 * a16((int)sizeof(T) * 32 * lds_ld<T>(kNB));       // A (1 - A) per wave pair
+  b += 2 * 4 * a16((int)sizeof(T) * 32 * lds_ld<T>(kNB));   // A (1 - A) per wave pair, two blocks
   return b;
 }
 
@@ -379,13 +388,14 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_key2_kernel(BwdArgs a) {
   Carver cv{castle_smem};
   T* s_qc = cv.take<T>(kNB * LDK);
   T* s_do = cv.take<T>(kNB * LDK);
-  T* s_ku = cv.take<T>(kNB * LDK);
+  T* s_ku0 = cv.take<T>(kNB * LDK);
+  T* s_ku1 = cv.take<T>(kNB * LDK);
   T* s_vu = cv.take<T>(kNB * LDU);
   T* s_t = cv.take<T>(kNB * LDT);
   float* s_lse = cv.take<float>(kNB);
   float* s_delta = cv.take<float>(kNB);
   T* s_x = cv.take<T>(4 * 3 * 32 * LDX);
-  T* s_w = cv.take<T>(4 * 32 * LDX);
+  T* s_w = cv.take<T>(2 * 4 * 32 * LDX);
 
   int kb, bh;
   work_item(a.s.B * a.s.H, kb, bh);
@@ -399,43 +409,58 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_key2_kernel(BwdArgs a) {
   const int k = kw0 + c;
   const int Iw = kw0 / kNB;
   const int I0 = (kb * 128) / kNB;
+  const int Ilast = a.s.nblk - 1;
   T* x_p = s_x + pw * 3 * 32 * LDX;   // [key][query of the block]
   T* x_ds = x_p + 32 * LDX;
   T* x_dsu = x_ds + 32 * LDX;
-  T* x_w = s_w + pw * 32 * LDX;       // [key][source of the block]
+  T* x_w = s_w + pw * 32 * LDX;       // [key][source of the block], + 4*32*LDX for odd blocks
 
-  const TI* qc = head_ptr<TI>(a.qc, b, h);
-  const TI* ku = head_ptr<TI>(a.ku, b, h);
-  const TI* vu = head_ptr<TI>(a.vu, b, h);
-  const TI* dout = head_ptr<TI>(a.dout, b, h);
+  const T* qc = prep_ptr<T>(a.ws.qc_p, bh, a.s.Lp, HD);
+  const T* ku = prep_ptr<T>(a.ws.ku_p, bh, a.s.Lp, HD);
+  const T* vu = prep_ptr<T>(a.ws.vu_p, bh, a.s.Lp, HD);
+  const T* dout = prep_ptr<T>(a.dout_p, bh, a.s.Lp, HD);
   const T* tb = reinterpret_cast<const T*>(a.ws.t_blk) + (int64_t)bh * a.s.Lp * kNB;
-  // All 512 threads stage the five tiles of a block: the loads of block I - 1 are issued right
-  // after the tiles of block I have been written and stay in flight for the whole block.
-#define CASTLE_BK2_STAGE_DECL                                \
-  RowStage<T, TI, kNB, HD, 2 * kThreads> pqc, pdo, pku, pvu; \
-  RowStage<T, T, kNB, kNB, 2 * kThreads> ptb
+  // The score waves (threads 0..255) stage the five tiles of a block: the loads of block I - 1 are
+  // issued right after the tiles of block I have been written.  Ku (needed first, by the gate of
+  // the next block) goes to its other buffer one slot later, the rest when block I is done.
+  // The gradient waves keep out of it: their global stores would sit in front of such loads in
+  // the in-order memory counter.
+#define CASTLE_BK2_STAGE_DECL                 \
+  RowStage<T, T, kNB, HD> pku, pqc, pdo, pvu; \
+  RowStage<T, T, kNB, kNB> ptb;               \
+  float plse = 0.f, pdelta = 0.f
 #define CASTLE_BK2_STAGE_LOAD(I_)                            \
   do {                                                       \
     const int64_t r_ = (int64_t)(I_) * kNB;                  \
-    pqc.load(qc, a.qc.sl, r_, L);                            \
-    pdo.load(dout, a.dout.sl, r_, L);                        \
-    pku.load(ku, a.ku.sl, r_, L);                            \
-    pvu.load(vu, a.vu.sl, r_, L);                            \
+    pku.load(ku, HD, r_, kNoRowLimit);                            \
+    pqc.load(qc, HD, r_, kNoRowLimit);                            \
+    pdo.load(dout, HD, r_, kNoRowLimit);                        \
+    pvu.load(vu, HD, r_, kNoRowLimit);                            \
     ptb.load(tb, kNB, r_, (int64_t)1 << 40);                 \
+    if (threadIdx.x < kNB) {                                 \
+      const int64_t i_ = r_ + threadIdx.x;                   \
+      plse = i_ < L ? lse[i_] : INFINITY;                    \
+      pdelta = i_ < L ? delta[i_] : 0.f;                     \
+    }                                                        \
   } while (0)
 #define CASTLE_BK2_STAGE_STORE()                             \
   do {                                                       \
-    pqc.store_scaled(s_qc, LDK, c1);                         \
+    pqc.store(s_qc, LDK);                         \
     pdo.store(s_do, LDK);                                    \
-    pku.store(s_ku, LDK);                                    \
     pvu.store_halves(s_vu, LDU);                             \
     ptb.store_halves(s_t, LDT);                              \
+    if (threadIdx.x < kNB) {                                 \
+      s_lse[threadIdx.x] = -plse * kLog2e;                   \
+      s_delta[threadIdx.x] = -pdelta;                        \
+    }                                                        \
   } while (0)
+#define CASTLE_BK2_KU(I_) (((I_) & 1) ? s_ku1 : s_ku0)
+#define CASTLE_BK2_W(I_) (x_w + ((I_) & 1) * 4 * 32 * LDX)
 
   if (scorer) {
-    const TI* kc = head_ptr<TI>(a.kc, b, h);
-    const TI* vc = head_ptr<TI>(a.vc, b, h);
-    const TI* qu = head_ptr<TI>(a.qu, b, h);
+    const T* kc = prep_ptr<T>(a.ws.kc_p, bh, a.s.Lp, HD);
+    const T* vc = prep_ptr<T>(a.ws.vc_p, bh, a.s.Lp, HD);
+    const T* qu = prep_ptr<T>(a.ws.qu_p, bh, a.s.Lp, HD);
     const T* usnap = reinterpret_cast<const T*>(a.ws.usnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
     const float* lse = a.ws.lse + (int64_t)bh * a.s.Lp;
     const float* delta = a.delta + (int64_t)bh * a.s.Lp;
@@ -443,75 +468,73 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_key2_kernel(BwdArgs a) {
     frag<T> fkc[KS], fvc[KS], fqu[KS], fub[KS];
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
-      fkc[s] = ldg_nat<T, TI>(kc, a.kc.sl, k, 16 * s + 8 * g, k < L);
-      fvc[s] = ldg_nat<T, TI>(vc, a.vc.sl, k, 16 * s + 8 * g, k < L);
-      fqu[s] = ldg_nat_scaled<T, TI>(qu, a.qu.sl, k, 16 * s + 8 * g, k < L, -c1);
+      fkc[s] = ldg_nat<T>(kc, HD, k, 16 * s + 8 * g, true);
+      fvc[s] = ldg_nat<T>(vc, HD, k, 16 * s + 8 * g, true);
+      fqu[s] = ldg_nat_scaled<T, T>(qu, HD, k, 16 * s + 8 * g, true, -c1);
       fub[s] = zero_frag<T>();
     }
     CASTLE_BK2_STAGE_DECL;
-#define CASTLE_BK2_LOAD(I_)                                                                        \
-  do {                                                                                             \
-    CASTLE_BK2_STAGE_LOAD(I_);                                                                     \
-    if ((I_) > Iw) {                                                                               \
-      _Pragma("unroll") for (int s = 0; s < KS; ++s)                                               \
-        fub[s] = ldg_snap_nat<T>(usnap + (usnap_off(I_) + kw0) * HD, c, 16 * s + 8 * g);           \
-    }                                                                                              \
+    frag<T> fa[BT][2];
+    // gate tiles A^T[j rows, k lanes] of source block J: operand fragments for the score tiles of
+    // that block and A (1 - A) for the partner wave
+#define CASTLE_BK2_GATE(J_)                                                                          \
+  do {                                                                                               \
+    const T* ku_tile_ = CASTLE_BK2_KU(J_);                                                           \
+    T* w_tile_ = CASTLE_BK2_W(J_);                                                                   \
+    _Pragma("unroll") for (int jt = 0; jt < BT; ++jt) {                                              \
+      acc_t aT;                                                                                      \
+      zero(aT);                                                                                      \
+      {                                                                                              \
+        frag<T> oku[KS];                                                                             \
+        _Pragma("unroll") for (int s = 0; s < KS; ++s)                                               \
+          oku[s] = ld_nat<T>(ku_tile_, LDK, 32 * jt + c, 16 * s + 8 * g);                            \
+        __builtin_amdgcn_sched_barrier(0);                                                           \
+        _Pragma("unroll") for (int s = 0; s < KS; ++s) mma(aT, oku[s], fqu[s]);                      \
+      }                                                                                              \
+      const int j0 = (J_) * kNB + 32 * jt;                                                           \
+      _Pragma("unroll") for (int r = 0; r < 16; ++r) aT[r] = fast_rcp(1.f + fast_exp2(aT[r]));       \
+      if (j0 <= kw0 + 31) { /* tile touches the diagonal: keep j > k only */                         \
+        _Pragma("unroll") for (int r = 0; r < 16; ++r)                                               \
+          if (j0 + acc_row(r, g) <= k) aT[r] = 0.f;                                                  \
+      }                                                                                              \
+      fa[jt][0] = chain<T>(aT, 0);                                                                   \
+      fa[jt][1] = chain<T>(aT, 1);                                                                   \
+      _Pragma("unroll") for (int r = 0; r < 16; ++r) aT[r] = aT[r] * (1.f - aT[r]);                  \
+      _Pragma("unroll") for (int q = 0; q < 4; ++q)                                                  \
+        st4<T>(w_tile_ + c * LDX + 32 * jt + 8 * q + 4 * g, pack4<T>(aT, q));                        \
+    }                                                                                                \
   } while (0)
 
-    CASTLE_BK2_LOAD(a.s.nblk - 1);
-    frag<T> fa[BT][2];
-    for (int I = a.s.nblk - 1; I >= I0; --I) {
+    CASTLE_BK2_STAGE_LOAD(Ilast);
+    if (Ilast > Iw) {
+#pragma unroll
+      for (int s = 0; s < KS; ++s) fub[s] = ldg_snap_nat<T>(usnap + (usnap_off(Ilast) + kw0) * HD, c, 16 * s + 8 * g);
+    }
+    pku.store(CASTLE_BK2_KU(Ilast), LDK);
+    __syncthreads();   // 0: first Ku tile staged
+    if (Ilast >= Iw) CASTLE_BK2_GATE(Ilast);
+    for (int I = Ilast; I >= I0; --I) {
       const bool active = I >= Iw;
       const bool inter = I > Iw;   // lookahead state from earlier blocks exists
       CASTLE_BK2_STAGE_STORE();
-      if (threadIdx.x < kNB) {
-        const int64_t i = (int64_t)I * kNB + threadIdx.x;
-        s_lse[threadIdx.x] = i < L ? lse[i] * kLog2e : INFINITY;
-        s_delta[threadIdx.x] = i < L ? delta[i] : 0.f;
-      }
       __syncthreads();   // 1: tiles staged
       if (I > I0) CASTLE_BK2_STAGE_LOAD(I - 1);   // in flight for the whole block
 #pragma unroll
       for (int it = 0; it < BT; ++it) {
-        if (it == 0 && active) {
-          // gate tiles A^T[j rows, k lanes] of the whole source block
-#pragma unroll
-          for (int jt = 0; jt < BT; ++jt) {
-            acc_t aT;
-            zero(aT);
-            {
-              frag<T> oku[KS];
-#pragma unroll
-              for (int s = 0; s < KS; ++s) oku[s] = ld_nat<T>(s_ku, LDK, 32 * jt + c, 16 * s + 8 * g);
-              __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-              for (int s = 0; s < KS; ++s) mma(aT, oku[s], fqu[s]);
-            }
-            const int j0 = I * kNB + 32 * jt;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) aT[r] = fast_rcp(1.f + fast_exp2(aT[r]));
-            if (j0 <= kw0 + 31) {   // tile touches the diagonal: keep j > k only
-#pragma unroll
-              for (int r = 0; r < 16; ++r)
-                if (j0 + acc_row(r, g) <= k) aT[r] = 0.f;
-            }
-            fa[jt][0] = chain<T>(aT, 0);
-            fa[jt][1] = chain<T>(aT, 1);
-#pragma unroll
-            for (int r = 0; r < 16; ++r) aT[r] = aT[r] * (1.f - aT[r]);
-#pragma unroll
-            for (int q = 0; q < 4; ++q) st4<T>(x_w + c * LDX + 32 * jt + 8 * q + 4 * g, pack4<T>(aT, q));
-          }
-        }
+        if (it == 1 && I > I0) pku.store(CASTLE_BK2_KU(I - 1), LDK);
         const int i0 = I * kNB + 32 * it;
         if (active && i0 + 31 >= kw0) {   // else every query precedes every key of this wave
-          acc_t sc, su, dp;
+          acc_t sc, su, dp;   // sc starts from -lse, dp from -delta of its row
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int il = 32 * it + acc_row(r, g);
-            sc[r] = -s_lse[il];
-            dp[r] = -s_delta[il];
-            su[r] = 0.f;
+          for (int q = 0; q < 4; ++q) {
+            const vec<float, 4> nl = *reinterpret_cast<const vec<float, 4>*>(s_lse + 32 * it + 8 * q + 4 * g);
+            const vec<float, 4> nd = *reinterpret_cast<const vec<float, 4>*>(s_delta + 32 * it + 8 * q + 4 * g);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              sc[4 * q + e] = nl[e];
+              dp[4 * q + e] = nd[e];
+              su[4 * q + e] = 0.f;
+            }
           }
           {
             frag<T> oq[KS], od[KS], ot[BT][2];
@@ -542,12 +565,15 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_key2_kernel(BwdArgs a) {
                 if (jt <= it) mma(su, ot[jt][s2], fa[jt][s2]);
           }
           acc_t ds, dsu;
-          const bool diag = i0 < kw0 + 31;   // tile touches the diagonal
+          if (i0 < kw0 + 31) {   // tile touches the diagonal: queries before the key see nothing
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+              if (i0 + acc_row(r, g) < k) sc[r] = -INFINITY;
+          }
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             const float sg = fast_rcp(1.f + fast_exp2(-su[r]));
-            float p = fast_exp2(__builtin_fmaf(-su[r], sg, sc[r]));   // sc carries -lse
-            if (diag && i0 + acc_row(r, g) < k) p = 0.f;
+            const float p = fast_exp2(__builtin_fmaf(-su[r], sg, sc[r]));   // sc carries -lse
             const float dsv = p * dp[r];                      // dp carries -delta
             const float y = su[r] * kLn2;                     // true Su
             const float t = __builtin_fmaf(-y, sg, y);        // y (1 - sigmoid)
@@ -566,13 +592,16 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_key2_kernel(BwdArgs a) {
         }
         __syncthreads();   // 2, 3: sub-tile handed over
       }
-      if (I - 1 > Iw && I > I0) {   // lookahead state as of the next block
+      if (I > I0) {
+        if (I - 1 > Iw) {   // lookahead state as of the next block: in flight behind the gate
 #pragma unroll
-        for (int s = 0; s < KS; ++s) fub[s] = ldg_snap_nat<T>(usnap + (usnap_off(I - 1) + kw0) * HD, c, 16 * s + 8 * g);
+          for (int s = 0; s < KS; ++s) fub[s] = ldg_snap_nat<T>(usnap + (usnap_off(I - 1) + kw0) * HD, c, 16 * s + 8 * g);
+        }
+        if (I - 1 >= Iw) CASTLE_BK2_GATE(I - 1);   // while the gradient waves finish block I
       }
       __syncthreads();   // 4: tiles free
     }
-#undef CASTLE_BK2_LOAD
+#undef CASTLE_BK2_GATE
   } else {
     T* gsnap = reinterpret_cast<T*>(a.gsnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
     T* ds_mat = reinterpret_cast<T*>(a.ds_mat) + (int64_t)bh * a.s.Lp * a.s.Lp;
@@ -580,17 +609,39 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_key2_kernel(BwdArgs a) {
     acc_t dvc[NT], dkc[NT], dqu[NT], G[NT];   // [n rows, k lanes]
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) { zero(dvc[nt]); zero(dkc[nt]); zero(dqu[nt]); zero(G[nt]); }
-    CASTLE_BK2_STAGE_DECL;
-    CASTLE_BK2_STAGE_LOAD(a.s.nblk - 1);
-    for (int I = a.s.nblk - 1; I >= I0; --I) {
+    acc_t dA[BT];   // dA^T[j rows, k lanes] of the block in flight
+#pragma unroll
+    for (int jt = 0; jt < BT; ++jt) zero(dA[jt]);
+    // dZ^T = dA^T * A (1 - A)  ->  dQu, for source block J (its Ku tile and A(1-A) are still there)
+#define CASTLE_BK2_DQU(J_)                                                                           \
+  do {                                                                                               \
+    const T* ku_tile_ = CASTLE_BK2_KU(J_);                                                           \
+    const T* w_tile_ = CASTLE_BK2_W(J_);                                                             \
+    _Pragma("unroll") for (int jt = 0; jt < BT; ++jt) {                                              \
+      _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                                \
+        const vec<T, 4> w = *reinterpret_cast<const vec4_mem<T>*>(w_tile_ + c * LDX + 32 * jt + 8 * q + 4 * g); \
+        _Pragma("unroll") for (int e = 0; e < 4; ++e) dA[jt][4 * q + e] *= (float)w[e];              \
+      }                                                                                              \
+      frag<T> okt[2][NT];                                                                            \
+      _Pragma("unroll") for (int s2 = 0; s2 < 2; ++s2)                                               \
+        _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                            \
+          okt[s2][nt] = ld_free<T, true>(ku_tile_, LDK, 32 * nt, HD, 32 * jt + 16 * s2, c, g);       \
+      __builtin_amdgcn_sched_barrier(0);                                                             \
+      _Pragma("unroll") for (int s2 = 0; s2 < 2; ++s2) {                                             \
+        const frag<T> fdz = chain<T>(dA[jt], s2);                                                    \
+        _Pragma("unroll") for (int nt = 0; nt < NT; ++nt) mma(dqu[nt], okt[s2][nt], fdz);            \
+      }                                                                                              \
+    }                                                                                                \
+  } while (0)
+
+    __syncthreads();   // 0
+    for (int I = Ilast; I >= I0; --I) {
       const bool active = I >= Iw;
-      CASTLE_BK2_STAGE_STORE();
       if (active && I <= a.s.nblk - 2)   // reverse state as of block I
         store_snap_tile<T, HD, NT>(gsnap + (gsnap_off(I) + kw0) * HD, G, c, g);
       __syncthreads();   // 1
-      if (I > I0) CASTLE_BK2_STAGE_LOAD(I - 1);
-      // dA^T[j rows, k lanes], second term first: G (before this block) times Vu^T
-      acc_t dA[BT];
+      if (I < Ilast && I + 1 >= Iw) CASTLE_BK2_DQU(I + 1);   // finish the previous block
+      // dA^T of this block, second term first: G (before this block) times Vu^T
 #pragma unroll
       for (int jt = 0; jt < BT; ++jt) {
         zero(dA[jt]);
@@ -617,8 +668,8 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_key2_kernel(BwdArgs a) {
             const frag<T> fdsu = ld_nat<T>(x_dsu, LDX, c, ic + 8 * g);
             {   // hand the tile to the query-stationary kernel: 1 KB contiguous per store
               const int64_t tile = ((int64_t)(kw0 / 32) * (a.s.Lp / 32) + i0 / 32) * 1024 + s2 * 512 + c * 16 + g * 8;
-              *reinterpret_cast<frag_mem<T>*>(ds_mat + tile) = fds;
-              *reinterpret_cast<frag_mem<T>*>(dsu_mat + tile) = fdsu;
+              __builtin_nontemporal_store(fds, reinterpret_cast<frag_mem<T>*>(ds_mat + tile));
+              __builtin_nontemporal_store(fdsu, reinterpret_cast<frag_mem<T>*>(dsu_mat + tile));
             }
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
@@ -641,32 +692,10 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_key2_kernel(BwdArgs a) {
           }
         }
       }
-      // dZ^T = dA^T * A (1 - A)  ->  dQu
-      if (active) {
-#pragma unroll
-        for (int jt = 0; jt < BT; ++jt) {
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const vec<T, 4> w = *reinterpret_cast<const vec4_mem<T>*>(x_w + c * LDX + 32 * jt + 8 * q + 4 * g);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) dA[jt][4 * q + e] *= (float)w[e];
-          }
-          frag<T> okt[2][NT];
-#pragma unroll
-          for (int s2 = 0; s2 < 2; ++s2)
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) okt[s2][nt] = ld_free<T, true>(s_ku, LDK, 32 * nt, HD, 32 * jt + 16 * s2, c, g);
-          __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int s2 = 0; s2 < 2; ++s2) {
-            const frag<T> fdz = chain<T>(dA[jt], s2);
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) mma(dqu[nt], okt[s2][nt], fdz);
-          }
-        }
-      }
       __syncthreads();   // 4
     }
+    if (I0 >= Iw) CASTLE_BK2_DQU(I0);
+#undef CASTLE_BK2_DQU
     if (k < L) {
       store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dkc, b, h) + (int64_t)k * a.dkc.sl, dkc, kLn2, g);
       store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvc, b, h) + (int64_t)k * a.dvc.sl, dvc, 1.f, g);
@@ -676,6 +705,8 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_key2_kernel(BwdArgs a) {
 #undef CASTLE_BK2_STAGE_DECL
 #undef CASTLE_BK2_STAGE_LOAD
 #undef CASTLE_BK2_STAGE_STORE
+#undef CASTLE_BK2_KU
+#undef CASTLE_BK2_W
 }
 
 // ---------------------------------------------------------------------------
@@ -735,13 +766,13 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
   const T* s_ubw = qw == 0 ? s_ub0 : s_ub1;
   const T* s_gw = qw == 0 ? s_g0 : s_g1;
 
-  const TI* qc = head_ptr<TI>(a.qc, b, h);
-  const TI* kc = head_ptr<TI>(a.kc, b, h);
-  const TI* vc = head_ptr<TI>(a.vc, b, h);
-  const TI* qu = head_ptr<TI>(a.qu, b, h);
-  const TI* ku = head_ptr<TI>(a.ku, b, h);
-  const TI* vu = head_ptr<TI>(a.vu, b, h);
-  const TI* dout = head_ptr<TI>(a.dout, b, h);
+  const T* qc = prep_ptr<T>(a.ws.qc_p, bh, a.s.Lp, HD);
+  const T* kc = prep_ptr<T>(a.ws.kc_p, bh, a.s.Lp, HD);
+  const T* vc = prep_ptr<T>(a.ws.vc_p, bh, a.s.Lp, HD);
+  const T* qu = prep_ptr<T>(a.ws.qu_p, bh, a.s.Lp, HD);
+  const T* ku = prep_ptr<T>(a.ws.ku_p, bh, a.s.Lp, HD);
+  const T* vu = prep_ptr<T>(a.ws.vu_p, bh, a.s.Lp, HD);
+  const T* dout = prep_ptr<T>(a.dout_p, bh, a.s.Lp, HD);
   const T* tb = reinterpret_cast<const T*>(a.ws.t_blk) + (int64_t)bh * a.s.Lp * kNB;
   const T* ttb = reinterpret_cast<const T*>(a.ws.tt_blk) + (int64_t)bh * a.s.Lp * kNB;
   const T* usnap = reinterpret_cast<const T*>(a.ws.usnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
@@ -750,10 +781,10 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
   frag<T> fqc[KS], fdo[KS], fku[KS], fvu[KS], ft[TS], ftt[TS];
 #pragma unroll
   for (int s = 0; s < KS; ++s) {
-    fqc[s] = ldg_nat_scaled<T, TI>(qc, a.qc.sl, i, 16 * s + 8 * g, i < L, c1);
-    fdo[s] = ldg_nat<T, TI>(dout, a.dout.sl, i, 16 * s + 8 * g, i < L);
-    fku[s] = ldg_nat_scaled<T, TI>(ku, a.ku.sl, i, 16 * s + 8 * g, i < L, -c1);
-    fvu[s] = ldg_nat<T, TI>(vu, a.vu.sl, i, 16 * s + 8 * g, i < L);
+    fqc[s] = ldg_nat<T>(qc, HD, i, 16 * s + 8 * g, true);
+    fdo[s] = ldg_nat<T>(dout, HD, i, 16 * s + 8 * g, true);
+    fku[s] = ldg_nat_scaled<T, T>(ku, HD, i, 16 * s + 8 * g, true, -c1);
+    fvu[s] = ldg_nat<T>(vu, HD, i, 16 * s + 8 * g, true);
   }
 #pragma unroll
   for (int s = 0; s < TS; ++s) {
@@ -771,15 +802,15 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
   for (int jt = 0; jt < BT; ++jt) zero(dtacc[jt]);
 
   // staging: every thread carries one 16-byte piece of each of the 7 tiles of the next chunk
-  RowStage<T, TI, kCK, HD> pkc, pvc, pqu;
+  RowStage<T, T, kCK, HD> pkc, pvc, pqu;
   SnapStage<T, kCK, HD> pu0, pu1, pg0, pg1;
   const int blk0 = Ifirst, blk1 = Ifirst + 1;
 #define CASTLE_BQ_LOAD(K0)                                                                                      \
   do {                                                                                                          \
     const int kb_ = (K0) / kNB;                                                                                 \
-    pkc.load(kc, a.kc.sl, (K0), L);                                                                             \
-    pvc.load(vc, a.vc.sl, (K0), L);                                                                             \
-    pqu.load(qu, a.qu.sl, (K0), L);                                                                             \
+    pkc.load(kc, HD, (K0), kNoRowLimit);                                                                             \
+    pvc.load(vc, HD, (K0), kNoRowLimit);                                                                             \
+    pqu.load(qu, HD, (K0), kNoRowLimit);                                                                             \
     if (kb_ < blk0) pu0.load(usnap + (usnap_off(blk0) + (K0)) * HD);                          \
     if (kb_ < blk1 && blk1 < a.s.nblk) pu1.load(usnap + (usnap_off(blk1) + (K0)) * HD);        \
     if (DO_S && kb_ <= blk0 && blk0 <= a.s.nblk - 2) pg0.load(gsnap + (gsnap_off(blk0) + (K0)) * HD);  \
@@ -929,22 +960,20 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
 #pragma unroll
         for (int s = 0; s < TS; ++s) ods[s] = ld_free<T, false>(s_dsut + cb * LDC, LDC, 32 * kt, kCK, 16 * s, c, g);
 #pragma unroll
-        for (int s = 0; s < KS; ++s) og[s] = ld_nat<T>(s_gw, LDK, 32 * kt + c, 16 * s + 8 * g);
+        for (int s = 0; s < KS; ++s) og[s] = has_g ? ld_nat<T>(s_gw, LDK, 32 * kt + c, 16 * s + 8 * g) : zero_frag<T>();
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
           for (int nt = 0; nt < NT; ++nt) {
             oqt[s2][nt] = ld_free<T, true>(s_qu, LDK, 32 * nt, HD, 32 * kt + 16 * s2, c, g);
-            ogt[s2][nt] = ld_free<T, true>(s_gw, LDK, 32 * nt, HD, 32 * kt + 16 * s2, c, g);
+            ogt[s2][nt] = has_g ? ld_free<T, true>(s_gw, LDK, 32 * nt, HD, 32 * kt + 16 * s2, c, g) : zero_frag<T>();
           }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int s = 0; s < TS; ++s)
           if (s >= ifirst) mma(dA, ods[s], ftt[s]);
-        if (has_g) {
 #pragma unroll
-          for (int s = 0; s < KS; ++s) mma(dA, og[s], fvu[s]);
-        }
+        for (int s = 0; s < KS; ++s) mma(dA, og[s], fvu[s]);   // og is zero where no reverse state exists
       }
       acc_t dz;
 #pragma unroll
@@ -955,7 +984,7 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
           mma(dku[nt], oqt[s2][nt], fdz);
-          if (has_g) mma(dvu[nt], ogt[s2][nt], fa);
+          mma(dvu[nt], ogt[s2][nt], fa);
         }
       }
     }
@@ -972,11 +1001,11 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
   T* e_dt0 = ce.take<T>(kNB * LDT);   // dT, [query i][source j] (block local)
   T* e_dt1 = ce.take<T>(kNB * LDT);
   {
-    RowStage<T, TI, kNB, HD> st;
-    st.load(vu, a.vu.sl, (int64_t)blk0 * kNB, L); st.store(e_vu0, LDK);
-    st.load(vu, a.vu.sl, (int64_t)blk1 * kNB, L); st.store(e_vu1, LDK);
-    st.load(qc, a.qc.sl, (int64_t)blk0 * kNB, L); st.store_scaled(e_qc0, LDK, c1);
-    st.load(qc, a.qc.sl, (int64_t)blk1 * kNB, L); st.store_scaled(e_qc1, LDK, c1);
+    RowStage<T, T, kNB, HD> st;
+    st.load(vu, HD, (int64_t)blk0 * kNB, kNoRowLimit); st.store(e_vu0, LDK);
+    st.load(vu, HD, (int64_t)blk1 * kNB, kNoRowLimit); st.store(e_vu1, LDK);
+    st.load(qc, HD, (int64_t)blk0 * kNB, kNoRowLimit); st.store(e_qc0, LDK);
+    st.load(qc, HD, (int64_t)blk1 * kNB, kNoRowLimit); st.store(e_qc1, LDK);
   }
   const T* e_vuw = qw == 0 ? e_vu0 : e_vu1;
   const T* e_qcw = qw == 0 ? e_qc0 : e_qc1;
@@ -1114,8 +1143,8 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
   T* e_dtw = qw == 0 ? e_dt0 : e_dt1;
   const int blk0 = Ifirst, blk1 = Ifirst + 1;
 
-  const TI* qc = head_ptr<TI>(a.qc, b, h);
-  const TI* vu = head_ptr<TI>(a.vu, b, h);
+  const T* qc = prep_ptr<T>(a.ws.qc_p, bh, a.s.Lp, HD);
+  const T* vu = prep_ptr<T>(a.ws.vu_p, bh, a.s.Lp, HD);
   const T* usnap = reinterpret_cast<const T*>(a.ws.usnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
   const T* gsnap = reinterpret_cast<const T*>(a.gsnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
   const int64_t tile_row = (int64_t)(a.s.Lp / 32) * 1024;   // elements between the tiles of consecutive key groups
@@ -1126,15 +1155,15 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
   TileStage<T> pds, pdsu;   // every thread: one piece of each
 
   if (source_role) {
-    const TI* kc = head_ptr<TI>(a.kc, b, h);
-    const TI* qu = head_ptr<TI>(a.qu, b, h);
-    const TI* ku = head_ptr<TI>(a.ku, b, h);
+    const T* kc = prep_ptr<T>(a.ws.kc_p, bh, a.s.Lp, HD);
+    const T* qu = prep_ptr<T>(a.ws.qu_p, bh, a.s.Lp, HD);
+    const T* ku = prep_ptr<T>(a.ws.ku_p, bh, a.s.Lp, HD);
     const T* ttb = reinterpret_cast<const T*>(a.ws.tt_blk) + (int64_t)bh * a.s.Lp * kNB;
     frag<T> fku[KS], fvu[KS], ftt[TS];
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
-      fku[s] = ldg_nat_scaled<T, TI>(ku, a.ku.sl, i, 16 * s + 8 * g, i < L, -c1);
-      fvu[s] = ldg_nat<T, TI>(vu, a.vu.sl, i, 16 * s + 8 * g, i < L);
+      fku[s] = ldg_nat_scaled<T, T>(ku, HD, i, 16 * s + 8 * g, true, -c1);
+      fvu[s] = ldg_nat<T>(vu, HD, i, 16 * s + 8 * g, true);
     }
 #pragma unroll
     for (int s = 0; s < TS; ++s) ftt[s] = ldg_nat<T>(ttb, kNB, i, 16 * s + 8 * g, s >= ifirst);
@@ -1143,12 +1172,12 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
     for (int nt = 0; nt < NT; ++nt) { zero(dku[nt]); zero(dvu[nt]); }
 
     // this role stages kc, qu and the lookahead state of the first block
-    RowStage<T, TI, kCK, HD> pkc, pqu;
+    RowStage<T, T, kCK, HD> pkc, pqu;
     SnapStage<T, kCK, HD> pu0;
 #define CASTLE_BQ2_LOAD_A(K0)                                                            \
   do {                                                                                   \
-    pkc.load(kc, a.kc.sl, (K0), L, tid);                                                 \
-    pqu.load(qu, a.qu.sl, (K0), L, tid);                                                 \
+    pkc.load(kc, HD, (K0), kNoRowLimit, tid);                                                 \
+    pqu.load(qu, HD, (K0), kNoRowLimit, tid);                                                 \
     if ((K0) / kNB < blk0) pu0.load(usnap + (usnap_off(blk0) + (K0)) * HD, tid);         \
     pds.load(dsm + (int64_t)((K0) / 32) * tile_row);                                     \
     pdsu.load(dsum + (int64_t)((K0) / 32) * tile_row);                                   \
@@ -1199,22 +1228,20 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
 #pragma unroll
         for (int s = 0; s < TS; ++s) ods[s] = ld_nat<T>(s_dsu, LDD, c, cb + 16 * s + 8 * g);
 #pragma unroll
-        for (int s = 0; s < KS; ++s) og[s] = ld_nat<T>(s_gw, LDK, c, 16 * s + 8 * g);
+        for (int s = 0; s < KS; ++s) og[s] = has_g ? ld_nat<T>(s_gw, LDK, c, 16 * s + 8 * g) : zero_frag<T>();
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
           for (int nt = 0; nt < NT; ++nt) {
             oqt[s2][nt] = ld_free<T, true>(s_qu, LDK, 32 * nt, HD, 16 * s2, c, g);
-            ogt[s2][nt] = ld_free<T, true>(s_gw, LDK, 32 * nt, HD, 16 * s2, c, g);
+            ogt[s2][nt] = has_g ? ld_free<T, true>(s_gw, LDK, 32 * nt, HD, 16 * s2, c, g) : zero_frag<T>();
           }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int s = 0; s < TS; ++s)
           if (s >= ifirst) mma(dA, ods[s], ftt[s]);
-        if (has_g) {
 #pragma unroll
-          for (int s = 0; s < KS; ++s) mma(dA, og[s], fvu[s]);
-        }
+        for (int s = 0; s < KS; ++s) mma(dA, og[s], fvu[s]);   // og is zero where no reverse state exists
       }
       acc_t dz;
 #pragma unroll
@@ -1225,7 +1252,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
           mma(dku[nt], oqt[s2][nt], fdz);
-          if (has_g) mma(dvu[nt], ogt[s2][nt], fa);
+          mma(dvu[nt], ogt[s2][nt], fa);
         }
       }
     }
@@ -1233,11 +1260,11 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
     // ---- epilogue: in-block term dvu += dT^T Qc' --------------------------------------------
     __syncthreads();   // e1: chunk tiles dead
     {
-      RowStage<T, TI, kNB, HD, 2 * kThreads> st;
-      st.load(vu, a.vu.sl, (int64_t)blk0 * kNB, L); st.store(e_vu0, LDK);
-      st.load(vu, a.vu.sl, (int64_t)blk1 * kNB, L); st.store(e_vu1, LDK);
-      st.load(qc, a.qc.sl, (int64_t)blk0 * kNB, L); st.store_scaled(e_qc0, LDK, c1);
-      st.load(qc, a.qc.sl, (int64_t)blk1 * kNB, L); st.store_scaled(e_qc1, LDK, c1);
+      RowStage<T, T, kNB, HD, 2 * kThreads> st;
+      st.load(vu, HD, (int64_t)blk0 * kNB, kNoRowLimit); st.store(e_vu0, LDK);
+      st.load(vu, HD, (int64_t)blk1 * kNB, kNoRowLimit); st.store(e_vu1, LDK);
+      st.load(qc, HD, (int64_t)blk0 * kNB, kNoRowLimit); st.store(e_qc0, LDK);
+      st.load(qc, HD, (int64_t)blk1 * kNB, kNoRowLimit); st.store(e_qc1, LDK);
     }
     __syncthreads();   // e2: epilogue tiles and dT shared
 #pragma unroll
@@ -1325,11 +1352,11 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
     // ---- epilogue: dT = tril(dTacc):  dqc += dT Vu -------------------------------------------
     __syncthreads();   // e1
     {
-      RowStage<T, TI, kNB, HD, 2 * kThreads> st;
-      st.load(vu, a.vu.sl, (int64_t)blk0 * kNB, L); st.store(e_vu0, LDK);
-      st.load(vu, a.vu.sl, (int64_t)blk1 * kNB, L); st.store(e_vu1, LDK);
-      st.load(qc, a.qc.sl, (int64_t)blk0 * kNB, L); st.store_scaled(e_qc0, LDK, c1);
-      st.load(qc, a.qc.sl, (int64_t)blk1 * kNB, L); st.store_scaled(e_qc1, LDK, c1);
+      RowStage<T, T, kNB, HD, 2 * kThreads> st;
+      st.load(vu, HD, (int64_t)blk0 * kNB, kNoRowLimit); st.store(e_vu0, LDK);
+      st.load(vu, HD, (int64_t)blk1 * kNB, kNoRowLimit); st.store(e_vu1, LDK);
+      st.load(qc, HD, (int64_t)blk0 * kNB, kNoRowLimit); st.store(e_qc0, LDK);
+      st.load(qc, HD, (int64_t)blk1 * kNB, kNoRowLimit); st.store(e_qc1, LDK);
     }
     // dT^T[j rows, i lanes] masked to j <= i, shared as dT[i][j] for the source-side product
 #pragma unroll
@@ -1395,7 +1422,7 @@ template <typename T, typename TI, int HD> static int launch_bwd_t(const BwdArgs
   const dim3 grid(a.s.Lp / 128 * BH), block(kThreads);
   {
     ProfScope ps(kSlotDelta, stream);
-    hipLaunchKernelGGL((delta_kernel<TI, HD>), dim3((a.s.Lp + RPB - 1) / RPB, BH), block, 0, stream, a);
+    hipLaunchKernelGGL((delta_kernel<T, TI, HD>), dim3((a.s.Lp + RPB - 1) / RPB, BH), block, 0, stream, a);
   }
   {
     ProfScope ps(kSlotBwdKey, stream);

@@ -1,5 +1,8 @@
 // CASTLE parallel forward for gfx950: O(L^2 d) state form in three kernels.
 //
+//   prep_kernel  the six operands -> compute type, [B*H][Lp][d] contiguous, rows >= L zero, Qc
+//                pre-multiplied by scale*log2(e); every other kernel reads these copies, so its
+//                tile loads need neither conversions nor bounds nor strides
 //   tqv_kernel   per 64-row block I:  T_II = tril(Qc_I Vu_I^T)  (and its transpose)
 //   scan_kernel  key-stationary: for a group of 128 keys sweep the source blocks I,
 //                A_KI = sigmoid(s Qu_K Ku_I^T) (strictly j>k), state += A_KI Vu_I.
@@ -43,6 +46,39 @@ template <typename T> __device__ __forceinline__ T* head_ptr_mut(const View4& v,
 }
 
 // ---------------------------------------------------------------------------
+// One 16-byte piece of one operand per thread; blockIdx.z selects the operand.
+template <typename T, typename TI, int HD>
+__global__ __launch_bounds__(kThreads) void prep_kernel(FwdArgs a) {
+  constexpr int V = elem_traits<T>::vec16;
+  constexpr int VPR = HD / V;
+  const int bh = blockIdx.y, b = bh / a.s.H, h = bh % a.s.H;
+  const int64_t piece = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  const int64_t row = piece / VPR;
+  const int cv = (int)(piece % VPR);
+  if (row >= a.s.Lp) return;
+  View4 src;
+  void* dstv;
+  float mul = 1.f;
+  switch (blockIdx.z) {
+    case 0: src = a.qc; dstv = a.ws.qc_p; mul = a.s.scale * kLog2e; break;
+    case 1: src = a.kc; dstv = a.ws.kc_p; break;
+    case 2: src = a.vc; dstv = a.ws.vc_p; break;
+    case 3: src = a.qu; dstv = a.ws.qu_p; break;
+    case 4: src = a.ku; dstv = a.ws.ku_p; break;
+    default: src = a.vu; dstv = a.ws.vu_p; break;
+  }
+  vec<float, V> f;
+#pragma unroll
+  for (int e = 0; e < V; ++e) f[e] = 0.f;
+  if (row < a.s.L)
+    f = __builtin_convertvector(*reinterpret_cast<const vec<TI, V>*>(head_ptr<TI>(src, b, h) + row * src.sl + cv * V), vec<float, V>);
+#pragma unroll
+  for (int e = 0; e < V; ++e) f[e] *= mul;
+  T* dst = reinterpret_cast<T*>(dstv) + ((int64_t)bh * a.s.Lp + row) * HD + cv * V;
+  *reinterpret_cast<vec<T, V>*>(dst) = __builtin_convertvector(f, vec<T, V>);
+}
+
+// ---------------------------------------------------------------------------
 template <typename T, typename TI, int HD>
 __global__ __launch_bounds__(kThreads) void tqv_kernel(FwdArgs a) {
   constexpr int KS = HD / 16;
@@ -50,8 +86,8 @@ __global__ __launch_bounds__(kThreads) void tqv_kernel(FwdArgs a) {
   const int I = blockIdx.x, bh = blockIdx.y, b = bh / a.s.H, h = bh % a.s.H;
   const int lane = lane_id(), c = lane & 31, g = lane >> 5;
   const float c1 = a.s.scale * kLog2e;
-  const TI* qc = head_ptr<TI>(a.qc, b, h);
-  const TI* vu = head_ptr<TI>(a.vu, b, h);
+  const T* qc = prep_ptr<T>(a.ws.qc_p, bh, a.s.Lp, HD);   // pre-scaled by c1
+  const T* vu = prep_ptr<T>(a.ws.vu_p, bh, a.s.Lp, HD);
   T* tb = reinterpret_cast<T*>(a.ws.t_blk) + (int64_t)bh * a.s.Lp * kNB;
   T* ttb = reinterpret_cast<T*>(a.ws.tt_blk) + (int64_t)bh * a.s.Lp * kNB;
   for (int t = wave_id(); t < TB * TB; t += kThreads / 64) {
@@ -62,13 +98,13 @@ __global__ __launch_bounds__(kThreads) void tqv_kernel(FwdArgs a) {
     zero(acc);
 #pragma unroll
     for (int s = 0; s < KS; ++s)
-      mma(acc, ldg_nat<T, TI>(qc, a.qc.sl, i, 16 * s + 8 * g, i < a.s.L), ldg_nat<T, TI>(vu, a.vu.sl, j, 16 * s + 8 * g, j < a.s.L));
-    // acc[r] = (Qc Vu^T)[il = 32 it + acc_row][jl = 32 jt + c]; stored as T' = c1 * tril(.)
+      mma(acc, ldg_nat<T>(qc, HD, i, 16 * s + 8 * g, true), ldg_nat<T>(vu, HD, j, 16 * s + 8 * g, true));
+    // acc[r] = (Qc' Vu^T)[il = 32 it + acc_row][jl = 32 jt + c]; stored as T' = tril(.)
     const int jl = 32 * jt + c;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int il = 32 * it + acc_row(r, g);
-      acc[r] = jl > il ? 0.f : acc[r] * c1;
+      acc[r] = jl > il ? 0.f : acc[r];
       tb[((int64_t)I * kNB + il) * kNB + jl] = (T)acc[r];
     }
 #pragma unroll
@@ -97,25 +133,25 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(FwdArgs a) {
   const float c1 = a.s.scale * kLog2e;
   const int kw0 = kb * 128 + 32 * wave;
   const int k = kw0 + c;
-  const TI* qu = head_ptr<TI>(a.qu, b, h);
-  const TI* ku = head_ptr<TI>(a.ku, b, h);
-  const TI* vu = head_ptr<TI>(a.vu, b, h);
+  const T* qu = prep_ptr<T>(a.ws.qu_p, bh, a.s.Lp, HD);
+  const T* ku = prep_ptr<T>(a.ws.ku_p, bh, a.s.Lp, HD);
+  const T* vu = prep_ptr<T>(a.ws.vu_p, bh, a.s.Lp, HD);
   T* snap = reinterpret_cast<T*>(a.ws.usnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
 
   frag<T> fq[KS];   // -c1 * Qu rows of this wave
 #pragma unroll
-  for (int s = 0; s < KS; ++s) fq[s] = ldg_nat_scaled<T, TI>(qu, a.qu.sl, k, 16 * s + 8 * g, k < L, -c1);
+  for (int s = 0; s < KS; ++s) fq[s] = ldg_nat_scaled<T, T>(qu, HD, k, 16 * s + 8 * g, true, -c1);
   acc_t st[NT];   // state^T : rows n (head dim), columns k (lanes)
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) zero(st[nt]);
   if (HDP > HD) lds_zero(s_vut + HD * LDV, (HDP - HD) * LDV);
 
-  RowStage<T, TI, kNB, HD> pku;
-  ColStage<T, TI, kNB, HD> pvu;
+  RowStage<T, T, kNB, HD> pku;
+  ColStage<T, T, kNB, HD> pvu;
   const int I0 = (kb * 128) / kNB;
   if (PF) {
-    pku.load(ku, a.ku.sl, (int64_t)I0 * kNB, L);
-    pvu.load(vu, a.vu.sl, (int64_t)I0 * kNB, L);
+    pku.load(ku, HD, (int64_t)I0 * kNB, kNoRowLimit);
+    pvu.load(vu, HD, (int64_t)I0 * kNB, kNoRowLimit);
   }
   for (int I = I0; I < a.s.nblk; ++I) {
     if (I * kNB >= kw0 + 32) {   // all keys of this wave precede block I: snapshot
@@ -123,14 +159,14 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(FwdArgs a) {
     }
     __syncthreads();
     if (!PF) {
-      pku.load(ku, a.ku.sl, (int64_t)I * kNB, L);
-      pvu.load(vu, a.vu.sl, (int64_t)I * kNB, L);
+      pku.load(ku, HD, (int64_t)I * kNB, kNoRowLimit);
+      pvu.load(vu, HD, (int64_t)I * kNB, kNoRowLimit);
     }
     pku.store(s_ku, LDK);
     pvu.store(s_vut, LDV);
     if (PF && I + 1 < a.s.nblk) {   // in flight while this block is processed
-      pku.load(ku, a.ku.sl, (int64_t)(I + 1) * kNB, L);
-      pvu.load(vu, a.vu.sl, (int64_t)(I + 1) * kNB, L);
+      pku.load(ku, HD, (int64_t)(I + 1) * kNB, kNoRowLimit);
+      pvu.load(vu, HD, (int64_t)(I + 1) * kNB, kNoRowLimit);
     }
     __syncthreads();
 #pragma unroll
@@ -200,19 +236,19 @@ __global__ __launch_bounds__(kThreads, (sizeof(T) == 2 && HD <= 64) ? 2 : 1) voi
   const int cb = (jw / kNB) * kNB;              // first column of its block
   const int nintra = ((jw % kNB) + 32) / 16;    // contraction steps of the in-block term
 
-  const TI* qc = head_ptr<TI>(a.qc, b, h);
-  const TI* kc = head_ptr<TI>(a.kc, b, h);
-  const TI* vc = head_ptr<TI>(a.vc, b, h);
-  const TI* qu = head_ptr<TI>(a.qu, b, h);
-  const TI* ku = head_ptr<TI>(a.ku, b, h);
+  const T* qc = prep_ptr<T>(a.ws.qc_p, bh, a.s.Lp, HD);   // pre-scaled by c1
+  const T* kc = prep_ptr<T>(a.ws.kc_p, bh, a.s.Lp, HD);
+  const T* vc = prep_ptr<T>(a.ws.vc_p, bh, a.s.Lp, HD);
+  const T* qu = prep_ptr<T>(a.ws.qu_p, bh, a.s.Lp, HD);
+  const T* ku = prep_ptr<T>(a.ws.ku_p, bh, a.s.Lp, HD);
   const T* tb = reinterpret_cast<const T*>(a.ws.t_blk) + (int64_t)bh * a.s.Lp * kNB;
   const T* snap = reinterpret_cast<const T*>(a.ws.usnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
 
   frag<T> fqc[KS], fku[KS], ft[kNB / 16];   // c1 Qc rows, -c1 Ku rows, T' rows of this wave
 #pragma unroll
   for (int s = 0; s < KS; ++s) {
-    fqc[s] = ldg_nat_scaled<T, TI>(qc, a.qc.sl, i, 16 * s + 8 * g, i < L, c1);
-    fku[s] = ldg_nat_scaled<T, TI>(ku, a.ku.sl, i, 16 * s + 8 * g, i < L, -c1);
+    fqc[s] = ldg_nat<T>(qc, HD, i, 16 * s + 8 * g, true);
+    fku[s] = ldg_nat_scaled<T, T>(ku, HD, i, 16 * s + 8 * g, true, -c1);
   }
 #pragma unroll
   for (int s = 0; s < kNB / 16; ++s) ft[s] = ldg_nat<T>(tb, kNB, i, 16 * s + 8 * g, s < nintra);
@@ -226,13 +262,13 @@ __global__ __launch_bounds__(kThreads, (sizeof(T) == 2 && HD <= 64) ? 2 : 1) voi
   int nchunks = (qb * QB + QB) / kNB;
   if (nchunks > a.s.nblk) nchunks = a.s.nblk;
 
-  RowStage<T, TI, kNB, HD> pkc, pqu;
-  ColStage<T, TI, kNB, HD> pvc;
+  RowStage<T, T, kNB, HD> pkc, pqu;
+  ColStage<T, T, kNB, HD> pvc;
   SnapStage<T, kNB, HD> pub[NBLK_Q];
   auto load_chunk = [&](int Kb) __attribute__((always_inline)) {
-    pkc.load(kc, a.kc.sl, (int64_t)Kb * kNB, L);
-    pvc.load(vc, a.vc.sl, (int64_t)Kb * kNB, L);
-    pqu.load(qu, a.qu.sl, (int64_t)Kb * kNB, L);
+    pkc.load(kc, HD, (int64_t)Kb * kNB, kNoRowLimit);
+    pvc.load(vc, HD, (int64_t)Kb * kNB, kNoRowLimit);
+    pqu.load(qu, HD, (int64_t)Kb * kNB, kNoRowLimit);
 #pragma unroll
     for (int q = 0; q < NBLK_Q; ++q) {
       const int blk = Ifirst + q;
@@ -368,6 +404,8 @@ template <typename T, typename TI, int HD> static int launch_fwd_t(const FwdArgs
   }
   {
     ProfScope ps(kSlotTqv, stream);
+    constexpr int PIECES_PER_ROW = HD / elem_traits<T>::vec16;
+    hipLaunchKernelGGL((prep_kernel<T, TI, HD>), dim3((a.s.Lp * PIECES_PER_ROW + kThreads - 1) / kThreads, BH, 6), dim3(kThreads), 0, stream, a);
     hipLaunchKernelGGL((tqv_kernel<T, TI, HD>), dim3(a.s.nblk, BH), dim3(kThreads), 0, stream, a);
   }
   {

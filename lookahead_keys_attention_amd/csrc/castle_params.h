@@ -23,6 +23,10 @@ struct FwdWorkspace {
   void* tt_blk;   // [B*H][Lp][kNB]  T^T per block: [j][i_local]
   void* usnap;    // [B*H][snap_rows(nblk)][d]  forward state at block starts
   float* lse;     // [B*H][Lp] natural-log softmax normaliser
+  // The six operands in the compute type, each [B*H][Lp][d] contiguous, rows >= L zero
+  // (written by the prep kernel; every other kernel reads these instead of the caller's tensors).
+  // qc_p is pre-multiplied by scale * log2(e).
+  void *qc_p, *kc_p, *vc_p, *qu_p, *ku_p, *vu_p;
 };
 
 struct FwdArgs {
@@ -44,6 +48,7 @@ struct BwdArgs {
   // operands, d <= 64 only, else nullptr): per head (Lp/32)^2 tiles of 32 keys x 32 queries,
   // tile (kt, it) at ((kt * (Lp/32) + it) * 1024 elements; only tiles with kt <= it are written.
   // Inside a tile, element (key k, query i) sits at (i / 16) * 512 + k * 16 + i % 16.
+  void* dout_p;   // [B*H][Lp][d]  dO in the compute type, rows >= L zero (written by the delta kernel)
   void* ds_mat;   // dS
   void* dsu_mat;  // dSu
 };

@@ -29,6 +29,7 @@ template <typename T> using vec4_mem = vec<T, 4> __attribute__((aligned(8)));
 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
+constexpr int64_t kNoRowLimit = (int64_t)1 << 40;   // row_end of staging loads from padded arrays
 constexpr int kNB = 64;        // block size of the state snapshots (rows per block)
 constexpr int kThreads = 256;  // 4 waves per workgroup in every tiled kernel
 constexpr int kMaxLds = 160 * 1024;
@@ -516,6 +517,11 @@ struct SnapStage {
     }
   }
 };
+
+// head bh of an operand copy in the compute type ([B*H][Lp][HD] contiguous, rows >= L zero)
+template <typename T> __device__ __forceinline__ const T* prep_ptr(const void* base, int bh, int Lp, int HD) {
+  return reinterpret_cast<const T*>(base) + (int64_t)bh * Lp * HD;
+}
 
 // offsets (in rows) of block I inside the snapshot arrays
 __host__ __device__ inline int64_t usnap_off(int64_t I) { return (int64_t)kNB * I * (I - 1) / 2; }   // I >= 1, I*kNB rows
