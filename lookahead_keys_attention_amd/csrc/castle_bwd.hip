@@ -432,11 +432,11 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_key2_kernel(BwdArgs a) {
 #define CASTLE_BK2_STAGE_LOAD(I_)                            \
   do {                                                       \
     const int64_t r_ = (int64_t)(I_) * kNB;                  \
-    pku.load(ku, HD, r_, kNoRowLimit);                            \
-    pqc.load(qc, HD, r_, kNoRowLimit);                            \
-    pdo.load(dout, HD, r_, kNoRowLimit);                        \
-    pvu.load(vu, HD, r_, kNoRowLimit);                            \
-    ptb.load(tb, kNB, r_, (int64_t)1 << 40);                 \
+    pku.load_flat(ku + r_ * HD);                             \
+    pqc.load_flat(qc + r_ * HD);                             \
+    pdo.load_flat(dout + r_ * HD);                           \
+    pvu.load_flat(vu + r_ * HD);                             \
+    ptb.load_flat(tb + r_ * kNB);                            \
     if (threadIdx.x < kNB) {                                 \
       const int64_t i_ = r_ + threadIdx.x;                   \
       plse = i_ < L ? lse[i_] : INFINITY;                    \
@@ -517,6 +517,11 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_key2_kernel(BwdArgs a) {
       const bool active = I >= Iw;
       const bool inter = I > Iw;   // lookahead state from earlier blocks exists
       CASTLE_BK2_STAGE_STORE();
+      // The staged pieces were the oldest loads in flight, so the lookahead state requested after
+      // them has arrived too; pin that here, or the wait for it would land behind the loads of
+      // the next block, which are issued below.
+#pragma unroll
+      for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(fub[s]));
       __syncthreads();   // 1: tiles staged
       if (I > I0) CASTLE_BK2_STAGE_LOAD(I - 1);   // in flight for the whole block
 #pragma unroll
@@ -1176,8 +1181,8 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
     SnapStage<T, kCK, HD> pu0;
 #define CASTLE_BQ2_LOAD_A(K0)                                                            \
   do {                                                                                   \
-    pkc.load(kc, HD, (K0), kNoRowLimit, tid);                                                 \
-    pqu.load(qu, HD, (K0), kNoRowLimit, tid);                                                 \
+    pkc.load_flat(kc + (int64_t)(K0) * HD, tid);                                         \
+    pqu.load_flat(qu + (int64_t)(K0) * HD, tid);                                         \
     if ((K0) / kNB < blk0) pu0.load(usnap + (usnap_off(blk0) + (K0)) * HD, tid);         \
     pds.load(dsm + (int64_t)((K0) / 32) * tile_row);                                     \
     pdsu.load(dsum + (int64_t)((K0) / 32) * tile_row);                                   \

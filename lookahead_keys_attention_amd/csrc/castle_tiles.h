@@ -259,6 +259,16 @@ struct RowStage {
         r[n] = *reinterpret_cast<const vec<TI, V>*>(src + (row0 + v / VPR) * row_stride + (v % VPR) * V);
     }
   }
+  // Same for a tile whose ROWS rows of COLS elements are contiguous in memory and all exist (the
+  // operand copies in the compute type): piece v of the tile sits at tile + v * V.
+  __device__ __forceinline__ void load_flat(const TI* tile, int tid = threadIdx.x) {
+    static_assert(TOTAL % THREADS == 0 || TOTAL < THREADS, "tile must split evenly over the threads");
+#pragma unroll
+    for (int n = 0; n < N; ++n) {
+      const int v = tid + n * THREADS;
+      if (TOTAL >= THREADS || v < TOTAL) r[n] = *reinterpret_cast<const vec<TI, V>*>(tile + v * V);
+    }
+  }
   __device__ __forceinline__ void store(T* dst, int ld, int tid = threadIdx.x) const {
 #pragma unroll
     for (int n = 0; n < N; ++n) {
