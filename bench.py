@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the CASTLE hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-decode] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-decode] [--no-lm] [--no-cpu]
 
 Workload (BASELINE config 2): one Castle layer (dim 512, 8 heads, dim_head 64), bf16,
 x and the upstream gradient ~ N(0,1) of shape (4, 4096, 512), seeded random-init weights;
@@ -12,6 +12,8 @@ HBM.  Prints ONE JSON line:
   roofline     the longest-running kernel against the bf16 MFMA peak (2.5 PFLOP/s)
   decode       BASELINE config 4 (B32, prefill 2048, 512 cached steps): tokens/s and the decode
                stream kernel against the HBM peak (8 TB/s)
+  lm           BASELINE config 5 (12 x [Castle + MLP], tied embedding, (16, 1024) tokens, bf16): one
+               forward + loss + backward, and greedy generation through prefill + cached decode
   cpu_baseline the CPU oracle (dense PyTorch restatement of the reference's non-Triton path)
                on a bounded sample of the same workload, host cores stated
 """
@@ -150,6 +152,47 @@ def bench_decode(n_steps=512, prefill=2048):
     return out
 
 
+def bench_lm(steps=5, warmup=2):
+    import torch
+
+    from lookahead_keys_attention_amd import CastleLM
+
+    dev = torch.device("cuda:0")
+    B, n, depth, dim, H, d = 16, 1024, 12, 512, 8, 64
+    torch.manual_seed(0)
+    model = CastleLM(num_tokens=256, dim=dim, depth=depth, heads=H, dim_head=d, use_triton=True,
+                     tie_embedding=True).to(dev).bfloat16()
+    x = torch.randint(0, 256, (B, n + 1), generator=torch.Generator().manual_seed(0)).to(dev)
+
+    def step():
+        model.zero_grad(set_to_none=True)
+        model(x, return_loss=True).backward()
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    core = 19.0 * B * H * float(n) * n * d * depth
+    # generation: 16 prompts of 512 tokens, 128 new tokens each, every layer on its own cache
+    prompt = x[:, :512]
+    model.eval()
+    model.sample(prompt, 512 + 8, temperature=0.0)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    model.sample(prompt, 512 + 128, temperature=1.0)
+    torch.cuda.synchronize()
+    gen_s = time.perf_counter() - t0
+    return {"workload": "config 5: 12 x [Castle(512, 8 heads, 64) + MLP], tied embedding, rotary, prenorm, tokens (16, 1024), bf16",
+            "ms_per_step": round(ms, 3), "tokens_per_s": round(B * n / (ms * 1e-3), 1),
+            "attention_core_tflops_lower_bound": round(core / (ms * 1e-3) / 1e12, 2),
+            "generate_tokens_per_s": round(B * 128 / gen_s, 1),
+            "generate": "16 prompts x 512 tokens pre-filled, 128 sampled tokens each (top-k 0.9, temperature 1)"}
+
+
 def cpu_baseline(budget_s=20.0):
     """Dense oracle (fp32, autograd backward) on single heads of config 2, as many as fit the budget."""
     import torch
@@ -187,6 +230,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-lm", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device-to-device copy four times (reference for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters to bytes)")
@@ -237,6 +281,8 @@ def main():
     }
     if not args.no_decode:
         line["decode"] = bench_decode()
+    if not args.no_lm:
+        line["lm"] = bench_lm()
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline()
     print(json.dumps(line))

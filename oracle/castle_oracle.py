@@ -20,6 +20,9 @@ How each function is pinned (tests/test_oracle_*.py):
                      and expose its intermediate tensors).
   module_forward     the reference's own test properties (parallel == cached
                      sequential, causality) with default-initialised weights.
+  lm_forward         composition of module_forward with library routines (embedding,
+                     rms_norm, gelu, cross_entropy): parallel == cached sequential,
+                     causality, and loss = ln(vocabulary) for zero logits weights.
 Rotary embedding (LKA:71-73,106-112) depends on a third-party package that is
 not present; it is not restated here: parity unpinned for rotary_emb=True.
 """
@@ -141,6 +144,35 @@ def module_forward(x, params, heads, cache=None, return_next_cache=None):
     B, H = o.shape[0], o.shape[1]
     y = o.permute(0, 2, 1, 3).reshape(B, n, H * d) @ w_out.t()   # LKA:207-209
     return (y, nxt) if return_next_cache else y                  # LKA:211-214
+
+
+def lm_forward(tokens, params, heads, depth, return_loss=False, cache=None, return_next_cache=False):
+    """Functional restatement of the reference's language model around the layer
+    (train_triton.py:141-175), without rotary: embedding, `depth` x [h += castle(h); h += ff(h)]
+    with ff = RMSNorm, Linear(4x), GELU, Linear (train_triton.py:103-108), final RMSNorm, logits,
+    and the shift-by-one cross entropy (train_triton.py:143-144,172-175).
+    params: state-dict style keys of the module tree (token_emb.weight, layers.<i>.0.<castle key>,
+    layers.<i>.1.{0,1,3}.weight, final_norm.weight, to_logits.weight)."""
+    if return_loss:
+        tokens, target = tokens[:, :-1], tokens[:, 1:]
+    h = params["token_emb.weight"][tokens]
+    nxt = []
+    for i in range(depth):
+        layer = {k[len(f"layers.{i}.0."):]: v for k, v in params.items() if k.startswith(f"layers.{i}.0.")}
+        layer_cache = cache[i] if cache is not None else None
+        if return_next_cache:
+            y, c = module_forward(h, layer, heads, cache=layer_cache, return_next_cache=True)
+            nxt.append(c)
+        else:
+            y = module_forward(h, layer, heads, cache=layer_cache, return_next_cache=False)
+        h = h + y
+        f = F.rms_norm(h, (h.shape[-1],), params[f"layers.{i}.1.0.weight"])
+        f = F.gelu(f @ params[f"layers.{i}.1.1.weight"].t()) @ params[f"layers.{i}.1.3.weight"].t()
+        h = h + f
+    logits = F.rms_norm(h, (h.shape[-1],), params["final_norm.weight"]) @ params["to_logits.weight"].t()
+    if return_loss:
+        return F.cross_entropy(logits.transpose(1, 2), target)
+    return (logits, nxt) if return_next_cache else logits
 
 
 # --------------------------------------------------------------------------

@@ -1,0 +1,169 @@
+"""The language model around the layer and its sampler (reference: train_triton.py:56-175).
+
+CPU tests pin the oracle's lm_forward (causality, parallel == cached, a closed-form loss) and check
+the product's dense PyTorch formulation and sampling helpers against it; GPU tests compare the
+native path (HIP prefill + cached decode) with the oracle.
+"""
+import math
+
+import pytest
+import torch
+
+from lookahead_keys_attention_amd.lm import CastleLM, gumbel_sample, top_k
+from oracle import castle_oracle as O
+
+VOCAB = 256
+
+
+def make_lm(depth=2, dim=64, heads=2, dim_head=16, rotary=False, native=False, tie=False, seed=0):
+    torch.manual_seed(seed)
+    return CastleLM(num_tokens=VOCAB, dim=dim, depth=depth, heads=heads, dim_head=dim_head,
+                    use_triton=native, rotary_emb=rotary, prenorm=True, tie_embedding=tie)
+
+
+def params_of(model):
+    return {k: v.detach().double().cpu() for k, v in model.state_dict().items()}
+
+
+def tokens(B, n, seed=1):
+    return torch.randint(0, VOCAB, (B, n), generator=torch.Generator().manual_seed(seed))
+
+
+# ---------------------------------------------------------------- oracle pins
+def test_oracle_lm_is_causal_and_cached_equals_parallel():
+    model = make_lm()
+    p = params_of(model)
+    x = tokens(2, 12)
+    full = O.lm_forward(x, p, heads=2, depth=2)
+    assert full.shape == (2, 12, VOCAB)
+    x2 = x.clone()
+    x2[:, 8:] = (x2[:, 8:] + 7) % VOCAB
+    assert torch.allclose(O.lm_forward(x2, p, 2, 2)[:, :8], full[:, :8], atol=1e-12)   # causality
+    logits, cache = O.lm_forward(x[:, :5], p, 2, 2, return_next_cache=True)
+    steps = [logits[:, -1]]
+    for t in range(5, 12):
+        logits, cache = O.lm_forward(x[:, t:t + 1], p, 2, 2, cache=cache, return_next_cache=True)
+        steps.append(logits[:, -1])
+    assert torch.allclose(torch.stack(steps, 1), full[:, 4:], atol=1e-10)
+
+
+def test_oracle_lm_loss_is_log_vocab_for_zero_logits():
+    model = make_lm()
+    p = params_of(model)
+    p["to_logits.weight"] = torch.zeros_like(p["to_logits.weight"])
+    loss = O.lm_forward(tokens(2, 9), p, 2, 2, return_loss=True)
+    assert abs(loss.item() - math.log(VOCAB)) < 1e-12
+
+
+# ---------------------------------------------------------------- host logic
+def test_top_k_keeps_the_largest_fraction():
+    logits = torch.randn(3, 50, generator=torch.Generator().manual_seed(0))
+    kept = top_k(logits, thres=0.9)
+    assert (kept > float("-inf")).sum(-1).tolist() == [5, 5, 5]          # ceil(0.1 * 50)
+    assert torch.equal(kept.max(-1).values, logits.max(-1).values)
+    assert torch.equal(kept[kept > float("-inf")].sort().values, logits.topk(5).values.flatten().sort().values)
+
+
+def test_gumbel_sample_draws_from_the_softmax():
+    logits = torch.tensor([1.0, 0.0, -1.0, 2.0])
+    g = torch.Generator().manual_seed(0)
+    draws = gumbel_sample(logits.expand(40000, 4), temperature=1.0, generator=g).flatten()
+    freq = torch.bincount(draws, minlength=4).double() / draws.numel()
+    assert torch.allclose(freq, logits.double().softmax(0), atol=0.01)
+    cold = gumbel_sample(logits.expand(100, 4), temperature=1e-6, generator=g).flatten()
+    assert torch.all(cold == 3)
+
+
+@pytest.mark.parametrize("tie", [False, True])
+def test_dense_model_matches_oracle(tie):
+    model = make_lm(tie=tie).double()
+    p = params_of(model)
+    x = tokens(2, 17)
+    assert torch.allclose(model(x), O.lm_forward(x, p, 2, 2), atol=1e-10)
+    loss = model(x, return_loss=True)
+    assert torch.allclose(loss, O.lm_forward(x, p, 2, 2, return_loss=True), atol=1e-10)
+    if not tie:   # near-uniform prediction at initialisation (a tied N(0,1) embedding gives large logits)
+        assert abs(loss.item() - math.log(VOCAB)) < 0.5
+    assert (model.to_logits.weight is model.token_emb.weight) == tie
+
+
+def test_dense_model_with_rotary_cached_equals_parallel():
+    model = make_lm(rotary=True).double()
+    x = tokens(2, 14)
+    full = model(x)
+    logits, cache = model(x[:, :6], return_next_cache=True)
+    steps = [logits[:, -1]]
+    for t in range(6, 14):
+        logits, cache = model(x[:, t:t + 1], cache=cache, return_next_cache=True)
+        steps.append(logits[:, -1])
+    assert len(cache) == 2 and cache[0].kc_cache.shape[-2] == 14
+    assert torch.allclose(torch.stack(steps, 1), full[:, 5:], atol=1e-9)
+
+
+def test_sample_is_a_greedy_rollout_at_zero_temperature():
+    model = make_lm().double()
+    prompt = tokens(2, 5)
+    new = model.sample(prompt, seq_len=11, temperature=0.0)
+    assert new.shape == (2, 6)
+    seq = prompt
+    for _ in range(6):
+        seq = torch.cat((seq, model(seq)[:, -1].argmax(-1, keepdim=True)), dim=-1)
+    assert torch.equal(new, seq[:, 5:])
+    g1, g2 = torch.Generator().manual_seed(3), torch.Generator().manual_seed(3)
+    assert torch.equal(model.sample(prompt, 9, generator=g1), model.sample(prompt, 9, generator=g2))
+    assert model.sample(prompt, 5).shape == (2, 0)
+
+
+# ---------------------------------------------------------------- native path
+@pytest.mark.gpu
+def test_native_model_matches_oracle_forward_and_backward():
+    model = make_lm(depth=2, dim=128, heads=2, dim_head=64, native=True).cuda()
+    p = params_of(model)
+    x = tokens(2, 150)
+    logits = model(x.cuda())
+    ref = O.lm_forward(x, p, 2, 2)
+    assert (logits.cpu().double() - ref).abs().max() <= 1e-3
+    loss = model(x.cuda(), return_loss=True)
+    loss.backward()
+    leaves = {k: v.clone().requires_grad_() for k, v in p.items()}
+    ref_loss = O.lm_forward(x, leaves, 2, 2, return_loss=True)
+    ref_loss.backward()
+    assert abs(loss.item() - ref_loss.item()) <= 1e-4
+    for name, param in model.named_parameters():
+        got, want = param.grad.cpu().double(), leaves[name].grad
+        assert (got - want).abs().max() <= 2e-2 * max(want.abs().max().item(), 1e-6) + 1e-6, name
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rotary", [False, True])
+def test_native_sampler_follows_the_parallel_logits(rotary):
+    """Greedy generation through HIP prefill + cached decode steps across layers: every token it
+    picks must be (within rounding) the arg-max of the logits a full parallel pass assigns."""
+    model = make_lm(depth=3, dim=128, heads=2, dim_head=64, rotary=rotary, native=True).cuda()
+    prompt = tokens(2, 37)
+    new = model.sample(prompt.cuda(), seq_len=37 + 20, temperature=0.0).cpu()
+    assert new.shape == (2, 20)
+    seq = torch.cat((prompt, new), dim=-1)
+    if rotary:      # no oracle for rotary: the product's dense formulation on the CPU is the comparison
+        dense = make_lm(depth=3, dim=128, heads=2, dim_head=64, rotary=True, native=False)
+        dense.load_state_dict(model.state_dict())
+        ref = dense.double()(seq)
+    else:
+        ref = O.lm_forward(seq, params_of(model), 2, 3)
+    at_pick = ref[:, 36:-1].gather(-1, new.unsqueeze(-1)).squeeze(-1)
+    assert torch.all(ref[:, 36:-1].max(-1).values - at_pick <= 2e-3)
+
+
+@pytest.mark.gpu
+def test_config5_language_model_step_bf16():
+    """BASELINE config 5: 12 x [Castle(512, 8 heads, 64) + MLP], tied embedding, (16, 1024) tokens,
+    forward + loss + backward."""
+    torch.manual_seed(0)
+    model = CastleLM(num_tokens=VOCAB, dim=512, depth=12, heads=8, dim_head=64, use_triton=True,
+                     tie_embedding=True).cuda().bfloat16()
+    x = tokens(16, 1025).cuda()
+    loss = model(x, return_loss=True)
+    loss.backward()
+    assert math.isfinite(loss.item())
+    for name, param in model.named_parameters():
+        assert param.grad is not None and torch.isfinite(param.grad).all(), name
