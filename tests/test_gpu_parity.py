@@ -66,6 +66,7 @@ BWD_CASES = [
     (1, 2, 200, 32, torch.float32), (1, 2, 321, 64, torch.float32), (2, 2, 384, 64, torch.bfloat16),
     (1, 2, 300, 32, torch.bfloat16), (1, 2, 256, 16, torch.bfloat16), (1, 2, 256, 64, torch.float16),
     (1, 2, 300, 128, torch.bfloat16), (1, 1, 130, 128, torch.float16),
+    (1, 3, 129, 16, torch.bfloat16), (3, 1, 448, 64, torch.float16), (1, 9, 640, 64, torch.bfloat16),
 ]
 
 
@@ -80,6 +81,25 @@ def test_operator_backward(B, Hh, L, d, dtype):
         assert_close(leaf.grad, r, dtype, name, 2e-2)
         if dtype == torch.float32:      # far inside the bound in practice
             assert (leaf.grad.cpu().double() - r).abs().max() <= 1e-4, name
+
+
+@pytest.mark.parametrize("L,d", [(256, 64), (200, 32)])
+def test_bf16_operand_flag_forward_and_backward(L, d, monkeypatch):
+    """CASTLE_FLAG_BF16_OPERANDS keeps bf16 MFMA operands (default: fp16 operands for bf16 tensors)."""
+    from lookahead_keys_attention_amd import _native
+
+    monkeypatch.setattr(H(), "DEFAULT_FLAGS", _native.FLAG_BF16_OPERANDS)
+    ops, dout = rand_ops(2, 2, L, d, torch.bfloat16, seed=L + 7 * d)
+    s = d ** -0.5
+    leaves = [t.to(DEV).requires_grad_() for t in ops]
+    out, U = H().castle_attention_hip(*leaves, s, True)
+    out.backward(dout.to(DEV))
+    ref_out, ref_U = O.parallel_core(*[t.double() for t in ops], s, want_U=True)
+    assert_close(out, ref_out, torch.bfloat16, "out", 1e-3)
+    assert_close(U, ref_U, torch.bfloat16, "U", 1e-3)
+    ref = O.closed_form_grads(*[t.double() for t in ops], s, dout.double())
+    for name, leaf, r in zip(NAMES, leaves, ref):
+        assert_close(leaf.grad, r, torch.bfloat16, name, 2e-2)
 
 
 def test_lookahead_keys_carry_no_gradient():
