@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define CASTLE_ABI_VERSION 1
+#define CASTLE_ABI_VERSION 2
 
 /* element types of the tensors (accumulation is always fp32) */
 #define CASTLE_F32 0
@@ -33,8 +33,14 @@ extern "C" {
  * loaded (exact for |x| < 65504) and every operand the kernels produce internally is fp16:
  * same MFMA rate, 3 more mantissa bits, which keeps the gradients of long sequences inside the
  * bf16 tolerance.  CASTLE_FLAG_BF16_OPERANDS keeps bf16 MFMA operands instead (full bf16 range).
- * castle_bwd must get the same flags as the castle_fwd call whose workspace it reads. */
+ * castle_bwd must get the same flags as the castle_fwd call whose workspace it reads.
+ * CASTLE_FLAG_ROTARY: the kernels rotate qc, kc, qu, ku, vu (not vc) by their row position
+ * (rotary position embedding over interleaved pairs, base 10000: what Castle(rotary_emb=True) does
+ * before its core, lookahead_keys_attention.py:106-112); castle_bwd then returns the gradients with
+ * respect to the un-rotated operands; castle_decode_step rotates the new token by position t and
+ * appends the rotated qu, kc rows.  The final lookahead keys U are those of the rotated operands. */
 #define CASTLE_FLAG_BF16_OPERANDS 1
+#define CASTLE_FLAG_ROTARY 2
 
 /* error codes */
 #define CASTLE_OK 0
@@ -103,14 +109,20 @@ int64_t castle_decode_workspace_bytes(int B, int H, int d, int t_max);
  * writes row t of all four (U_t = 0, qu, kc, vc of the new token) and writes
  * out (B,H,1,d) = softmax_k(s qc.kc_k - silu(s qc.U_k)) vc_k over k = 0..t.
  * qc..vu: the new token's (B,H,1,d) operands (stride_l unused).  After the call the cache
- * holds t+1 rows.  d in {16,32,64,128}. */
+ * holds t+1 rows.  d in {16,32,64,128}.  flags: 0 or CASTLE_FLAG_ROTARY. */
 int castle_decode_step(const castle_view4* U, const castle_view4* qu_cache,
                        const castle_view4* kc_cache, const castle_view4* vc_cache, int t,
                        const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
                        const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
-                       int B, int H, int d, int dtype, float scale,
+                       int B, int H, int d, int dtype, float scale, int flags,
                        const castle_view4* out,
                        void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Rotary position embedding of one tensor, out of place: out[b,h,l,:] = R(first_position + l) x[b,h,l,:]
+ * (the rotation CASTLE_FLAG_ROTARY applies inside the kernels; lookahead_keys_attention.py:112).  Used to
+ * fill the qu / kc rows of a decode cache after a rotary prefill. */
+int castle_rope(const castle_view4* x, const castle_view4* out, int B, int H, int L, int d, int dtype,
+                int first_position, void* stream);
 
 /* Per-kernel timing (no counterpart in the reference; for benchmarks).  While enabled, every
  * kernel launched by the entry points above is bracketed by a HIP event pair on its stream.

@@ -141,24 +141,20 @@ class Castle(nn.Module):
         store = None
         if want_cache:
             store = _CacheStore(B, H, d, _reserve_rows(n), proj.dtype, proj.device)
-        if not self.rotary_emb:
-            U_view = store.buffers[0][:, :, :n] if want_cache else None
-            res = ops.castle_attention_packed(proj, H, self.scale, want_cache, U_view)
-            merged = res[0] if want_cache else res
-            qu, _, _, _, kc, vc = self._split(proj)
-        else:
-            qu, ku, vu, qc, kc, vc = self._split(proj)
-            qc, kc, qu, ku, vu = self._rotate((qc, kc, qu, ku, vu), 0, n, proj.device)
-            res = ops.castle_attention_hip(qc, kc, vc, qu, ku, vu, self.scale, want_cache)
-            o = res[0] if want_cache else res
-            merged = o.permute(0, 2, 1, 3).reshape(B, n, H * d)
-            if want_cache:
-                store.buffers[0][:, :, :n].copy_(res[1])
+        U_view = store.buffers[0][:, :, :n] if want_cache else None
+        res = ops.castle_attention_packed(proj, H, self.scale, want_cache, U_view, rotary=self.rotary_emb)
+        merged = res[0] if want_cache else res
+        qu, _, _, _, kc, vc = self._split(proj)
         if not want_cache:
             return merged, None
         with torch.no_grad():
-            for buf, src in zip(store.buffers[1:], (qu, kc, vc)):
-                buf[:, :, :n].copy_(src)
+            if self.rotary_emb:   # the cache holds the rotated qu / kc rows
+                ops.castle_rope_hip(qu, store.buffers[1][:, :, :n])
+                ops.castle_rope_hip(kc, store.buffers[2][:, :, :n])
+            else:
+                store.buffers[1][:, :, :n].copy_(qu)
+                store.buffers[2][:, :, :n].copy_(kc)
+            store.buffers[3][:, :, :n].copy_(vc)
         store.length = n
         return merged, store.as_cache()
 
@@ -179,13 +175,11 @@ class Castle(nn.Module):
             raise RuntimeError("this cache was already advanced by a later decode step; the native "
                                "decode updates its cache in place, so a cache can be used once")
         t = store.length
-        if self.rotary_emb:
-            qc, kc, qu, ku, vu = self._rotate((qc, kc, qu, ku, vu), t, 1, proj.device)
         if t + 1 > store.capacity:
             store = store.grown(_reserve_rows(t + 1))
         out = torch.empty((B, 1, H, d), dtype=proj.dtype, device=proj.device)
         ops.castle_decode_step_hip(*store.buffers, t, qc, kc, vc, qu, ku, vu, self.scale,
-                                   out.permute(0, 2, 1, 3), store.workspace)
+                                   out.permute(0, 2, 1, 3), store.workspace, rotary=self.rotary_emb)
         store.length = t + 1
         return out.view(B, 1, H * d), store.as_cache()
 

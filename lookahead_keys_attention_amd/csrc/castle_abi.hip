@@ -12,6 +12,7 @@ namespace castle {
 int launch_fwd(const FwdArgs& a, int dtype, bool bf16_operands, hipStream_t stream);
 int launch_bwd(const BwdArgs& a, int dtype, bool bf16_operands, hipStream_t stream);
 int launch_decode(const DecodeArgs& a, int dtype, hipStream_t stream);
+int launch_rope(const View4& src, const View4& dst, int B, int H, int L, int d, int dtype, int pos0, hipStream_t stream);
 int decode_pick_splits(int BH, int t);
 }  // namespace castle
 
@@ -146,6 +147,7 @@ int castle_fwd(const castle_view4* qc, const castle_view4* kc, const castle_view
 
   castle::FwdArgs a;
   a.s.B = B; a.s.H = H; a.s.L = L; a.s.d = d; a.s.Lp = g.Lp; a.s.nblk = g.nblk; a.s.scale = scale;
+  a.s.rotary = (flags & CASTLE_FLAG_ROTARY) != 0;
   a.qc = to_view(qc); a.kc = to_view(kc); a.vc = to_view(vc);
   a.qu = to_view(qu); a.ku = to_view(ku); a.vu = to_view(vu);
   a.out = to_view(out);
@@ -184,6 +186,7 @@ int castle_bwd(const castle_view4* qc, const castle_view4* kc, const castle_view
 
   castle::BwdArgs a;
   a.s.B = B; a.s.H = H; a.s.L = L; a.s.d = d; a.s.Lp = g.Lp; a.s.nblk = g.nblk; a.s.scale = scale;
+  a.s.rotary = (flags & CASTLE_FLAG_ROTARY) != 0;
   a.qc = to_view(qc); a.kc = to_view(kc); a.vc = to_view(vc);
   a.qu = to_view(qu); a.ku = to_view(ku); a.vu = to_view(vu);
   a.out = to_view(out); a.dout = to_view(dout);
@@ -207,7 +210,7 @@ int castle_decode_step(const castle_view4* U, const castle_view4* qu_cache,
                        const castle_view4* kc_cache, const castle_view4* vc_cache, int t,
                        const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
                        const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
-                       int B, int H, int d, int dtype, float scale,
+                       int B, int H, int d, int dtype, float scale, int flags,
                        const castle_view4* out,
                        void* workspace, int64_t workspace_bytes, void* stream) {
   const int es = elem_size(dtype);
@@ -225,6 +228,7 @@ int castle_decode_step(const castle_view4* U, const castle_view4* qu_cache,
 
   castle::DecodeArgs a;
   a.B = B; a.H = H; a.d = d; a.t = t; a.scale = scale;
+  a.rotary = (flags & CASTLE_FLAG_ROTARY) != 0;
   a.splits = castle::decode_pick_splits(B * H, t);
   a.U = to_view(U); a.qu_cache = to_view(qu_cache); a.kc_cache = to_view(kc_cache); a.vc_cache = to_view(vc_cache);
   a.qc = to_view(qc); a.kc = to_view(kc); a.vc = to_view(vc);
@@ -232,6 +236,15 @@ int castle_decode_step(const castle_view4* U, const castle_view4* qu_cache,
   a.out = to_view(out);
   a.part = static_cast<float*>(workspace);
   return castle::launch_decode(a, dtype, static_cast<hipStream_t>(stream));
+}
+
+int castle_rope(const castle_view4* x, const castle_view4* out, int B, int H, int L, int d, int dtype,
+                int first_position, void* stream) {
+  const int es = elem_size(dtype);
+  if (es == 0) return CASTLE_ERR_DTYPE;
+  if (B <= 0 || H <= 0 || L <= 0 || first_position < 0 || !head_dim_ok(d) || (int64_t)B * H > 65535) return CASTLE_ERR_SHAPE;
+  if (!view_ok(x, es, true) || !view_ok(out, es, true)) return CASTLE_ERR_ARG;
+  return castle::launch_rope(to_view(x), to_view(out), B, H, L, d, dtype, first_position, static_cast<hipStream_t>(stream));
 }
 
 int castle_profile_enable(int on) { return castle::profile_enable(on); }

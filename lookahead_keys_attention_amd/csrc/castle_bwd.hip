@@ -47,10 +47,22 @@ struct Carver {
 constexpr int a16(int bytes) { return (bytes + 15) / 16 * 16; }
 
 // [n rows, lanes] accumulator tiles -> (row = lane index, 4 consecutive n) stores, scaled
+// Writes one gradient row held as accumulator tiles [n rows, this lane's row].  rope_pos >= 0: the
+// operand was rotated by that position before use, so its gradient is rotated back first.
 template <typename T, int HD, int NT>   // T: element type of the destination tensor
-__device__ __forceinline__ void store_rows(T* dst_row, acc_t (&acc)[NT], float mul, int g) {
+__device__ __forceinline__ void store_rows(T* dst_row, acc_t (&acc)[NT], float mul, int g, int rope_pos = -1) {
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
+    if (rope_pos >= 0) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = 32 * nt + 8 * q + 4 * g;
+        if (n < HD) {
+          CASTLE_ROPE_PAIR(acc[nt][4 * q], acc[nt][4 * q + 1], (float)rope_pos, n / 2, HD, true);
+          CASTLE_ROPE_PAIR(acc[nt][4 * q + 2], acc[nt][4 * q + 3], (float)rope_pos, n / 2 + 1, HD, true);
+        }
+      }
+    }
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[nt][r] *= mul;
 #pragma unroll
@@ -347,10 +359,10 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
 #undef CASTLE_BK_LOAD
   if (k < L) {
     if constexpr (DO_KV) {
-      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dkc, b, h) + (int64_t)k * a.dkc.sl, dkc, kLn2, g);
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dkc, b, h) + (int64_t)k * a.dkc.sl, dkc, kLn2, g, a.s.rotary ? k : -1);
       store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvc, b, h) + (int64_t)k * a.dvc.sl, dvc, 1.f, g);
     }
-    if constexpr (DO_QG) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqu, b, h) + (int64_t)k * a.dqu.sl, dqu, c0 * kLn2, g);
+    if constexpr (DO_QG) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqu, b, h) + (int64_t)k * a.dqu.sl, dqu, c0 * kLn2, g, a.s.rotary ? k : -1);
   }
 }
 
@@ -702,9 +714,9 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_key2_kernel(BwdArgs a) {
     if (I0 >= Iw) CASTLE_BK2_DQU(I0);
 #undef CASTLE_BK2_DQU
     if (k < L) {
-      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dkc, b, h) + (int64_t)k * a.dkc.sl, dkc, kLn2, g);
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dkc, b, h) + (int64_t)k * a.dkc.sl, dkc, kLn2, g, a.s.rotary ? k : -1);
       store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvc, b, h) + (int64_t)k * a.dvc.sl, dvc, 1.f, g);
-      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqu, b, h) + (int64_t)k * a.dqu.sl, dqu, c0 * kLn2, g);
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqu, b, h) + (int64_t)k * a.dqu.sl, dqu, c0 * kLn2, g, a.s.rotary ? k : -1);
     }
   }
 #undef CASTLE_BK2_STAGE_DECL
@@ -1046,10 +1058,10 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
       mma(dvu[nt], ld_free<T, false>(e_qcw, LDK, 32 * nt, HD, 16 * s, c, g), fdt);
   }
   if (i < L) {
-    if constexpr (DO_Q) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqc, b, h) + (int64_t)i * a.dqc.sl, dqc, c0, g);
+    if constexpr (DO_Q) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqc, b, h) + (int64_t)i * a.dqc.sl, dqc, c0, g, a.s.rotary ? i : -1);
     if constexpr (DO_S) {
-      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dku, b, h) + (int64_t)i * a.dku.sl, dku, c0 * kLn2, g);
-      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvu, b, h) + (int64_t)i * a.dvu.sl, dvu, kLn2, g);
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dku, b, h) + (int64_t)i * a.dku.sl, dku, c0 * kLn2, g, a.s.rotary ? i : -1);
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvu, b, h) + (int64_t)i * a.dvu.sl, dvu, kLn2, g, a.s.rotary ? i : -1);
     }
   }
 }
@@ -1282,8 +1294,8 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
         mma(dvu[nt], ld_free<T, false>(e_qcw, LDK, 32 * nt, HD, 16 * s, c, g), fdt);
     }
     if (i < L) {
-      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dku, b, h) + (int64_t)i * a.dku.sl, dku, c0 * kLn2, g);
-      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvu, b, h) + (int64_t)i * a.dvu.sl, dvu, kLn2, g);
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dku, b, h) + (int64_t)i * a.dku.sl, dku, c0 * kLn2, g, a.s.rotary ? i : -1);
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvu, b, h) + (int64_t)i * a.dvu.sl, dvu, kLn2, g, a.s.rotary ? i : -1);
     }
   } else {
     acc_t dqc[NT];     // [n rows, i lanes]
@@ -1384,7 +1396,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
           mma(dqc[nt], ld_free<T, true>(e_vuw, LDK, 32 * nt, HD, 32 * jt + 16 * s2, c, g), fdt);
       }
     }
-    if (i < L) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqc, b, h) + (int64_t)i * a.dqc.sl, dqc, c0, g);
+    if (i < L) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqc, b, h) + (int64_t)i * a.dqc.sl, dqc, c0, g, a.s.rotary ? i : -1);
   }
 }
 

@@ -54,6 +54,15 @@ __global__ __launch_bounds__(kThreads) void decode_stream_kernel(DecodeArgs a) {
   load_f32<T, V>(view_row<T>(a.ku, b, h, 0) + sub * V, ku);
   load_f32<T, V>(view_row<T>(a.vu, b, h, 0) + sub * V, vu);
   load_f32<T, V>(view_row<T>(a.qc, b, h, 0) + sub * V, qc);
+  if (a.rotary) {   // the new token sits at position t
+#pragma unroll
+    for (int e = 0; e < V / 2; ++e) {
+      const int pair = sub * (V / 2) + e;
+      CASTLE_ROPE_PAIR(ku[2 * e], ku[2 * e + 1], (float)a.t, pair, HD, false);
+      CASTLE_ROPE_PAIR(vu[2 * e], vu[2 * e + 1], (float)a.t, pair, HD, false);
+      CASTLE_ROPE_PAIR(qc[2 * e], qc[2 * e + 1], (float)a.t, pair, HD, false);
+    }
+  }
 
   float acc[V];
 #pragma unroll
@@ -169,11 +178,21 @@ __global__ __launch_bounds__(64) void decode_finish_kernel(DecodeArgs a) {
 #pragma unroll
   for (int e = 0; e < EPL; ++e) {
     const int n = lane + 64 * e;
+    float quv = n < HD ? (float)qu[n] : 0.f, kcv = n < HD ? (float)kc[n] : 0.f;
+    if (a.rotary) {   // element n and its pair partner n ^ 1 sit on neighbouring lanes
+      const float qup = __shfl_xor(quv, 1), kcp = __shfl_xor(kcv, 1);
+      const bool even = (n & 1) == 0;
+      float q0 = even ? quv : qup, q1 = even ? qup : quv, k0 = even ? kcv : kcp, k1 = even ? kcp : kcv;
+      CASTLE_ROPE_PAIR(q0, q1, (float)a.t, n / 2, HD, false);
+      CASTLE_ROPE_PAIR(k0, k1, (float)a.t, n / 2, HD, false);
+      quv = even ? q0 : q1;
+      kcv = even ? k0 : k1;
+    }
     if (n < HD) {
       out[n] = (T)(o[e] * inv);
       Ut[n] = (T)0.f;
-      qut[n] = qu[n];
-      kct[n] = kc[n];
+      qut[n] = (T)quv;
+      kct[n] = (T)kcv;
       vct[n] = vc[n];
     }
   }
@@ -207,6 +226,45 @@ int launch_decode(const DecodeArgs& a, int dtype, hipStream_t stream) {
     case 0: return launch_decode_d<float>(a, stream);
     case 1: return launch_decode_d<bf16_t>(a, stream);
     case 2: return launch_decode_d<fp16_t>(a, stream);
+    default: return -1;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Out-of-place rotary embedding of one (B, H, L, d) view: dst = R(pos0 + row) src.
+template <typename T, int HD>
+__global__ __launch_bounds__(kThreads) void rope_kernel(View4 src, View4 dst, int H, int L, int pos0) {
+  constexpr int V = elem_traits<T>::vec16;
+  constexpr int VPR = HD / V;
+  const int bh = blockIdx.y, b = bh / H, h = bh % H;
+  const int64_t piece = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  const int64_t row = piece / VPR;
+  const int cv = (int)(piece % VPR);
+  if (row >= L) return;
+  vec<float, V> f = __builtin_convertvector(*reinterpret_cast<const vec<T, V>*>(view_row<T>(src, b, h, row) + cv * V), vec<float, V>);
+#pragma unroll
+  for (int e = 0; e < V / 2; ++e) CASTLE_ROPE_PAIR(f[2 * e], f[2 * e + 1], (float)(pos0 + row), cv * (V / 2) + e, HD, false);
+  *reinterpret_cast<vec<T, V>*>(view_row<T>(dst, b, h, row) + cv * V) = __builtin_convertvector(f, vec<T, V>);
+}
+
+template <typename T> static int launch_rope_d(const View4& src, const View4& dst, int B, int H, int L, int d, int pos0, hipStream_t stream) {
+  const int pieces_per_row = d / elem_traits<T>::vec16;
+  const dim3 grid((unsigned)(((int64_t)L * pieces_per_row + kThreads - 1) / kThreads), B * H);
+  switch (d) {
+    case 16: hipLaunchKernelGGL((rope_kernel<T, 16>), grid, dim3(kThreads), 0, stream, src, dst, H, L, pos0); break;
+    case 32: hipLaunchKernelGGL((rope_kernel<T, 32>), grid, dim3(kThreads), 0, stream, src, dst, H, L, pos0); break;
+    case 64: hipLaunchKernelGGL((rope_kernel<T, 64>), grid, dim3(kThreads), 0, stream, src, dst, H, L, pos0); break;
+    case 128: hipLaunchKernelGGL((rope_kernel<T, 128>), grid, dim3(kThreads), 0, stream, src, dst, H, L, pos0); break;
+    default: return -2;
+  }
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+int launch_rope(const View4& src, const View4& dst, int B, int H, int L, int d, int dtype, int pos0, hipStream_t stream) {
+  switch (dtype) {
+    case 0: return launch_rope_d<float>(src, dst, B, H, L, d, pos0, stream);
+    case 1: return launch_rope_d<bf16_t>(src, dst, B, H, L, d, pos0, stream);
+    case 2: return launch_rope_d<fp16_t>(src, dst, B, H, L, d, pos0, stream);
     default: return -1;
   }
 }

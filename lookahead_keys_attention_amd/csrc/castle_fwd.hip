@@ -72,6 +72,10 @@ __global__ __launch_bounds__(kThreads) void prep_kernel(FwdArgs a) {
   for (int e = 0; e < V; ++e) f[e] = 0.f;
   if (row < a.s.L)
     f = __builtin_convertvector(*reinterpret_cast<const vec<TI, V>*>(head_ptr<TI>(src, b, h) + row * src.sl + cv * V), vec<float, V>);
+  if (a.s.rotary && blockIdx.z != 2) {   // every operand but Vc is rotated by its position
+#pragma unroll
+    for (int e = 0; e < V / 2; ++e) CASTLE_ROPE_PAIR(f[2 * e], f[2 * e + 1], (float)row, cv * (V / 2) + e, HD, false);
+  }
 #pragma unroll
   for (int e = 0; e < V; ++e) f[e] *= mul;
   T* dst = reinterpret_cast<T*>(dstv) + ((int64_t)bh * a.s.Lp + row) * HD + cv * V;

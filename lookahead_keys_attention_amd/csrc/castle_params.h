@@ -15,6 +15,7 @@ struct CoreShape {
   int Lp;     // L rounded up to 128
   int nblk;   // Lp / kNB
   float scale;
+  int rotary;   // 1: qc, kc, qu, ku, vu are rotated by their row position (RoPE) inside the kernels
 };
 
 // Workspace written by the forward pass and read again by the backward pass.
@@ -58,6 +59,7 @@ struct DecodeArgs {
   int t;            // rows already in the cache
   int splits;       // partitions of the t rows per (b, h)
   float scale;
+  int rotary;       // 1: the new token's qc, kc, qu, ku, vu are rotated by position t
   View4 U, qu_cache, kc_cache, vc_cache;   // capacity buffers, row t is appended
   View4 qc, kc, vc, qu, ku, vu;            // new token, L == 1
   View4 out;                               // (B, H, 1, d)

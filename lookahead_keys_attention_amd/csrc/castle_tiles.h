@@ -528,6 +528,29 @@ struct SnapStage {
   }
 };
 
+// Rotary position embedding over the interleaved pairs (x[2i], x[2i+1]) of a row of HD elements:
+// angle = pos * 10000^(-2i/HD) (lookahead_keys_attention.py:71-73,106-112 apply it to qc, kc, qu,
+// ku, vu through a third-party module; this is the standard form).  `inverse` rotates by the
+// opposite angle, which is the transpose: what the gradient of a rotated operand needs.
+__device__ __forceinline__ vec<float, 2> rope_rot(float x0, float x1, float pos, int pair, int HD, bool inverse) {
+  const float inv_freq = exp2f(-(float)(2 * pair) / (float)HD * 13.287712379549449f);   // 10000^(-2i/HD)
+  // the hardware sine / cosine take their argument in turns; reduce it to [0, 1) first
+  const float turns = pos * inv_freq * 0.15915494309189535f;
+  const float fr = turns - floorf(turns);
+  float sn = __builtin_amdgcn_sinf(fr);
+  const float cs = __builtin_amdgcn_cosf(fr);
+  if (inverse) sn = -sn;
+  vec<float, 2> y = {x0 * cs - x1 * sn, x1 * cs + x0 * sn};
+  return y;
+}
+// the same on two lvalues (vector elements cannot be bound to references)
+#define CASTLE_ROPE_PAIR(X0, X1, POS, PAIR, HD_, INV)                          \
+  do {                                                                         \
+    const vec<float, 2> y_ = rope_rot((X0), (X1), (POS), (PAIR), (HD_), (INV)); \
+    (X0) = y_[0];                                                              \
+    (X1) = y_[1];                                                              \
+  } while (0)
+
 // head bh of an operand copy in the compute type ([B*H][Lp][HD] contiguous, rows >= L zero)
 template <typename T> __device__ __forceinline__ const T* prep_ptr(const void* base, int bh, int Lp, int HD) {
   return reinterpret_cast<const T*>(base) + (int64_t)bh * Lp * HD;

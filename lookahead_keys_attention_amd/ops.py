@@ -21,7 +21,7 @@ from . import _native as N
 
 
 # flags handed to castle_fwd / castle_bwd (0, or _native.FLAG_BF16_OPERANDS); read when the
-# forward runs and remembered for its backward
+# forward runs and remembered for its backward.  The `rotary` arguments below add FLAG_ROTARY.
 DEFAULT_FLAGS = 0
 
 
@@ -75,14 +75,14 @@ class _CastleAttention(torch.autograd.Function):
     """Six separate operands (the reference operator's signature)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, qu, ku, vu, scale, want_U):
+    def forward(ctx, q, k, v, qu, ku, vu, scale, want_U, rotary=False):
         _require_gpu(q, "castle_attention_hip")
         B, H, L, d = q.shape
         _check_dims(d, q.dtype)
         ops = [_as_readable(t) for t in (q, k, v, qu, ku, vu)]
         out = torch.empty((B, L, H, d), dtype=q.dtype, device=q.device).permute(0, 2, 1, 3)
         U = torch.empty((B, H, L, d), dtype=q.dtype, device=q.device) if want_U else None
-        ctx.flags = DEFAULT_FLAGS
+        ctx.flags = DEFAULT_FLAGS | (N.FLAG_ROTARY if rotary else 0)
         ws = _fwd_raw(*ops, scale, out, U, ctx.flags)
         ctx.save_for_backward(*ops, out, ws)
         ctx.scale = scale
@@ -99,14 +99,14 @@ class _CastleAttention(torch.autograd.Function):
         packed = torch.empty((6, B, H, L, d), dtype=out.dtype, device=out.device)
         grads = list(packed.unbind(0))
         _bwd_raw(*ops, out, dout, ctx.scale, grads, ws, ctx.flags)
-        return (*grads, None, None)
+        return (*grads, None, None, None)
 
 
 class _CastleAttentionPacked(torch.autograd.Function):
     """Fused-projection layout in, merged heads out."""
 
     @staticmethod
-    def forward(ctx, proj, heads, scale, U_out):
+    def forward(ctx, proj, heads, scale, U_out, rotary=False):
         # U_out: None, or a (B,H,L,d) view without gradient history that receives the lookahead keys
         _require_gpu(proj, "castle_attention_packed")
         B, L, width = proj.shape
@@ -117,7 +117,7 @@ class _CastleAttentionPacked(torch.autograd.Function):
         qu, ku, vu, qc, kc, vc = six.unbind(0)
         merged = torch.empty((B, L, heads * d), dtype=proj.dtype, device=proj.device)
         out = merged.view(B, L, heads, d).permute(0, 2, 1, 3)
-        ctx.flags = DEFAULT_FLAGS
+        ctx.flags = DEFAULT_FLAGS | (N.FLAG_ROTARY if rotary else 0)
         ws = _fwd_raw(qc, kc, vc, qu, ku, vu, scale, out, U_out, ctx.flags)
         ctx.save_for_backward(proj, merged, ws)
         ctx.heads, ctx.scale = heads, scale
@@ -137,23 +137,24 @@ class _CastleAttentionPacked(torch.autograd.Function):
         dproj = torch.empty_like(proj)
         dqu, dku, dvu, dqc, dkc, dvc = dproj.view(B, L, 6, heads, d).permute(2, 0, 3, 1, 4).unbind(0)
         _bwd_raw(qc, kc, vc, qu, ku, vu, out, dout, scale, (dqc, dkc, dvc, dqu, dku, dvu), ws, ctx.flags)
-        return dproj, None, None, None
+        return dproj, None, None, None, None
 
 
-def castle_attention_hip(q, k, v, qu, ku, vu, scale, return_U_for_cache=False):
-    """Drop-in for castle_attention_triton: returns out, or (out, U)."""
-    return _CastleAttention.apply(q, k, v, qu, ku, vu, float(scale), bool(return_U_for_cache))
+def castle_attention_hip(q, k, v, qu, ku, vu, scale, return_U_for_cache=False, rotary=False):
+    """Drop-in for castle_attention_triton: returns out, or (out, U).  rotary=True applies the
+    rotary position embedding (positions 0..L-1) to q, k, qu, ku, vu inside the kernels."""
+    return _CastleAttention.apply(q, k, v, qu, ku, vu, float(scale), bool(return_U_for_cache), bool(rotary))
 
 
-def castle_attention_packed(proj, heads, scale, return_U_for_cache=False, U_out=None):
+def castle_attention_packed(proj, heads, scale, return_U_for_cache=False, U_out=None, rotary=False):
     """proj (B, L, 6*H*d) -> merged out (B, L, H*d), or (out, U (B,H,L,d)).  `U_out`, if given,
     is the (B,H,L,d) view (any row stride) the lookahead keys are written into."""
     if not return_U_for_cache:
-        return _CastleAttentionPacked.apply(proj, int(heads), float(scale), None)
+        return _CastleAttentionPacked.apply(proj, int(heads), float(scale), None, bool(rotary))
     if U_out is None:
         B, L, width = proj.shape
         U_out = torch.empty((B, heads, L, width // (6 * heads)), dtype=proj.dtype, device=proj.device)
-    return _CastleAttentionPacked.apply(proj, int(heads), float(scale), U_out), U_out
+    return _CastleAttentionPacked.apply(proj, int(heads), float(scale), U_out, bool(rotary)), U_out
 
 
 def decode_workspace(B, H, d, device):
@@ -162,9 +163,11 @@ def decode_workspace(B, H, d, device):
 
 
 @torch.no_grad()
-def castle_decode_step_hip(U, qu_cache, kc_cache, vc_cache, t, qc, kc, vc, qu, ku, vu, scale, out, workspace):
+def castle_decode_step_hip(U, qu_cache, kc_cache, vc_cache, t, qc, kc, vc, qu, ku, vu, scale, out, workspace,
+                           rotary=False):
     """In-place cached step.  The four cache tensors are (B,H,capacity,d) buffers with t valid
-    rows (capacity > t); the new-token operands and `out` are (B,H,1,d)."""
+    rows (capacity > t); the new-token operands and `out` are (B,H,1,d).  rotary=True rotates the
+    new token by position t inside the kernels (the cache rows are stored rotated)."""
     _require_gpu(U, "castle_decode_step_hip")
     B, H, cap, d = U.shape
     if not (0 <= t < cap):
@@ -176,7 +179,22 @@ def castle_decode_step_hip(U, qu_cache, kc_cache, vc_cache, t, qc, kc, vc, qu, k
     views = [N.view4(x) for x in (U, qu_cache, kc_cache, vc_cache)]
     tviews = [N.view4(x) for x in toks]
     with torch.cuda.device(U.device):
-        rc = N.lib().castle_decode_step(*views, int(t), *tviews, B, H, d, code, float(scale), N.view4(out),
+        rc = N.lib().castle_decode_step(*views, int(t), *tviews, B, H, d, code, float(scale),
+                                        N.FLAG_ROTARY if rotary else 0, N.view4(out),
                                         workspace.data_ptr(), workspace.numel(), N.stream_ptr(U.device))
     N.check(rc, "castle_decode_step")
+    return out
+
+
+@torch.no_grad()
+def castle_rope_hip(x, out, first_position=0):
+    """out[b,h,l,:] = R(first_position + l) x[b,h,l,:]: the rotary position embedding the kernels
+    apply under FLAG_ROTARY, for one (B,H,L,d) tensor, out of place (used to fill cache rows)."""
+    _require_gpu(x, "castle_rope_hip")
+    B, H, L, d = x.shape
+    x = _as_readable(x)
+    with torch.cuda.device(x.device):
+        rc = N.lib().castle_rope(N.view4(x), N.view4(out), B, H, L, d, N.dtype_code(x.dtype), int(first_position),
+                                 N.stream_ptr(x.device))
+    N.check(rc, "castle_rope")
     return out
