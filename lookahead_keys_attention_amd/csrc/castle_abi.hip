@@ -4,6 +4,7 @@
 #include <stdint.h>
 
 #include "../../include/castle_hip.h"
+#include <stdlib.h>
 #include "castle_params.h"
 #include "castle_profile.h"
 #include "castle_tiles.h"
@@ -33,6 +34,15 @@ bool head_dim_ok(int d) { return d == 16 || d == 32 || d == 64 || d == 128; }
 
 int64_t align_up(int64_t x, int64_t a) { return (x + a - 1) / a * a; }
 
+// upper limit of the dS / dSu tile buffers (they grow with B*H*L^2); beyond it the backward
+// falls back to recomputing the score chain in its second kernel
+constexpr int64_t kMaxScoreTileBytes = (int64_t)16 << 30;
+// CASTLE_MAX_SCORE_TILE_BYTES in the environment overrides the limit (0 = never use the tiles)
+int64_t max_score_tile_bytes() {
+  const char* e = getenv("CASTLE_MAX_SCORE_TILE_BYTES");
+  return e != nullptr ? strtoll(e, nullptr, 10) : kMaxScoreTileBytes;
+}
+
 struct Geometry {
   int Lp, nblk;
   int64_t lse_bytes, tblk_bytes, snap_bytes, mat_bytes, op_bytes;
@@ -49,6 +59,7 @@ Geometry geometry(int B, int H, int L, int d, int es) {
   g.snap_bytes = align_up(BH * castle::snap_rows(g.nblk) * d * es, 256);
   // dS / dSu tiles between the two backward kernels: only the 16-bit, d <= 64 path uses them
   g.mat_bytes = (es == 2 && d <= 64) ? align_up(BH * g.Lp * g.Lp * es, 256) : 0;
+  if (2 * g.mat_bytes > max_score_tile_bytes()) g.mat_bytes = 0;   // too long: the query kernel recomputes the scores instead
   g.off_lse = 0;
   g.off_t = g.off_lse + g.lse_bytes;
   g.off_tt = g.off_t + g.tblk_bytes;

@@ -683,7 +683,7 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_key2_kernel(BwdArgs a) {
             const frag<T> fp = ld_nat<T>(x_p, LDX, c, ic + 8 * g);
             const frag<T> fds = ld_nat<T>(x_ds, LDX, c, ic + 8 * g);
             const frag<T> fdsu = ld_nat<T>(x_dsu, LDX, c, ic + 8 * g);
-            {   // hand the tile to the query-stationary kernel: 1 KB contiguous per store
+            if (a.ds_mat != nullptr) {   // hand the tile to the query-stationary kernel: 1 KB contiguous per store
               const int64_t tile = ((int64_t)(kw0 / 32) * (a.s.Lp / 32) + i0 / 32) * 1024 + s2 * 512 + c * 16 + g * 8;
               __builtin_nontemporal_store(fds, reinterpret_cast<frag_mem<T>*>(ds_mat + tile));
               __builtin_nontemporal_store(fdsu, reinterpret_cast<frag_mem<T>*>(dsu_mat + tile));
@@ -1459,8 +1459,12 @@ template <typename T, typename TI, int HD> static int launch_bwd_t(const BwdArgs
       hipLaunchKernelGGL((bwd_query_kernel<T, TI, HD, 1>), grid, block, query_lds, stream, a);
       hipLaunchKernelGGL((bwd_query_kernel<T, TI, HD, 2>), grid, block, query_lds, stream, a);
     } else if constexpr (TWO_ROLE) {
-      constexpr int query2_lds = bwd_query2_lds_bytes<T, HD>();
-      hipLaunchKernelGGL((bwd_query2_kernel<T, TI, HD>), grid, dim3(2 * kThreads), query2_lds, stream, a);
+      if (a.ds_mat != nullptr) {
+        constexpr int query2_lds = bwd_query2_lds_bytes<T, HD>();
+        hipLaunchKernelGGL((bwd_query2_kernel<T, TI, HD>), grid, dim3(2 * kThreads), query2_lds, stream, a);
+      } else {   // no room for the dS / dSu tiles (long sequences): the recomputing kernel
+        hipLaunchKernelGGL((bwd_query_kernel<T, TI, HD, 0>), grid, block, query_lds, stream, a);
+      }
     } else {
       hipLaunchKernelGGL((bwd_query_kernel<T, TI, HD, 0>), grid, block, query_lds, stream, a);
     }

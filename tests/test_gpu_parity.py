@@ -140,6 +140,25 @@ def test_rope_entry_point_matches_formula():
         assert (out.float().cpu() - want).abs().max() <= tol
 
 
+def test_backward_without_score_tiles(monkeypatch):
+    """Long sequences do not get the dS / dSu tile buffers (they grow with L^2); the second backward
+    kernel then recomputes the score chain.  Forced here through the environment override."""
+    monkeypatch.setenv("CASTLE_MAX_SCORE_TILE_BYTES", "0")
+    from lookahead_keys_attention_amd import _native
+
+    small = _native.lib().castle_bwd_workspace_bytes(2, 2, 300, 64, 1)
+    monkeypatch.delenv("CASTLE_MAX_SCORE_TILE_BYTES")
+    assert small < _native.lib().castle_bwd_workspace_bytes(2, 2, 300, 64, 1)
+    monkeypatch.setenv("CASTLE_MAX_SCORE_TILE_BYTES", "0")
+    ops, dout = rand_ops(2, 2, 300, 64, torch.bfloat16, seed=77)
+    s = 64 ** -0.5
+    leaves = [t.to(DEV).requires_grad_() for t in ops]
+    H().castle_attention_hip(*leaves, s).backward(dout.to(DEV))
+    ref = O.closed_form_grads(*[t.double() for t in ops], s, dout.double())
+    for name, leaf, r in zip(NAMES, leaves, ref):
+        assert_close(leaf.grad, r, torch.bfloat16, name, 2e-2)
+
+
 def test_lookahead_keys_carry_no_gradient():
     ops, dout = rand_ops(1, 1, 40, 16, torch.float32, seed=5)
     leaves = [t.to(DEV).requires_grad_() for t in ops]
