@@ -48,6 +48,7 @@ class _CacheStore:
         self.capacity = capacity
         self.length = 0
         self.workspace = ops.decode_workspace(B, H, d, device)
+        self.views = tuple(_native.view4(buf) for buf in self.buffers)   # reused by every step on these buffers
 
     def as_cache(self) -> Cache:
         n = self.length
@@ -178,8 +179,12 @@ class Castle(nn.Module):
         if t + 1 > store.capacity:
             store = store.grown(_reserve_rows(t + 1))
         out = torch.empty((B, 1, H, d), dtype=proj.dtype, device=proj.device)
-        ops.castle_decode_step_hip(*store.buffers, t, qc, kc, vc, qu, ku, vu, self.scale,
-                                   out.permute(0, 2, 1, 3), store.workspace, rotary=self.rotary_emb)
+        if proj.is_contiguous() and proj.data_ptr() % 16 == 0:
+            ops.castle_decode_step_packed(store.views, store.capacity, t, proj, H, self.scale, out, store.workspace,
+                                          rotary=self.rotary_emb)
+        else:
+            ops.castle_decode_step_hip(*store.buffers, t, qc, kc, vc, qu, ku, vu, self.scale,
+                                       out.permute(0, 2, 1, 3), store.workspace, rotary=self.rotary_emb)
         store.length = t + 1
         return out.view(B, 1, H * d), store.as_cache()
 

@@ -198,3 +198,26 @@ def castle_rope_hip(x, out, first_position=0):
                                  N.stream_ptr(x.device))
     N.check(rc, "castle_rope")
     return out
+
+
+@torch.no_grad()
+def castle_decode_step_packed(cache_views, capacity, t, proj, heads, scale, out, workspace, rotary=False):
+    """The cached step for a fused projection: `proj` is the contiguous (B, 1, 6*H*d) output of the
+    layer's projection for the new token (order qu, ku, vu, qc, kc, vc), `cache_views` the four
+    castle_view4 of the (B, H, capacity, d) cache buffers (built once per buffer set), `out` a
+    (B, 1, H, d) tensor.  Same kernels as castle_decode_step_hip, without per-call view building."""
+    B, n, width = proj.shape
+    d = width // (6 * heads)
+    if n != 1 or not proj.is_contiguous() or proj.data_ptr() % 16 != 0 or not proj.is_cuda:
+        raise ValueError("castle_decode_step_packed needs a contiguous, 16-byte aligned (B, 1, 6*H*d) GPU tensor")
+    if not (0 <= t < capacity):
+        raise ValueError(f"cache capacity {capacity} cannot take row {t}")
+    es, base, part = proj.element_size(), proj.data_ptr(), heads * d
+    qu, ku, vu, qc, kc, vc = (N.View4(base + i * part * es, width, d, width) for i in range(6))
+    with torch.cuda.device(proj.device):
+        rc = N.lib().castle_decode_step(*cache_views, int(t), qc, kc, vc, qu, ku, vu, B, heads, d,
+                                        N.dtype_code(proj.dtype), float(scale), N.FLAG_ROTARY if rotary else 0,
+                                        N.View4(out.data_ptr(), heads * d, d, heads * d),
+                                        workspace.data_ptr(), workspace.numel(), N.stream_ptr(proj.device))
+    N.check(rc, "castle_decode_step")
+    return out
