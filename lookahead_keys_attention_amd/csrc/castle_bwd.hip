@@ -172,10 +172,10 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
 #define CASTLE_BK_LOAD(I_)                                   \
   do {                                                       \
     const int64_t r_ = (int64_t)(I_) * kNB;                  \
-    pqc.load(qc, HD, r_, kNoRowLimit);                            \
-    pdo.load(dout, HD, r_, kNoRowLimit);                        \
-    pku.load(ku, HD, r_, kNoRowLimit);                            \
-    pvu.load(vu, HD, r_, kNoRowLimit);                            \
+    pqc.load_flat(qc + r_ * HD);                            \
+    pdo.load_flat(dout + r_ * HD);                        \
+    pku.load_flat(ku + r_ * HD);                            \
+    pvu.load_flat(vu + r_ * HD);                            \
     ptb.load(tb, kNB, r_, (int64_t)1 << 40);                 \
   } while (0)
 
@@ -825,9 +825,9 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
 #define CASTLE_BQ_LOAD(K0)                                                                                      \
   do {                                                                                                          \
     const int kb_ = (K0) / kNB;                                                                                 \
-    pkc.load(kc, HD, (K0), kNoRowLimit);                                                                             \
-    pvc.load(vc, HD, (K0), kNoRowLimit);                                                                             \
-    pqu.load(qu, HD, (K0), kNoRowLimit);                                                                             \
+    pkc.load_flat(kc + (int64_t)(K0) * HD);                                                                             \
+    pvc.load_flat(vc + (int64_t)(K0) * HD);                                                                             \
+    pqu.load_flat(qu + (int64_t)(K0) * HD);                                                                             \
     if (kb_ < blk0) pu0.load(usnap + (usnap_off(blk0) + (K0)) * HD);                          \
     if (kb_ < blk1 && blk1 < a.s.nblk) pu1.load(usnap + (usnap_off(blk1) + (K0)) * HD);        \
     if (DO_S && kb_ <= blk0 && blk0 <= a.s.nblk - 2) pg0.load(gsnap + (gsnap_off(blk0) + (K0)) * HD);  \
