@@ -29,11 +29,16 @@ extern __shared__ __attribute__((aligned(16))) unsigned char castle_smem[];
 //   gate operand (Qu or Ku, whichever is resident) is multiplied by -c1, so that
 //   A = 1 / (1 + exp2(acc)) needs no multiply.
 // Then sigmoid(Su) = 1/(1+exp2(-Su')), S' = Sc' - Su' sigmoid(Su) = log2(e) S, P = exp2(S' - m').
+// value tile of the scan / attention kernels: 16-bit operands keep it row-major and read it with
+// transpose loads, fp32 stores it transposed
+template <typename T, int HD> constexpr int vtile_elems() {
+  return sizeof(T) == 2 ? kNB * lds_ld<T>(HD) : (HD < 32 ? 32 : HD) * lds_ld_chain<T>(kNB);
+}
 template <typename T, int HD> constexpr int scan_lds_bytes() {
-  return (int)sizeof(T) * (kNB * lds_ld<T>(HD) + (HD < 32 ? 32 : HD) * lds_ld_chain<T>(kNB));
+  return (int)sizeof(T) * (kNB * lds_ld<T>(HD) + vtile_elems<T, HD>());
 }
 template <typename T, int HD> constexpr int attn_lds_bytes() {
-  return (int)sizeof(T) * (4 * kNB * lds_ld<T>(HD) + (HD < 32 ? 32 : HD) * lds_ld_chain<T>(kNB) + kNB * lds_ld<T>(128));
+  return (int)sizeof(T) * (4 * kNB * lds_ld<T>(HD) + vtile_elems<T, HD>() + kNB * lds_ld<T>(128));
 }
 // register prefetch of the next tile is affordable for 16-bit operands up to d = 64
 template <typename T, int HD> constexpr bool use_prefetch() { return sizeof(T) == 2 && HD <= 64; }
@@ -127,7 +132,8 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(FwdArgs a) {
   constexpr int LDK = lds_ld<T>(HD), LDV = lds_ld_chain<T>(kNB);
   constexpr bool PF = use_prefetch<T, HD>();
   T* s_ku = reinterpret_cast<T*>(castle_smem);   // [kNB][LDK]
-  T* s_vut = s_ku + kNB * LDK;                   // [HDP][LDV]
+  T* s_vut = s_ku + kNB * LDK;                   // fp32: [HDP][LDV] (transposed); 16-bit: [kNB][LDK]
+  constexpr bool TRV = sizeof(T) == 2;
 
   int kb, bh;   // key group 0 sweeps every source block: rank order = kb
   work_item(a.s.B * a.s.H, kb, bh);
@@ -148,30 +154,31 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(FwdArgs a) {
   acc_t st[NT];   // state^T : rows n (head dim), columns k (lanes)
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) zero(st[nt]);
-  if (HDP > HD) lds_zero(s_vut + HD * LDV, (HDP - HD) * LDV);
+  if (!TRV && HDP > HD) lds_zero(s_vut + HD * LDV, (HDP - HD) * LDV);
 
-  RowStage<T, T, kNB, HD> pku;
+#pragma unroll
+  for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(fq[s]));   // loaded before the prefetches start
+  RowStage<T, T, kNB, HD> pku, pvr;
   ColStage<T, T, kNB, HD> pvu;
+  auto load_block = [&](int I) __attribute__((always_inline)) {
+    pku.load_flat(ku + (int64_t)I * kNB * HD);
+    if (TRV) pvr.load_flat(vu + (int64_t)I * kNB * HD);
+    else pvu.load(vu, HD, (int64_t)I * kNB, kNoRowLimit);
+  };
   const int I0 = (kb * 128) / kNB;
-  if (PF) {
-    pku.load(ku, HD, (int64_t)I0 * kNB, kNoRowLimit);
-    pvu.load(vu, HD, (int64_t)I0 * kNB, kNoRowLimit);
-  }
+  if (PF) load_block(I0);
   for (int I = I0; I < a.s.nblk; ++I) {
+    __syncthreads();
+    if (!PF) load_block(I);
+    pku.store(s_ku, LDK);
+    if (TRV) pvr.store(s_vut, LDK);
+    else pvu.store(s_vut, LDV);
+    // after the staging wait, not before it: the wait counter also covers stores, and these
+    // then have the whole block to drain
     if (I * kNB >= kw0 + 32) {   // all keys of this wave precede block I: snapshot
       store_snap_tile<T, HD, NT>(snap + (usnap_off(I) + kw0) * HD, st, c, g);
     }
-    __syncthreads();
-    if (!PF) {
-      pku.load(ku, HD, (int64_t)I * kNB, kNoRowLimit);
-      pvu.load(vu, HD, (int64_t)I * kNB, kNoRowLimit);
-    }
-    pku.store(s_ku, LDK);
-    pvu.store(s_vut, LDV);
-    if (PF && I + 1 < a.s.nblk) {   // in flight while this block is processed
-      pku.load(ku, HD, (int64_t)(I + 1) * kNB, kNoRowLimit);
-      pvu.load(vu, HD, (int64_t)(I + 1) * kNB, kNoRowLimit);
-    }
+    if (PF && I + 1 < a.s.nblk) load_block(I + 1);   // in flight while this block is processed
     __syncthreads();
 #pragma unroll
     for (int jt = 0; jt < JT; ++jt) {
@@ -192,7 +199,9 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(FwdArgs a) {
       for (int s2 = 0; s2 < 2; ++s2) {
         const frag<T> fa = chain<T>(aT, s2);
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) mma(st[nt], ld_chain<T>(s_vut, LDV, 32 * nt + c, 32 * jt + 16 * s2, g), fa);
+        for (int nt = 0; nt < NT; ++nt)
+          mma(st[nt], TRV ? ld_free<T, true>(s_vut, LDK, 32 * nt, HD, 32 * jt + 16 * s2, c, g)
+                          : ld_chain<T>(s_vut, LDV, 32 * nt + c, 32 * jt + 16 * s2, g), fa);
       }
     }
   }
@@ -222,8 +231,9 @@ __global__ __launch_bounds__(kThreads, (sizeof(T) == 2 && HD <= 64) ? 2 : 1) voi
   T* s_kc = reinterpret_cast<T*>(castle_smem);   // [kNB][LDK]
   T* s_qu = s_kc + kNB * LDK;                    // [kNB][LDK]
   T* s_ub0 = s_qu + kNB * LDK;                   // [NBLK_Q][kNB][LDK]
-  T* s_vct = s_ub0 + NBLK_Q * kNB * LDK;         // [HDP][LDV]
-  T* s_a = s_vct + HDP * LDV;                    // [kNB][LDA]
+  T* s_vct = s_ub0 + NBLK_Q * kNB * LDK;         // fp32: [HDP][LDV] (transposed); 16-bit: [kNB][LDK]
+  T* s_a = s_vct + vtile_elems<T, HD>();         // [kNB][LDA]
+  constexpr bool TRV = sizeof(T) == 2;
 
   int rank, bh;
   work_item(a.s.B * a.s.H, rank, bh);
@@ -261,18 +271,19 @@ __global__ __launch_bounds__(kThreads, (sizeof(T) == 2 && HD <= 64) ? 2 : 1) voi
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) zero(o[nt]);
   float m = -INFINITY, l = 0.f;
-  if (HDP > HD) lds_zero(s_vct + HD * LDV, (HDP - HD) * LDV);
+  if (!TRV && HDP > HD) lds_zero(s_vct + HD * LDV, (HDP - HD) * LDV);
 
   int nchunks = (qb * QB + QB) / kNB;
   if (nchunks > a.s.nblk) nchunks = a.s.nblk;
 
-  RowStage<T, T, kNB, HD> pkc, pqu;
+  RowStage<T, T, kNB, HD> pkc, pqu, pvr;
   ColStage<T, T, kNB, HD> pvc;
   SnapStage<T, kNB, HD> pub[NBLK_Q];
   auto load_chunk = [&](int Kb) __attribute__((always_inline)) {
-    pkc.load(kc, HD, (int64_t)Kb * kNB, kNoRowLimit);
-    pvc.load(vc, HD, (int64_t)Kb * kNB, kNoRowLimit);
-    pqu.load(qu, HD, (int64_t)Kb * kNB, kNoRowLimit);
+    pkc.load_flat(kc + (int64_t)Kb * kNB * HD);
+    if (TRV) pvr.load_flat(vc + (int64_t)Kb * kNB * HD);
+    else pvc.load(vc, HD, (int64_t)Kb * kNB, kNoRowLimit);
+    pqu.load_flat(qu + (int64_t)Kb * kNB * HD);
 #pragma unroll
     for (int q = 0; q < NBLK_Q; ++q) {
       const int blk = Ifirst + q;
@@ -281,7 +292,8 @@ __global__ __launch_bounds__(kThreads, (sizeof(T) == 2 && HD <= 64) ? 2 : 1) voi
   };
   auto store_chunk = [&](int Kb) __attribute__((always_inline)) {
     pkc.store(s_kc, LDK);
-    pvc.store(s_vct, LDV);
+    if (TRV) pvr.store(s_vct, LDK);
+    else pvc.store(s_vct, LDV);
     pqu.store(s_qu, LDK);
 #pragma unroll
     for (int q = 0; q < NBLK_Q; ++q) {
@@ -290,6 +302,12 @@ __global__ __launch_bounds__(kThreads, (sizeof(T) == 2 && HD <= 64) ? 2 : 1) voi
     }
   };
 
+  // the row fragments are consumed before the loop as far as the wait counters are concerned:
+  // otherwise every use inside the loop waits for the chunk prefetch issued after them
+#pragma unroll
+  for (int s = 0; s < KS; ++s) { asm volatile("" : "+v"(fqc[s])); asm volatile("" : "+v"(fku[s])); }
+#pragma unroll
+  for (int s = 0; s < kNB / 16; ++s) asm volatile("" : "+v"(ft[s]));
   if (PF) load_chunk(0);
   for (int Kb = 0; Kb < nchunks; ++Kb) {
     __syncthreads();
@@ -372,7 +390,9 @@ __global__ __launch_bounds__(kThreads, (sizeof(T) == 2 && HD <= 64) ? 2 : 1) voi
         for (int s2 = 0; s2 < 2; ++s2) {
           const frag<T> fp = chain<T>(sc, s2);
 #pragma unroll
-          for (int nt = 0; nt < NT; ++nt) mma(o[nt], ld_chain<T>(s_vct, LDV, 32 * nt + c, 32 * kt + 16 * s2, g), fp);
+          for (int nt = 0; nt < NT; ++nt)
+            mma(o[nt], TRV ? ld_free<T, true>(s_vct, LDK, 32 * nt, HD, 32 * kt + 16 * s2, c, g)
+                           : ld_chain<T>(s_vct, LDV, 32 * nt + c, 32 * kt + 16 * s2, g), fp);
         }
       }
     }
