@@ -34,7 +34,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 1 GiB copy
 # (profiles/castle_cfg2_cfg4_pmc_hbm_traffic.txt).  Recorded values, not measured by this script.
-MEASURED_TRAFFIC_BYTES = {"scan": 750.6e6, "attn": 719.0e6, "bwd_key": 2707.2e6, "bwd_query": 2475.3e6, "decode_stream": 378.9e6}
+MEASURED_TRAFFIC_BYTES = {"scan": 732.7e6, "attn": 732.4e6, "bwd_key": 2705.5e6, "bwd_query": 2474.4e6, "decode_stream": 378.9e6}
 
 # algorithmic contractions (unit: B*H*L^2*d flop = 2*d flop per causal pair) attributed to each kernel
 KERNEL_UNITS = {"tqv": 0.0, "scan": 2.0, "attn": 3.0, "delta": 0.0, "bwd_key": 9.0, "bwd_query": 4.0}
@@ -97,7 +97,12 @@ def bench_layer(steps, warmup):
                  "frac_of_peak": round(core / (core_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4), "kernels": table},
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(dom)},
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(dom),
+                     # the same launch seen from the memory side: measured HBM bytes / live duration
+                     "hbm_GBps": round(MEASURED_TRAFFIC_BYTES[dom] / (table[dom]["ms"] * 1e-3) / 1e9, 1)
+                     if dom in MEASURED_TRAFFIC_BYTES else None,
+                     "hbm_frac": round(MEASURED_TRAFFIC_BYTES[dom] / (table[dom]["ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)
+                     if dom in MEASURED_TRAFFIC_BYTES else None},
         "global_batch": B, "seq_len": L,
     }
 
