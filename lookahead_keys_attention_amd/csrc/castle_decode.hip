@@ -148,25 +148,45 @@ __global__ __launch_bounds__(64) void decode_finish_kernel(DecodeArgs a) {
   for (int o = 1; o < 64; o <<= 1) dot += __shfl_xor(dot, o);
   const float xt = dot * c1;            // row t: U_t = 0, so the lookahead term is silu(0) = 0
 
-  float M = xt;
+  // statistics of the partials: lane s holds split s (at most 64 splits), so the loads of all
+  // splits are in flight together instead of one dependent load per loop iteration
   const int nsplit = a.t > 0 ? a.splits : 0;
-  for (int s = 0; s < nsplit; ++s) M = fmaxf(M, part[s * (HD + 2) + HD]);
+  float ms_l = -INFINITY, ls_l = 0.f;
+  if (lane < nsplit) {
+    ms_l = part[lane * (HD + 2) + HD];
+    ls_l = part[lane * (HD + 2) + HD + 1];
+  }
+  float M = ms_l;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) M = fmaxf(M, __shfl_xor(M, o));
+  M = fmaxf(M, xt);
+  const float w_l = (ms_l == -INFINITY) ? 0.f : fast_exp2(ms_l - M);
+  float lsum = w_l * ls_l;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) lsum += __shfl_xor(lsum, o);
   const float pt = fast_exp2(xt - M);
-  float lsum = pt;
+  lsum += pt;
   float o[EPL];
 #pragma unroll
   for (int e = 0; e < EPL; ++e) {
     const int n = lane + 64 * e;
     o[e] = n < HD ? pt * (float)vc[n] : 0.f;
   }
-  for (int s = 0; s < nsplit; ++s) {
-    const float ms = part[s * (HD + 2) + HD];
-    const float w = (ms == -INFINITY) ? 0.f : fast_exp2(ms - M);
-    lsum = __builtin_fmaf(w, part[s * (HD + 2) + HD + 1], lsum);
+  constexpr int SU = 8;   // partial rows loaded per batch
+  for (int s0 = 0; s0 < nsplit; s0 += SU) {
+    float v[SU][EPL];
 #pragma unroll
-    for (int e = 0; e < EPL; ++e) {
-      const int n = lane + 64 * e;
-      if (n < HD) o[e] = __builtin_fmaf(w, part[s * (HD + 2) + n], o[e]);
+    for (int u = 0; u < SU; ++u)
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) {
+        const int n = lane + 64 * e;
+        v[u][e] = (s0 + u < nsplit && n < HD) ? part[(s0 + u) * (HD + 2) + n] : 0.f;
+      }
+#pragma unroll
+    for (int u = 0; u < SU; ++u) {
+      const float w = __shfl(w_l, (s0 + u) & 63);   // 0 for lanes beyond nsplit
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) o[e] = __builtin_fmaf(w, v[u][e], o[e]);
     }
   }
   const float inv = 1.f / lsum;
