@@ -12,6 +12,7 @@
  *                       math of lookahead_keys_attention.py:132-164
  *   castle_bwd          lookahead_keys_attention_triton.py:508-602  CastleAttentionFunction.backward
  *   castle_decode_step  lookahead_keys_attention.py:166-203         the seq_len == 1 branch of Castle.forward
+ *   castle_decode_step_device_count   the same step, row count in device memory (graph replay)
  */
 #ifndef CASTLE_HIP_H_
 #define CASTLE_HIP_H_
@@ -22,7 +23,7 @@
 extern "C" {
 #endif
 
-#define CASTLE_ABI_VERSION 2
+#define CASTLE_ABI_VERSION 3
 
 /* element types of the tensors (accumulation is always fp32) */
 #define CASTLE_F32 0
@@ -119,6 +120,22 @@ int castle_decode_step(const castle_view4* U, const castle_view4* qu_cache,
                        int B, int H, int d, int dtype, float scale, int flags,
                        const castle_view4* out,
                        void* workspace, int64_t workspace_bytes, void* stream);
+
+/* The same step with the row count t read by the kernels from device memory (*t_device, an int32
+ * the caller keeps and advances), so that the enqueued work does not depend on t: one captured HIP
+ * graph of a whole model step can be replayed for every token.  `capacity` = rows of the cache
+ * buffers; the work split is sized for it, and a step found at *t_device >= capacity (or < 0)
+ * writes nothing.  No counterpart in the reference (its step takes t from the tensor shapes,
+ * lookahead_keys_attention.py:166-203); meant for callers that replay a captured step.  The call
+ * itself records only kernel launches on `stream` (no memset, no allocation, no synchronisation). */
+int castle_decode_step_device_count(const castle_view4* U, const castle_view4* qu_cache,
+                                    const castle_view4* kc_cache, const castle_view4* vc_cache,
+                                    const int32_t* t_device, int capacity,
+                                    const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
+                                    const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
+                                    int B, int H, int d, int dtype, float scale, int flags,
+                                    const castle_view4* out,
+                                    void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Rotary position embedding of one tensor, out of place: out[b,h,l,:] = R(first_position + l) x[b,h,l,:]
  * (the rotation CASTLE_FLAG_ROTARY applies inside the kernels; lookahead_keys_attention.py:112).  Used to

@@ -6,6 +6,6 @@ operators run hand-written HIP kernels for gfx950 through the C ABI in include/c
 """
 from .castle import Castle, Cache
 from .ops import castle_attention_hip, castle_attention_packed, castle_decode_step_hip
-from .lm import CastleLM
+from .lm import CastleLM, GraphedDecoder
 
-__all__ = ["Castle", "Cache", "CastleLM", "castle_attention_hip", "castle_attention_packed", "castle_decode_step_hip"]
+__all__ = ["Castle", "Cache", "CastleLM", "GraphedDecoder", "castle_attention_hip", "castle_attention_packed", "castle_decode_step_hip"]

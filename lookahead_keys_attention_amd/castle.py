@@ -188,6 +188,19 @@ class Castle(nn.Module):
         store.length = t + 1
         return out.view(B, 1, H * d), store.as_cache()
 
+    def graph_step(self, x, store, t_device):
+        """The cached single-token step in the form a captured HIP graph needs: the same GPU work
+        as forward(x, cache) on the native path, but the row count is read by the kernels from the
+        one-element int32 GPU tensor `t_device`, and nothing on the host depends on it (no cache
+        object is built, `store.length` is left alone: the owner of the graph keeps the count).
+        x: (B, 1, dim); store: the `_CacheStore` behind a native cache.  Returns (B, 1, dim)."""
+        B = x.shape[0]
+        proj = self.to_all_qkv(self.norm(x))
+        out = torch.empty((B, 1, self.heads, self.dim_head), dtype=proj.dtype, device=proj.device)
+        ops.castle_decode_step_packed(store.views, store.capacity, 0, proj, self.heads, self.scale, out,
+                                      store.workspace, rotary=self.rotary_emb, t_device=t_device)
+        return self.combine_heads(out.view(B, 1, self.heads * self.dim_head))
+
     # -- dense PyTorch formulation (use_triton=False) -------------------------
     def _parallel_dense(self, proj, want_cache):
         B, n, _ = proj.shape

@@ -217,16 +217,17 @@ int64_t castle_decode_workspace_bytes(int B, int H, int d, int t_max) {
   return align_up((int64_t)B * H * 64 * (d + 2) * 4, 256);
 }
 
-int castle_decode_step(const castle_view4* U, const castle_view4* qu_cache,
-                       const castle_view4* kc_cache, const castle_view4* vc_cache, int t,
-                       const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
-                       const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
-                       int B, int H, int d, int dtype, float scale, int flags,
-                       const castle_view4* out,
-                       void* workspace, int64_t workspace_bytes, void* stream) {
+static int decode_step_common(const castle_view4* U, const castle_view4* qu_cache,
+                              const castle_view4* kc_cache, const castle_view4* vc_cache,
+                              int t, const int* t_device, int capacity,
+                              const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
+                              const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
+                              int B, int H, int d, int dtype, float scale, int flags,
+                              const castle_view4* out,
+                              void* workspace, int64_t workspace_bytes, void* stream) {
   const int es = elem_size(dtype);
   if (es == 0) return CASTLE_ERR_DTYPE;
-  if (B <= 0 || H <= 0 || t < 0 || !head_dim_ok(d) || (int64_t)B * H > 65535) return CASTLE_ERR_SHAPE;
+  if (B <= 0 || H <= 0 || t < 0 || capacity <= 0 || !head_dim_ok(d) || (int64_t)B * H > 65535) return CASTLE_ERR_SHAPE;
   const castle_view4* caches[] = {U, qu_cache, kc_cache, vc_cache};
   for (const castle_view4* v : caches)
     if (!view_ok(v, es, true)) return CASTLE_ERR_ARG;
@@ -239,14 +240,40 @@ int castle_decode_step(const castle_view4* U, const castle_view4* qu_cache,
 
   castle::DecodeArgs a;
   a.B = B; a.H = H; a.d = d; a.t = t; a.scale = scale;
+  a.t_dev = t_device; a.capacity = capacity;
   a.rotary = (flags & CASTLE_FLAG_ROTARY) != 0;
-  a.splits = castle::decode_pick_splits(B * H, t);
+  // with a device-side count the split must not depend on it: sized for a full cache
+  a.splits = castle::decode_pick_splits(B * H, t_device != nullptr ? capacity : t);
   a.U = to_view(U); a.qu_cache = to_view(qu_cache); a.kc_cache = to_view(kc_cache); a.vc_cache = to_view(vc_cache);
   a.qc = to_view(qc); a.kc = to_view(kc); a.vc = to_view(vc);
   a.qu = to_view(qu); a.ku = to_view(ku); a.vu = to_view(vu);
   a.out = to_view(out);
   a.part = static_cast<float*>(workspace);
   return castle::launch_decode(a, dtype, static_cast<hipStream_t>(stream));
+}
+
+int castle_decode_step(const castle_view4* U, const castle_view4* qu_cache,
+                       const castle_view4* kc_cache, const castle_view4* vc_cache, int t,
+                       const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
+                       const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
+                       int B, int H, int d, int dtype, float scale, int flags,
+                       const castle_view4* out,
+                       void* workspace, int64_t workspace_bytes, void* stream) {
+  return decode_step_common(U, qu_cache, kc_cache, vc_cache, t, nullptr, 0x7fffffff, qc, kc, vc, qu, ku, vu,
+                            B, H, d, dtype, scale, flags, out, workspace, workspace_bytes, stream);
+}
+
+int castle_decode_step_device_count(const castle_view4* U, const castle_view4* qu_cache,
+                                    const castle_view4* kc_cache, const castle_view4* vc_cache,
+                                    const int32_t* t_device, int capacity,
+                                    const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
+                                    const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
+                                    int B, int H, int d, int dtype, float scale, int flags,
+                                    const castle_view4* out,
+                                    void* workspace, int64_t workspace_bytes, void* stream) {
+  if (t_device == nullptr || reinterpret_cast<uintptr_t>(t_device) % 4 != 0) return CASTLE_ERR_ARG;
+  return decode_step_common(U, qu_cache, kc_cache, vc_cache, 0, t_device, capacity, qc, kc, vc, qu, ku, vu,
+                            B, H, d, dtype, scale, flags, out, workspace, workspace_bytes, stream);
 }
 
 int castle_rope(const castle_view4* x, const castle_view4* out, int B, int H, int L, int d, int dtype,

@@ -41,14 +41,16 @@ __global__ __launch_bounds__(kThreads) void decode_stream_kernel(DecodeArgs a) {
   __shared__ float s_acc[kThreads / LPR][HD + 2];
 
   const int split = blockIdx.x, bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
+  int t = a.t_dev != nullptr ? *a.t_dev : a.t;
+  if (t < 0 || t >= a.capacity) t = 0;   // out of range (device-side count only): no rows, the finish kernel writes nothing
   const int tid = threadIdx.x;
   const int grp = tid / LPR, sub = tid % LPR;
   const float c0 = a.scale, c1 = a.scale * kLog2e;
 
   // rows of this workgroup: [r0, r1), whole iterations of RPI rows
-  const int per = ((a.t + a.splits - 1) / a.splits + RPI - 1) / RPI * RPI;
+  const int per = ((t + a.splits - 1) / a.splits + RPI - 1) / RPI * RPI;
   const int r0 = split * per;
-  const int r1 = min(a.t, r0 + per);
+  const int r1 = min(t, r0 + per);
 
   float ku[V], vu[V], qc[V];
   load_f32<T, V>(view_row<T>(a.ku, b, h, 0) + sub * V, ku);
@@ -58,9 +60,9 @@ __global__ __launch_bounds__(kThreads) void decode_stream_kernel(DecodeArgs a) {
 #pragma unroll
     for (int e = 0; e < V / 2; ++e) {
       const int pair = sub * (V / 2) + e;
-      CASTLE_ROPE_PAIR(ku[2 * e], ku[2 * e + 1], (float)a.t, pair, HD, false);
-      CASTLE_ROPE_PAIR(vu[2 * e], vu[2 * e + 1], (float)a.t, pair, HD, false);
-      CASTLE_ROPE_PAIR(qc[2 * e], qc[2 * e + 1], (float)a.t, pair, HD, false);
+      CASTLE_ROPE_PAIR(ku[2 * e], ku[2 * e + 1], (float)t, pair, HD, false);
+      CASTLE_ROPE_PAIR(vu[2 * e], vu[2 * e + 1], (float)t, pair, HD, false);
+      CASTLE_ROPE_PAIR(qc[2 * e], qc[2 * e + 1], (float)t, pair, HD, false);
     }
   }
 
@@ -131,6 +133,8 @@ __global__ __launch_bounds__(64) void decode_finish_kernel(DecodeArgs a) {
   constexpr int EPL = (HD + 63) / 64;   // elements per lane
   const int bh = blockIdx.x, b = bh / a.H, h = bh % a.H;
   const int lane = threadIdx.x;
+  const int t = a.t_dev != nullptr ? *a.t_dev : a.t;
+  if (t < 0 || t >= a.capacity) return;   // only reachable with a device-side count: the cache is full
   const float c1 = a.scale * kLog2e;
   const float* part = a.part + (int64_t)bh * a.splits * (HD + 2);
   const T* qc = view_row<T>(a.qc, b, h, 0);
@@ -150,7 +154,7 @@ __global__ __launch_bounds__(64) void decode_finish_kernel(DecodeArgs a) {
 
   // statistics of the partials: lane s holds split s (at most 64 splits), so the loads of all
   // splits are in flight together instead of one dependent load per loop iteration
-  const int nsplit = a.t > 0 ? a.splits : 0;
+  const int nsplit = t > 0 ? a.splits : 0;
   float ms_l = -INFINITY, ls_l = 0.f;
   if (lane < nsplit) {
     ms_l = part[lane * (HD + 2) + HD];
@@ -191,10 +195,10 @@ __global__ __launch_bounds__(64) void decode_finish_kernel(DecodeArgs a) {
   }
   const float inv = 1.f / lsum;
   T* out = view_row<T>(a.out, b, h, 0);
-  T* Ut = view_row<T>(a.U, b, h, a.t);
-  T* qut = view_row<T>(a.qu_cache, b, h, a.t);
-  T* kct = view_row<T>(a.kc_cache, b, h, a.t);
-  T* vct = view_row<T>(a.vc_cache, b, h, a.t);
+  T* Ut = view_row<T>(a.U, b, h, t);
+  T* qut = view_row<T>(a.qu_cache, b, h, t);
+  T* kct = view_row<T>(a.kc_cache, b, h, t);
+  T* vct = view_row<T>(a.vc_cache, b, h, t);
 #pragma unroll
   for (int e = 0; e < EPL; ++e) {
     const int n = lane + 64 * e;
@@ -203,8 +207,8 @@ __global__ __launch_bounds__(64) void decode_finish_kernel(DecodeArgs a) {
       const float qup = __shfl_xor(quv, 1), kcp = __shfl_xor(kcv, 1);
       const bool even = (n & 1) == 0;
       float q0 = even ? quv : qup, q1 = even ? qup : quv, k0 = even ? kcv : kcp, k1 = even ? kcp : kcv;
-      CASTLE_ROPE_PAIR(q0, q1, (float)a.t, n / 2, HD, false);
-      CASTLE_ROPE_PAIR(k0, k1, (float)a.t, n / 2, HD, false);
+      CASTLE_ROPE_PAIR(q0, q1, (float)t, n / 2, HD, false);
+      CASTLE_ROPE_PAIR(k0, k1, (float)t, n / 2, HD, false);
       quv = even ? q0 : q1;
       kcv = even ? k0 : k1;
     }
@@ -220,7 +224,7 @@ __global__ __launch_bounds__(64) void decode_finish_kernel(DecodeArgs a) {
 
 template <typename T, int HD> static int launch_decode_t(const DecodeArgs& a, hipStream_t stream) {
   const int BH = a.B * a.H;
-  if (a.t > 0) {
+  if (a.t_dev != nullptr || a.t > 0) {
     ProfScope ps(kSlotDecodeStream, stream);
     hipLaunchKernelGGL((decode_stream_kernel<T, HD>), dim3(a.splits, BH), dim3(kThreads), 0, stream, a);
   }

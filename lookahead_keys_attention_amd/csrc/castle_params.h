@@ -56,7 +56,9 @@ struct BwdArgs {
 
 struct DecodeArgs {
   int B, H, d;
-  int t;            // rows already in the cache
+  int t;            // rows already in the cache (used when t_dev is NULL)
+  const int* t_dev; // optional: the row count lives in device memory and is read by the kernels
+  int capacity;     // rows the cache buffers can hold; with t_dev a step at t >= capacity writes nothing
   int splits;       // partitions of the t rows per (b, h)
   float scale;
   int rotary;       // 1: the new token's qc, kc, qu, ku, vu are rotated by position t

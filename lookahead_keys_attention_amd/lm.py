@@ -45,6 +45,98 @@ def top_k(logits: torch.Tensor, thres: float = 0.9) -> torch.Tensor:
     return torch.full_like(logits, float("-inf")).scatter_(-1, index, values)
 
 
+class GraphedDecoder:
+    """One captured HIP graph of a whole single-token step of a `CastleLM` on the native path.
+
+    A token step of a small model is a few hundred tiny launches, bound by the host; captured once
+    and replayed, it costs one launch.  The cached attention step supports this through a row
+    count kept in device memory (`Castle.graph_step`): the graph reads it, uses it and increments
+    it, so every replay is the next step.  The graph ends at the logits; sampling stays outside.
+
+    `caches`: the per-layer caches of a native prefill (they are consumed: the graph updates their
+    buffers in place; read them back with `caches()`).  `max_len`: rows the caches must hold."""
+
+    def __init__(self, model: "CastleLM", caches, max_len: int):
+        stores = [getattr(c, "_store", None) for c in caches]
+        if len(stores) != len(model.layers) or any(st is None for st in stores):
+            raise RuntimeError("GraphedDecoder needs the native caches of every layer (use_triton=True on a GPU)")
+        lengths = {st.length for st in stores}
+        if len(lengths) != 1:
+            raise RuntimeError("the layer caches disagree about their length")
+        self.length = lengths.pop()
+        self.stores = [st if st.capacity >= max_len else st.grown(max_len) for st in stores]
+        self.model = model
+        device = self.stores[0].buffers[0].device
+        batch = self.stores[0].buffers[0].shape[0]
+        self.capacity = min(st.capacity for st in self.stores)
+        # while warming up and capturing, the count is out of range for every layer: such a step writes nothing
+        self.t_device = torch.full((1,), max(st.capacity for st in self.stores), dtype=torch.int32, device=device)
+        self.token = torch.zeros((batch, 1), dtype=torch.long, device=device)
+        side = torch.cuda.Stream(device=device)
+        side.wait_stream(torch.cuda.current_stream(device))
+        with torch.cuda.stream(side), torch.no_grad():
+            for _ in range(2):   # library handles and workspaces are created outside the capture
+                self._step()
+        torch.cuda.current_stream(device).wait_stream(side)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph), torch.no_grad():
+            self.logits = self._step()
+            self.t_device += 1
+        self.t_device.fill_(self.length)
+        self.signature = self._signature()
+
+    def _signature(self):
+        """What the captured graph has baked in: the addresses of the weights it reads."""
+        return tuple(p.data_ptr() for p in self.model.parameters())
+
+    def fits(self, caches, max_len: int) -> bool:
+        """True if `load(caches)` can reuse this graph for a generation of up to max_len rows."""
+        first = getattr(caches[0], "_store", None)
+        mine = self.stores[0].buffers[0]
+        return (first is not None and max_len <= self.capacity and self.signature == self._signature()
+                and first.buffers[0].shape[:2] == mine.shape[:2] and first.buffers[0].shape[3] == mine.shape[3]
+                and first.buffers[0].dtype == mine.dtype and first.buffers[0].device == mine.device)
+
+    def load(self, caches):
+        """Restarts the decoder from the caches of a new prefill: their rows are copied into the
+        buffers the graph was captured on (the graph holds those addresses)."""
+        stores = [getattr(c, "_store", None) for c in caches]
+        if len(stores) != len(self.stores) or any(st is None for st in stores):
+            raise RuntimeError("GraphedDecoder.load needs the native caches of every layer")
+        length = stores[0].length
+        if any(st.length != length for st in stores) or length > self.capacity:
+            raise RuntimeError("these caches do not fit the buffers the graph was captured on")
+        for mine, theirs in zip(self.stores, stores):
+            for dst, src in zip(mine.buffers, theirs.buffers):
+                dst[:, :, :length].copy_(src[:, :, :length])
+        self.length = length
+        self.t_device.fill_(length)
+
+    def _step(self):
+        model = self.model
+        h = model.token_emb(self.token)
+        for (attention, feed_forward), store in zip(model.layers, self.stores):
+            h = h + attention.graph_step(h, store, self.t_device)
+            h = h + feed_forward(h)
+        return model.to_logits(model.final_norm(h))
+
+    def step(self, token):
+        """Feeds `token` (batch, 1) and returns the logits (batch, 1, num_tokens) of the next
+        position: a view of the graph's output buffer, overwritten by the next call."""
+        if self.length >= self.capacity:
+            raise RuntimeError(f"the graph was captured for caches of {self.capacity} rows")
+        self.token.copy_(token)
+        self.graph.replay()
+        self.length += 1
+        return self.logits
+
+    def caches(self):
+        """The per-layer caches as they stand after the steps replayed so far."""
+        for st in self.stores:
+            st.length = self.length
+        return [st.as_cache() for st in self.stores]
+
+
 class CastleLM(nn.Module):
     def __init__(self, *, num_tokens, dim, depth, max_seq_len=512, dim_head=64, heads=8, use_triton=True,
                  rotary_emb=True, prenorm=True, tie_embedding=False):
@@ -89,20 +181,48 @@ class CastleLM(nn.Module):
             return F.cross_entropy(logits.transpose(1, 2), target)
         return (logits, next_cache) if return_next_cache else logits
 
+    def _decoder_for(self, cache, max_len):
+        """A GraphedDecoder positioned on `cache`: the one kept from an earlier call when its graph
+        still fits (same weights, batch, type; enough rows), else a newly captured one."""
+        kept = self.__dict__.get("_kept_decoder")
+        if kept is not None and kept.fits(cache, max_len):
+            kept.load(cache)
+            return kept
+        decoder = GraphedDecoder(self, cache, max_len)
+        self.__dict__["_kept_decoder"] = decoder   # not a module attribute: never part of the state
+        return decoder
+
+    def _native_on_gpu(self, device) -> bool:
+        return device.type == "cuda" and all(attention.use_triton for attention, _ in self.layers)
+
     @torch.no_grad()
-    def sample(self, prompt, seq_len, temperature=1.0, filter_thres=0.9, generator=None):
+    def sample(self, prompt, seq_len, temperature=1.0, filter_thres=0.9, generator=None, graph=None):
         """Extends `prompt` (batch, p) to `seq_len` tokens and returns the seq_len - p new ones.
         The prompt goes through the parallel path once; afterwards each step feeds the last token
-        and the per-layer caches.  temperature = 0 picks the arg-max (no noise)."""
+        and the per-layer caches.  temperature = 0 picks the arg-max (no noise).
+        graph: replay the token steps as one captured HIP graph (`GraphedDecoder`).  None = when
+        the model runs the native kernels on a GPU and more than a few steps follow; True insists."""
         prompt_len = prompt.shape[-1]
-        out, cache = prompt, None
-        for _ in range(max(0, seq_len - prompt_len)):
-            step_input = out if cache is None else out[:, -1:]
-            logits, cache = self.forward(step_input, cache=cache, return_next_cache=True)
+        steps = max(0, seq_len - prompt_len)
+        if graph is None:
+            graph = self._native_on_gpu(prompt.device) and steps > 8
+        elif graph and not self._native_on_gpu(prompt.device):
+            raise RuntimeError("graph=True needs the native kernels on a GPU")
+
+        def pick(logits):
             logits = top_k(logits[:, -1].float(), thres=filter_thres)
             if temperature == 0:
-                token = logits.argmax(dim=-1, keepdim=True)
+                return logits.argmax(dim=-1, keepdim=True)
+            return gumbel_sample(logits, temperature=temperature, generator=generator)
+
+        out, cache, decoder = prompt, None, None
+        for _ in range(steps):
+            if decoder is not None:
+                logits = decoder.step(out[:, -1:])
             else:
-                token = gumbel_sample(logits, temperature=temperature, generator=generator)
-            out = torch.cat((out, token), dim=-1)
+                step_input = out if cache is None else out[:, -1:]
+                logits, cache = self.forward(step_input, cache=cache, return_next_cache=True)
+                if graph:
+                    decoder = self._decoder_for(cache, seq_len)
+            out = torch.cat((out, pick(logits)), dim=-1)
         return out[..., prompt_len:]

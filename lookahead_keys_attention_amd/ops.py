@@ -201,23 +201,37 @@ def castle_rope_hip(x, out, first_position=0):
 
 
 @torch.no_grad()
-def castle_decode_step_packed(cache_views, capacity, t, proj, heads, scale, out, workspace, rotary=False):
+def castle_decode_step_packed(cache_views, capacity, t, proj, heads, scale, out, workspace, rotary=False,
+                              t_device=None):
     """The cached step for a fused projection: `proj` is the contiguous (B, 1, 6*H*d) output of the
     layer's projection for the new token (order qu, ku, vu, qc, kc, vc), `cache_views` the four
     castle_view4 of the (B, H, capacity, d) cache buffers (built once per buffer set), `out` a
-    (B, 1, H, d) tensor.  Same kernels as castle_decode_step_hip, without per-call view building."""
+    (B, 1, H, d) tensor.  Same kernels as castle_decode_step_hip, without per-call view building.
+
+    With `t_device` (a one-element int32 GPU tensor) the kernels read the row count from it and `t`
+    is ignored: the launch is then identical for every step, which is what a captured HIP graph of
+    the step needs (the caller advances the counter, e.g. with an in-graph `t_device += 1`)."""
     B, n, width = proj.shape
     d = width // (6 * heads)
     if n != 1 or not proj.is_contiguous() or proj.data_ptr() % 16 != 0 or not proj.is_cuda:
         raise ValueError("castle_decode_step_packed needs a contiguous, 16-byte aligned (B, 1, 6*H*d) GPU tensor")
-    if not (0 <= t < capacity):
-        raise ValueError(f"cache capacity {capacity} cannot take row {t}")
     es, base, part = proj.element_size(), proj.data_ptr(), heads * d
     qu, ku, vu, qc, kc, vc = (N.View4(base + i * part * es, width, d, width) for i in range(6))
+    vout = N.View4(out.data_ptr(), heads * d, d, heads * d)
+    flags = N.FLAG_ROTARY if rotary else 0
     with torch.cuda.device(proj.device):
-        rc = N.lib().castle_decode_step(*cache_views, int(t), qc, kc, vc, qu, ku, vu, B, heads, d,
-                                        N.dtype_code(proj.dtype), float(scale), N.FLAG_ROTARY if rotary else 0,
-                                        N.View4(out.data_ptr(), heads * d, d, heads * d),
-                                        workspace.data_ptr(), workspace.numel(), N.stream_ptr(proj.device))
+        if t_device is None:
+            if not (0 <= t < capacity):
+                raise ValueError(f"cache capacity {capacity} cannot take row {t}")
+            rc = N.lib().castle_decode_step(*cache_views, int(t), qc, kc, vc, qu, ku, vu, B, heads, d,
+                                            N.dtype_code(proj.dtype), float(scale), flags, vout,
+                                            workspace.data_ptr(), workspace.numel(), N.stream_ptr(proj.device))
+        else:
+            if t_device.dtype != torch.int32 or t_device.numel() != 1 or t_device.device != proj.device:
+                raise ValueError("t_device must be a one-element int32 tensor on the GPU of the step")
+            rc = N.lib().castle_decode_step_device_count(
+                *cache_views, t_device.data_ptr(), int(capacity), qc, kc, vc, qu, ku, vu, B, heads, d,
+                N.dtype_code(proj.dtype), float(scale), flags, vout,
+                workspace.data_ptr(), workspace.numel(), N.stream_ptr(proj.device))
     N.check(rc, "castle_decode_step")
     return out

@@ -9,7 +9,7 @@ import math
 import pytest
 import torch
 
-from lookahead_keys_attention_amd.lm import CastleLM, gumbel_sample, top_k
+from lookahead_keys_attention_amd.lm import CastleLM, GraphedDecoder, gumbel_sample, top_k
 from oracle import castle_oracle as O
 
 VOCAB = 256
@@ -135,13 +135,15 @@ def test_native_model_matches_oracle_forward_and_backward():
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("graph", [False, True])
 @pytest.mark.parametrize("rotary", [False, True])
-def test_native_sampler_follows_the_parallel_logits(rotary):
-    """Greedy generation through HIP prefill + cached decode steps across layers: every token it
-    picks must be (within rounding) the arg-max of the logits a full parallel pass assigns."""
+def test_native_sampler_follows_the_parallel_logits(rotary, graph):
+    """Greedy generation through HIP prefill + cached decode steps across layers (step by step, or
+    as replays of one captured graph): every token it picks must be (within rounding) the arg-max
+    of the logits a full parallel pass assigns."""
     model = make_lm(depth=3, dim=128, heads=2, dim_head=64, rotary=rotary, native=True).cuda()
     prompt = tokens(2, 37)
-    new = model.sample(prompt.cuda(), seq_len=37 + 20, temperature=0.0).cpu()
+    new = model.sample(prompt.cuda(), seq_len=37 + 20, temperature=0.0, graph=graph).cpu()
     assert new.shape == (2, 20)
     seq = torch.cat((prompt, new), dim=-1)
     if rotary:      # no oracle for rotary: the product's dense formulation on the CPU is the comparison
@@ -152,6 +154,83 @@ def test_native_sampler_follows_the_parallel_logits(rotary):
         ref = O.lm_forward(seq, params_of(model), 2, 3)
     at_pick = ref[:, 36:-1].gather(-1, new.unsqueeze(-1)).squeeze(-1)
     assert torch.all(ref[:, 36:-1].max(-1).values - at_pick <= 2e-3)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_graphed_decode_replays_match_eager_steps(dtype):
+    """Every replay of the captured step is compared with the eager step on a second set of caches,
+    with that eager work (and a synchronisation) between the replays; afterwards both cache sets
+    must hold the same rows."""
+    model = make_lm(depth=3, dim=128, heads=2, dim_head=64, rotary=True, native=True).cuda().to(dtype)
+    x = tokens(2, 60).cuda()
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    with torch.no_grad():
+        _, eager_cache = model(x[:, :20], return_next_cache=True)
+        _, graph_cache = model(x[:, :20], return_next_cache=True)
+        decoder = GraphedDecoder(model, graph_cache, max_len=60)
+        for t in range(20, 60):
+            want, eager_cache = model(x[:, t:t + 1], cache=eager_cache, return_next_cache=True)
+            got = decoder.step(x[:, t:t + 1])
+            torch.cuda.synchronize()
+            assert (got.float() - want.float()).abs().max() <= tol * max(want.float().abs().max().item(), 1.0), t
+        for layer_eager, layer_graph in zip(eager_cache, decoder.caches()):
+            for a, b in zip(layer_eager, layer_graph):
+                assert a.shape == b.shape
+                assert (a.float() - b.float()).abs().max() <= tol * max(a.float().abs().max().item(), 1.0)
+        decoder.length = decoder.capacity   # as if the caches the graph was captured for were full
+        with pytest.raises(RuntimeError):
+            decoder.step(x[:, :1])
+
+
+@pytest.mark.gpu
+def test_sampler_reuses_its_captured_graph_for_a_new_prompt():
+    model = make_lm(depth=2, dim=128, heads=2, dim_head=64, rotary=True, native=True).cuda()
+    first = model.sample(tokens(2, 30, seed=3).cuda(), seq_len=50, temperature=0.0, graph=True)
+    kept = model._kept_decoder
+    for seed, n in ((4, 30), (5, 17)):   # same graph, other prompts (also a shorter one)
+        prompt = tokens(2, n, seed=seed).cuda()
+        again = model.sample(prompt, seq_len=n + 20, temperature=0.0, graph=True)
+        assert model._kept_decoder is kept
+        eager = model.sample(prompt, seq_len=n + 20, temperature=0.0, graph=False)
+        assert torch.equal(again, eager)
+    assert first.shape == (2, 20)
+    with torch.no_grad():   # new weights (other addresses): the kept graph must not be used again
+        model.to_logits.weight = torch.nn.Parameter(model.to_logits.weight.clone())
+    model.sample(tokens(2, 30, seed=3).cuda(), seq_len=50, temperature=0.0, graph=True)
+    assert model._kept_decoder is not kept
+
+
+@pytest.mark.gpu
+def test_decode_step_with_an_out_of_range_device_count_writes_nothing():
+    from lookahead_keys_attention_amd import ops
+    from lookahead_keys_attention_amd.castle import _CacheStore
+
+    torch.manual_seed(0)
+    B, H, d, cap = 2, 2, 64, 48
+    store = _CacheStore(B, H, d, cap, torch.bfloat16, torch.device("cuda"))
+    for buf in store.buffers:
+        buf.copy_(torch.randn(buf.shape, device="cuda"))
+    before = [buf.clone() for buf in store.buffers]
+    proj = torch.randn(B, 1, 6 * H * d, device="cuda", dtype=torch.bfloat16)
+    out = torch.full((B, 1, H, d), 7.0, device="cuda", dtype=torch.bfloat16)
+    for count in (cap, cap + 5, -1):
+        t_device = torch.tensor([count], dtype=torch.int32, device="cuda")
+        ops.castle_decode_step_packed(store.views, cap, 0, proj, H, d ** -0.5, out, store.workspace, t_device=t_device)
+    torch.cuda.synchronize()
+    assert all(torch.equal(a, b) for a, b in zip(before, store.buffers))
+    assert torch.all(out == 7.0)
+    # and a count inside the range gives what the host-side count gives
+    t_device = torch.tensor([17], dtype=torch.int32, device="cuda")
+    other = _CacheStore(B, H, d, cap, torch.bfloat16, torch.device("cuda"))
+    for dst, src in zip(other.buffers, before):
+        dst.copy_(src)
+    out_host = torch.empty_like(out)
+    ops.castle_decode_step_packed(store.views, cap, 0, proj, H, d ** -0.5, out, store.workspace, t_device=t_device)
+    ops.castle_decode_step_packed(other.views, cap, 17, proj, H, d ** -0.5, out_host, other.workspace)
+    torch.cuda.synchronize()
+    assert torch.equal(out, out_host)
+    assert all(torch.equal(a[:, :, :18], b[:, :, :18]) for a, b in zip(store.buffers, other.buffers))
 
 
 @pytest.mark.gpu
