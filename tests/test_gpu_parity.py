@@ -193,7 +193,9 @@ def test_packed_operator_equals_unpacked(dtype):
 
 
 DEC_CASES = [(2, 2, 0, 40, 64, torch.float32), (2, 2, 100, 30, 64, torch.float32), (1, 3, 300, 20, 16, torch.float32),
-             (1, 2, 70, 10, 32, torch.float32), (2, 2, 200, 20, 64, torch.bfloat16), (1, 2, 130, 10, 128, torch.bfloat16)]
+             (1, 2, 70, 10, 32, torch.float32), (2, 2, 200, 20, 64, torch.bfloat16), (1, 2, 130, 10, 128, torch.bfloat16),
+             # many row splits per (b, h): 24 (three batches of the merge) and the cap of 64
+             (1, 2, 1500, 4, 64, torch.float32), (1, 1, 4200, 3, 32, torch.bfloat16)]
 
 
 @pytest.mark.parametrize("B,Hh,t0,steps,d,dtype", DEC_CASES)
