@@ -46,7 +46,7 @@ int64_t max_score_tile_bytes() {
 struct Geometry {
   int Lp, nblk;
   int64_t lse_bytes, tblk_bytes, snap_bytes, mat_bytes, op_bytes;
-  int64_t off_lse, off_t, off_tt, off_snap, off_ops, total;
+  int64_t off_lse, off_t, off_tt, off_ttx, off_snap, off_ops, total;
 };
 
 Geometry geometry(int B, int H, int L, int d, int es) {
@@ -63,7 +63,8 @@ Geometry geometry(int B, int H, int L, int d, int es) {
   g.off_lse = 0;
   g.off_t = g.off_lse + g.lse_bytes;
   g.off_tt = g.off_t + g.tblk_bytes;
-  g.off_snap = g.off_tt + g.tblk_bytes;
+  g.off_ttx = g.off_tt + g.tblk_bytes;
+  g.off_snap = g.off_ttx + g.tblk_bytes;
   g.op_bytes = align_up(BH * g.Lp * d * es, 256);   // one operand in the compute type, padded to Lp rows
   g.off_ops = g.off_snap + g.snap_bytes;
   g.total = g.off_ops + 6 * g.op_bytes;
@@ -105,6 +106,7 @@ castle::FwdWorkspace carve(void* base, const Geometry& g) {
   w.lse = reinterpret_cast<float*>(p + g.off_lse);
   w.t_blk = p + g.off_t;
   w.tt_blk = p + g.off_tt;
+  w.ttx_blk = p + g.off_ttx;
   w.usnap = p + g.off_snap;
   w.qc_p = p + g.off_ops;
   w.kc_p = p + g.off_ops + g.op_bytes;

@@ -654,7 +654,9 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_key2_kernel(BwdArgs a) {
     __syncthreads();   // 0
     for (int I = Ilast; I >= I0; --I) {
       const bool active = I >= Iw;
-      if (active && I <= a.s.nblk - 2)   // reverse state as of block I
+      // reverse state as of block I; the tile-consuming query kernel only reads those behind a
+      // pair of blocks (odd I), the recomputing one all of them
+      if (active && I <= a.s.nblk - 2 && (a.ds_mat == nullptr || (I & 1)))
         store_snap_tile<T, HD, NT>(gsnap + (gsnap_off(I) + kw0) * HD, G, c, g);
       __syncthreads();   // 1
       if (I < Ilast && I + 1 >= Iw) CASTLE_BK2_DQU(I + 1);   // finish the previous block
@@ -1073,11 +1075,12 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
 //   row = source j:  dA = dSu^T T' + G' Vu^T,  dZ = dA A (1 - A),  dKu += dZ^T Qu,  dVu += A^T G'
 template <typename T> constexpr int kLdD = 128 + 8;   // dS / dSu tiles [key][128 queries]
 template <typename T> constexpr int kLdA = kCK + 8;   // gate tile [128 sources][key]
+template <typename T> constexpr int kLdT2 = 128 + 4;  // dT of the row pair [128 queries][128 sources]
 template <typename T, int HD> constexpr int bwd_query2_lds_bytes() {
-  int b = 6 * a16((int)sizeof(T) * kCK * lds_ld<T>(HD));          // kc, qu, ub[2], g[2]
+  int b = 4 * a16((int)sizeof(T) * kCK * lds_ld<T>(HD));          // kc, qu, ub, g
   b += a16((int)sizeof(T) * 128 * kLdA<T>);                       // A^T [j][k]
   b += 2 * a16((int)sizeof(T) * kCK * kLdD<T>);                   // dS, dSu [k][i]
-  int e = 4 * a16((int)sizeof(T) * kNB * lds_ld<T>(HD)) + 2 * a16((int)sizeof(T) * kNB * lds_ld_chain<T>(kNB));
+  int e = 2 * a16((int)sizeof(T) * 128 * lds_ld<T>(HD)) + a16((int)sizeof(T) * 128 * kLdT2<T>);
   return b > e ? b : e;
 }
 
@@ -1099,39 +1102,42 @@ struct TileStage {
   }
 };
 
-// 512 threads, two wave roles over the same 128 rows (wave pair (w, w + 4) owns rows 32 w ..):
+// 512 threads, two wave roles over the same 128 rows = one PAIR of 64-row blocks (2 qb, 2 qb + 1);
+// wave pair (w, w + 4) owns rows 32 w ..:
 //   waves 0-3, row = lookahead source j:  gate A, dA, dZ, dKu, dVu
 //   waves 4-7, row = query i:             dQc, dT
 // Keys are streamed in chunks of 32 (three barriers per chunk); two waves share a SIMD.
+// The pair is handled as ONE block with respect to the two states: the lookahead state U is the
+// one at the start of the pair and the reverse state G' the one behind the pair (one snapshot tile
+// of each per chunk instead of two), and what the states of the inner block boundary would have
+// carried goes through the pair's own 128 x 128 quarter-filled dT / T' instead:
+//   dA[k,j]  = sum_{i in pair, i >= j} dSu[i,k] T'[i,j] + G'[k] . vu_j
+//   dQc[i]  += sum_k dSu[i,k] U[k]  (keys before the pair)  + sum_{j in pair, j <= i} dT[i,j] vu_j
+//   dVu[j]  += sum_k A[k,j] G'[k] + sum_{i in pair, i >= j} dT[i,j] qc'_i,   dT[i,j] = sum_k dSu[i,k] A[k,j]
 template <typename T, typename TI, int HD>
 __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) {
   static_assert(sizeof(T) == 2 && HD <= 64 && kCK == 32, "tile consumer: 16-bit operands, d <= 64");
   constexpr int KS = HD / 16;
   constexpr int HDP = HD < 32 ? 32 : HD;
   constexpr int NT = HDP / 32;
-  constexpr int BT = kNB / 32;
-  constexpr int TS = kNB / 16;   // 16-deep steps across a block
   constexpr int QB = 128;
-  constexpr int LDK = lds_ld<T>(HD), LDT = lds_ld_chain<T>(kNB), LDA = kLdA<T>, LDD = kLdD<T>;
+  constexpr int PT = QB / 32;    // 32-row tiles across the pair
+  constexpr int PS = QB / 16;    // 16-deep steps across the pair
+  constexpr int LDK = lds_ld<T>(HD), LDT = kLdT2<T>, LDA = kLdA<T>, LDD = kLdD<T>;
 
   Carver cv{castle_smem};
   T* s_kc = cv.take<T>(kCK * LDK);
   T* s_qu = cv.take<T>(kCK * LDK);
-  T* s_ub0 = cv.take<T>(kCK * LDK);
-  T* s_ub1 = cv.take<T>(kCK * LDK);
-  T* s_g0 = cv.take<T>(kCK * LDK);
-  T* s_g1 = cv.take<T>(kCK * LDK);
+  T* s_ub = cv.take<T>(kCK * LDK);   // lookahead state at the start of the pair
+  T* s_g = cv.take<T>(kCK * LDK);    // reverse state behind the pair
   T* s_at = cv.take<T>(QB * LDA);    // gate, [source j][key k]
   T* s_ds = cv.take<T>(kCK * LDD);   // dS,  [key k][query i]
   T* s_dsu = cv.take<T>(kCK * LDD);  // dSu, [key k][query i]
   // the epilogue reuses the same memory
   Carver ce{castle_smem};
-  T* e_vu0 = ce.take<T>(kNB * LDK);
-  T* e_vu1 = ce.take<T>(kNB * LDK);
-  T* e_qc0 = ce.take<T>(kNB * LDK);
-  T* e_qc1 = ce.take<T>(kNB * LDK);
-  T* e_dt0 = ce.take<T>(kNB * LDT);   // dT, [query i][source j] (block local)
-  T* e_dt1 = ce.take<T>(kNB * LDT);
+  T* e_vu = ce.take<T>(QB * LDK);
+  T* e_qc = ce.take<T>(QB * LDK);
+  T* e_dt = ce.take<T>(QB * LDT);    // dT, [query i][source j] (pair local)
 
   int rank, bh;
   work_item(a.s.B * a.s.H, rank, bh);
@@ -1143,22 +1149,12 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
   const int tid = threadIdx.x & (kThreads - 1);   // thread index inside the role
   const int L = a.s.L;
   const float c0 = a.s.scale, c1 = a.s.scale * kLog2e;
-  const int i0w = qb * QB + 32 * pw;
-  const int i = i0w + c;                      // this lane's row
-  const int Ifirst = (qb * QB) / kNB;
-  const int Iw = i0w / kNB;
-  const int qw = Iw - Ifirst;                 // which of the workgroup's blocks
   const int jw = 32 * pw;                     // rows of this wave pair inside the 128-row exchange tiles
-  const int cb = (jw / kNB) * kNB;            // first row of its block there
-  const int lw = jw % kNB;                    // offset of the wave pair inside its block
-  const int ifirst = lw / 16;                 // first step covering queries i >= j
-  const bool has_g = Iw <= a.s.nblk - 2;
-  const T* s_ubw = qw == 0 ? s_ub0 : s_ub1;
-  const T* s_gw = qw == 0 ? s_g0 : s_g1;
-  const T* e_vuw = qw == 0 ? e_vu0 : e_vu1;
-  const T* e_qcw = qw == 0 ? e_qc0 : e_qc1;
-  T* e_dtw = qw == 0 ? e_dt0 : e_dt1;
-  const int blk0 = Ifirst, blk1 = Ifirst + 1;
+  const int i0w = qb * QB + jw;
+  const int i = i0w + c;                      // this lane's row
+  const int blk0 = 2 * qb, blk1 = 2 * qb + 1;
+  const int sfirst = jw / 16;                 // first step covering queries i >= j
+  const bool has_g = blk1 <= a.s.nblk - 2;    // a reverse state exists behind the pair
 
   const T* qc = prep_ptr<T>(a.ws.qc_p, bh, a.s.Lp, HD);
   const T* vu = prep_ptr<T>(a.ws.vu_p, bh, a.s.Lp, HD);
@@ -1176,26 +1172,33 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
     const T* qu = prep_ptr<T>(a.ws.qu_p, bh, a.s.Lp, HD);
     const T* ku = prep_ptr<T>(a.ws.ku_p, bh, a.s.Lp, HD);
     const T* ttb = reinterpret_cast<const T*>(a.ws.tt_blk) + (int64_t)bh * a.s.Lp * kNB;
-    frag<T> fku[KS], fvu[KS], ftt[TS];
+    const T* ttx = reinterpret_cast<const T*>(a.ws.ttx_blk) + (int64_t)bh * a.s.Lp * kNB;
+    // T'^T rows of this wave across the queries of the pair: its own block from tt_blk, and for a
+    // wave of the first block the second block from the cross quarter
+    frag<T> fku[KS], fvu[KS], ftt[PS];
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
       fku[s] = ldg_nat_scaled<T, T>(ku, HD, i, 16 * s + 8 * g, true, -c1);
       fvu[s] = ldg_nat<T>(vu, HD, i, 16 * s + 8 * g, true);
     }
 #pragma unroll
-    for (int s = 0; s < TS; ++s) ftt[s] = ldg_nat<T>(ttb, kNB, i, 16 * s + 8 * g, s >= ifirst);
+    for (int s = 0; s < PS; ++s) {
+      const bool own = (s < PS / 2) == (pw < 2);   // queries of step s lie in this wave's own block
+      const T* src = own ? ttb : ttx;
+      ftt[s] = ldg_nat<T>(src, kNB, i, 16 * (s % (PS / 2)) + 8 * g, s >= sfirst);
+    }
     acc_t dku[NT], dvu[NT];   // [n rows, j lanes]
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) { zero(dku[nt]); zero(dvu[nt]); }
 
-    // this role stages kc, qu and the lookahead state of the first block
+    // this role stages kc, qu and the lookahead state
     RowStage<T, T, kCK, HD> pkc, pqu;
-    SnapStage<T, kCK, HD> pu0;
+    SnapStage<T, kCK, HD> pu;
 #define CASTLE_BQ2_LOAD_A(K0)                                                            \
   do {                                                                                   \
     pkc.load_flat(kc + (int64_t)(K0) * HD, tid);                                         \
     pqu.load_flat(qu + (int64_t)(K0) * HD, tid);                                         \
-    if ((K0) / kNB < blk0) pu0.load(usnap + (usnap_off(blk0) + (K0)) * HD, tid);         \
+    if ((K0) / kNB < blk0) pu.load(usnap + (usnap_off(blk0) + (K0)) * HD, tid);          \
     pds.load(dsm + (int64_t)((K0) / 32) * tile_row);                                     \
     pdsu.load(dsum + (int64_t)((K0) / 32) * tile_row);                                   \
   } while (0)
@@ -1205,7 +1208,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
       __syncthreads();   // 1: tiles free
       pkc.store(s_kc, LDK, tid);
       pqu.store(s_qu, LDK, tid);
-      if (Kb < blk0) pu0.store(s_ub0, LDK, tid);
+      if (Kb < blk0) pu.store(s_ub, LDK, tid);
       pds.store(s_ds);
       pdsu.store(s_dsu);
       if (k0 + kCK < kend) CASTLE_BQ2_LOAD_A(k0 + kCK);   // in flight while this chunk is processed
@@ -1231,38 +1234,42 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
             if (i <= k0 + acc_row(r, g)) aK[r] = 0.f;
         }
       }
-      if (Kb <= Iw) {   // a wave the chunk has passed still owes zeros to the other rows of its block
+      // a wave the chunk has passed still owes zeros: the later rows of the pair read its rows
 #pragma unroll
-        for (int q = 0; q < 4; ++q) st4<T>(s_at + (jw + c) * LDA + 8 * q + 4 * g, pack4<T>(aK, q));
-      }
+      for (int q = 0; q < 4; ++q) st4<T>(s_at + (jw + c) * LDA + 8 * q + 4 * g, pack4<T>(aK, q));
       __syncthreads();   // 3: gate shared
       if (!live) continue;
       acc_t dA;
       zero(dA);
-      frag<T> oqt[2][NT], ogt[2][NT];
       {
-        frag<T> ods[TS], og[KS];
+        frag<T> og[KS];
 #pragma unroll
-        for (int s = 0; s < TS; ++s) ods[s] = ld_nat<T>(s_dsu, LDD, c, cb + 16 * s + 8 * g);
+        for (int s = 0; s < KS; ++s) og[s] = has_g ? ld_nat<T>(s_g, LDK, c, 16 * s + 8 * g) : zero_frag<T>();
 #pragma unroll
-        for (int s = 0; s < KS; ++s) og[s] = has_g ? ld_nat<T>(s_gw, LDK, c, 16 * s + 8 * g) : zero_frag<T>();
+        for (int half = 0; half < 2; ++half) {   // two batches keep the operand fragments in registers
+          frag<T> ods[PS / 2];
 #pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2)
+          for (int u = 0; u < PS / 2; ++u) ods[u] = ld_nat<T>(s_dsu, LDD, c, 16 * (half * (PS / 2) + u) + 8 * g);
+          __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-          for (int nt = 0; nt < NT; ++nt) {
-            oqt[s2][nt] = ld_free<T, true>(s_qu, LDK, 32 * nt, HD, 16 * s2, c, g);
-            ogt[s2][nt] = has_g ? ld_free<T, true>(s_gw, LDK, 32 * nt, HD, 16 * s2, c, g) : zero_frag<T>();
-          }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int s = 0; s < TS; ++s)
-          if (s >= ifirst) mma(dA, ods[s], ftt[s]);
+          for (int u = 0; u < PS / 2; ++u)
+            if (half * (PS / 2) + u >= sfirst) mma(dA, ods[u], ftt[half * (PS / 2) + u]);
+        }
 #pragma unroll
         for (int s = 0; s < KS; ++s) mma(dA, og[s], fvu[s]);   // og is zero where no reverse state exists
       }
       acc_t dz;
 #pragma unroll
       for (int r = 0; r < 16; ++r) dz[r] = dA[r] * aK[r] * (1.f - aK[r]);
+      frag<T> oqt[2][NT], ogt[2][NT];
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          oqt[s2][nt] = ld_free<T, true>(s_qu, LDK, 32 * nt, HD, 16 * s2, c, g);
+          ogt[s2][nt] = has_g ? ld_free<T, true>(s_g, LDK, 32 * nt, HD, 16 * s2, c, g) : zero_frag<T>();
+        }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
         const frag<T> fdz = chain<T>(dz, s2), fa = chain<T>(aK, s2);
@@ -1274,24 +1281,22 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
       }
     }
 #undef CASTLE_BQ2_LOAD_A
-    // ---- epilogue: in-block term dvu += dT^T Qc' --------------------------------------------
+    // ---- epilogue: in-pair term dvu += dT^T Qc' ----------------------------------------------
     __syncthreads();   // e1: chunk tiles dead
     {
-      RowStage<T, T, kNB, HD, 2 * kThreads> st;
-      st.load(vu, HD, (int64_t)blk0 * kNB, kNoRowLimit); st.store(e_vu0, LDK);
-      st.load(vu, HD, (int64_t)blk1 * kNB, kNoRowLimit); st.store(e_vu1, LDK);
-      st.load(qc, HD, (int64_t)blk0 * kNB, kNoRowLimit); st.store(e_qc0, LDK);
-      st.load(qc, HD, (int64_t)blk1 * kNB, kNoRowLimit); st.store(e_qc1, LDK);
+      RowStage<T, T, QB, HD, 2 * kThreads> st;
+      st.load_flat(vu + (int64_t)qb * QB * HD); st.store(e_vu, LDK);
+      st.load_flat(qc + (int64_t)qb * QB * HD); st.store(e_qc, LDK);
     }
     __syncthreads();   // e2: epilogue tiles and dT shared
 #pragma unroll
-    for (int s = 0; s < TS; ++s) {
-      if (s < ifirst) continue;
-      // B operand: source j = lw + c on lanes, queries i = 16 s .. in natural order, from dT[i][j]
-      const frag<T> fdt = ld_free<T, false>(e_dtw, LDT, lw, kNB, 16 * s, c, g);
+    for (int s = 0; s < PS; ++s) {
+      if (s < sfirst) continue;
+      // B operand: source j = jw + c on lanes, queries i = 16 s .. in natural order, from dT[i][j]
+      const frag<T> fdt = ld_free<T, false>(e_dt, LDT, jw, QB, 16 * s, c, g);
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt)
-        mma(dvu[nt], ld_free<T, false>(e_qcw, LDK, 32 * nt, HD, 16 * s, c, g), fdt);
+        mma(dvu[nt], ld_free<T, false>(e_qc, LDK, 32 * nt, HD, 16 * s, c, g), fdt);
     }
     if (i < L) {
       store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dku, b, h) + (int64_t)i * a.dku.sl, dku, c0 * kLn2, g, a.s.rotary ? i : -1);
@@ -1299,19 +1304,16 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
     }
   } else {
     acc_t dqc[NT];     // [n rows, i lanes]
-    acc_t dtacc[BT];   // [j rows (block local), i lanes]
+    acc_t dtacc[PT];   // [j rows (pair local), i lanes]
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) zero(dqc[nt]);
 #pragma unroll
-    for (int jt = 0; jt < BT; ++jt) zero(dtacc[jt]);
-    // this role stages the lookahead state of the second block and both reverse states
-    SnapStage<T, kCK, HD> pu1, pg0, pg1;
+    for (int jt = 0; jt < PT; ++jt) zero(dtacc[jt]);
+    // this role stages the reverse state
+    SnapStage<T, kCK, HD> pg;
 #define CASTLE_BQ2_LOAD_B(K0)                                                                             \
   do {                                                                                                    \
-    const int kb_ = (K0) / kNB;                                                                           \
-    if (kb_ < blk1 && blk1 < a.s.nblk) pu1.load(usnap + (usnap_off(blk1) + (K0)) * HD, tid);              \
-    if (kb_ <= blk0 && blk0 <= a.s.nblk - 2) pg0.load(gsnap + (gsnap_off(blk0) + (K0)) * HD, tid);        \
-    if (kb_ <= blk1 && blk1 <= a.s.nblk - 2) pg1.load(gsnap + (gsnap_off(blk1) + (K0)) * HD, tid);        \
+    if (has_g) pg.load(gsnap + (gsnap_off(blk1) + (K0)) * HD, tid);                                       \
     pds.load(dsm + (int64_t)((K0) / 32) * tile_row);                                                      \
     pdsu.load(dsum + (int64_t)((K0) / 32) * tile_row);                                                    \
   } while (0)
@@ -1319,9 +1321,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
     for (int k0 = 0; k0 < kend; k0 += kCK) {
       const int Kb = k0 / kNB;
       __syncthreads();   // 1
-      if (Kb < blk1 && blk1 < a.s.nblk) pu1.store(s_ub1, LDK, tid);
-      if (Kb <= blk0 && blk0 <= a.s.nblk - 2) pg0.store(s_g0, LDK, tid);
-      if (Kb <= blk1 && blk1 <= a.s.nblk - 2) pg1.store(s_g1, LDK, tid);
+      if (has_g) pg.store(s_g, LDK, tid);
       pds.store(s_ds);
       pdsu.store(s_dsu);
       if (k0 + kCK < kend) CASTLE_BQ2_LOAD_B(k0 + kCK);
@@ -1337,7 +1337,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
 #pragma unroll
           for (int nt = 0; nt < NT; ++nt) {
             okt[s2][nt] = ld_free<T, false>(s_kc, LDK, 32 * nt, HD, 16 * s2, c, g);
-            out[s2][nt] = ld_free<T, false>(s_ubw, LDK, 32 * nt, HD, 16 * s2, c, g);
+            out[s2][nt] = ld_free<T, false>(s_ub, LDK, 32 * nt, HD, 16 * s2, c, g);
           }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -1346,54 +1346,53 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
 #pragma unroll
           for (int nt = 0; nt < NT; ++nt) {
             mma(dqc[nt], okt[s2][nt], bds[s2]);
-            if (Kb < Iw) mma(dqc[nt], out[s2][nt], bdsu[s2]);
+            if (Kb < blk0) mma(dqc[nt], out[s2][nt], bdsu[s2]);
           }
       }
       __syncthreads();   // 3
       if (!live) continue;
       {
-        frag<T> oat[2][BT];
+        frag<T> oat[2][PT];
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
-          for (int jt = 0; jt < BT; ++jt) oat[s2][jt] = ld_nat<T>(s_at, LDA, cb + 32 * jt + c, 16 * s2 + 8 * g);
+          for (int jt = 0; jt < PT; ++jt)
+            if (jt <= pw) oat[s2][jt] = ld_nat<T>(s_at, LDA, 32 * jt + c, 16 * s2 + 8 * g);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
-          for (int jt = 0; jt < BT; ++jt)
-            if (32 * jt < lw + 32) mma(dtacc[jt], oat[s2][jt], bdsu[s2]);
+          for (int jt = 0; jt < PT; ++jt)
+            if (jt <= pw) mma(dtacc[jt], oat[s2][jt], bdsu[s2]);
       }
     }
 #undef CASTLE_BQ2_LOAD_B
-    // ---- epilogue: dT = tril(dTacc):  dqc += dT Vu -------------------------------------------
+    // ---- epilogue: dT = tril(dTacc) over the pair:  dqc += dT Vu ------------------------------
     __syncthreads();   // e1
     {
-      RowStage<T, T, kNB, HD, 2 * kThreads> st;
-      st.load(vu, HD, (int64_t)blk0 * kNB, kNoRowLimit); st.store(e_vu0, LDK);
-      st.load(vu, HD, (int64_t)blk1 * kNB, kNoRowLimit); st.store(e_vu1, LDK);
-      st.load(qc, HD, (int64_t)blk0 * kNB, kNoRowLimit); st.store(e_qc0, LDK);
-      st.load(qc, HD, (int64_t)blk1 * kNB, kNoRowLimit); st.store(e_qc1, LDK);
+      RowStage<T, T, QB, HD, 2 * kThreads> st;
+      st.load_flat(vu + (int64_t)qb * QB * HD); st.store(e_vu, LDK);
+      st.load_flat(qc + (int64_t)qb * QB * HD); st.store(e_qc, LDK);
     }
     // dT^T[j rows, i lanes] masked to j <= i, shared as dT[i][j] for the source-side product
 #pragma unroll
-    for (int jt = 0; jt < BT; ++jt) {
+    for (int jt = 0; jt < PT; ++jt) {
 #pragma unroll
       for (int r = 0; r < 16; ++r)
-        if (32 * jt + acc_row(r, g) > lw + c) dtacc[jt][r] = 0.f;
+        if (32 * jt + acc_row(r, g) > jw + c) dtacc[jt][r] = 0.f;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) st4<T>(e_dtw + (lw + c) * LDT + 32 * jt + 8 * q + 4 * g, pack4<T>(dtacc[jt], q));
+      for (int q = 0; q < 4; ++q) st4<T>(e_dt + (jw + c) * LDT + 32 * jt + 8 * q + 4 * g, pack4<T>(dtacc[jt], q));
     }
     __syncthreads();   // e2
 #pragma unroll
-    for (int jt = 0; jt < BT; ++jt) {
-      if (32 * jt >= lw + 32) continue;
+    for (int jt = 0; jt < PT; ++jt) {
+      if (jt > pw) continue;
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
         const frag<T> fdt = chain<T>(dtacc[jt], s2);
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
-          mma(dqc[nt], ld_free<T, true>(e_vuw, LDK, 32 * nt, HD, 32 * jt + 16 * s2, c, g), fdt);
+          mma(dqc[nt], ld_free<T, true>(e_vu, LDK, 32 * nt, HD, 32 * jt + 16 * s2, c, g), fdt);
       }
     }
     if (i < L) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqc, b, h) + (int64_t)i * a.dqc.sl, dqc, c0, g, a.s.rotary ? i : -1);

@@ -120,6 +120,24 @@ __global__ __launch_bounds__(kThreads) void tqv_kernel(FwdArgs a) {
     for (int q = 0; q < 4; ++q)
       st4<T>(ttb + ((int64_t)I * kNB + jl) * kNB + 32 * it + 8 * q + 4 * g, pack4<T>(acc, q));
   }
+  // cross quarter of a pair of blocks: (Qc'_{I+1} Vu_I^T)^T for even I, no mask (every query is later)
+  if ((I & 1) == 0 && I + 1 < a.s.nblk) {
+    T* ttx = reinterpret_cast<T*>(a.ws.ttx_blk) + (int64_t)bh * a.s.Lp * kNB;
+    for (int t = wave_id(); t < TB * TB; t += kThreads / 64) {
+      const int it = t / TB, jt = t % TB;
+      const int64_t i = (int64_t)(I + 1) * kNB + 32 * it + c;
+      const int64_t j = (int64_t)I * kNB + 32 * jt + c;
+      acc_t acc;
+      zero(acc);
+#pragma unroll
+      for (int s = 0; s < KS; ++s)
+        mma(acc, ldg_nat<T>(qc, HD, i, 16 * s + 8 * g, true), ldg_nat<T>(vu, HD, j, 16 * s + 8 * g, true));
+      const int jl = 32 * jt + c;
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        st4<T>(ttx + ((int64_t)I * kNB + jl) * kNB + 32 * it + 8 * q + 4 * g, pack4<T>(acc, q));
+    }
+  }
 }
 
 // ---------------------------------------------------------------------------

@@ -22,6 +22,7 @@ struct CoreShape {
 struct FwdWorkspace {
   void* t_blk;    // [B*H][Lp][kNB]  T[i][j_local]  = tril(Qc_I Vu_I^T), unscaled
   void* tt_blk;   // [B*H][Lp][kNB]  T^T per block: [j][i_local]
+  void* ttx_blk;  // [B*H][Lp][kNB]  rows j of even blocks I: (Qc'_{I+1} Vu_I^T)^T [j][i_local of block I+1]; odd blocks unused
   void* usnap;    // [B*H][snap_rows(nblk)][d]  forward state at block starts
   float* lse;     // [B*H][Lp] natural-log softmax normaliser
   // The six operands in the compute type, each [B*H][Lp][d] contiguous, rows >= L zero
