@@ -1104,8 +1104,8 @@ struct TileStage {
 
 // 512 threads, two wave roles over the same 128 rows = one PAIR of 64-row blocks (2 qb, 2 qb + 1);
 // wave pair (w, w + 4) owns rows 32 w ..:
-//   waves 0-3, row = lookahead source j:  gate A, dA, dZ, dKu, dVu
-//   waves 4-7, row = query i:             dQc, dT
+//   waves 0-3, row = lookahead source j:  gate A, dA, dZ, dKu
+//   waves 4-7, row = query i: dQc, dT;  row = source j: dVu (gate read back from the shared tile)
 // Keys are streamed in chunks of 32 (three barriers per chunk); two waves share a SIMD.
 // The pair is handled as ONE block with respect to the two states: the lookahead state U is the
 // one at the start of the pair and the reverse state G' the one behind the pair (one snapshot tile
@@ -1187,9 +1187,9 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
       const T* src = own ? ttb : ttx;
       ftt[s] = ldg_nat<T>(src, kNB, i, 16 * (s % (PS / 2)) + 8 * g, s >= sfirst);
     }
-    acc_t dku[NT], dvu[NT];   // [n rows, j lanes]
+    acc_t dku[NT];   // [n rows, j lanes]
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) { zero(dku[nt]); zero(dvu[nt]); }
+    for (int nt = 0; nt < NT; ++nt) zero(dku[nt]);
 
     // this role stages kc, qu and the lookahead state
     RowStage<T, T, kCK, HD> pkc, pqu;
@@ -1239,8 +1239,10 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
       for (int q = 0; q < 4; ++q) st4<T>(s_at + (jw + c) * LDA + 8 * q + 4 * g, pack4<T>(aK, q));
       __syncthreads();   // 3: gate shared
       if (!live) continue;
-      acc_t dA;
+      // dA in two accumulators (two dependent MFMA chains instead of one of up to twelve)
+      acc_t dA, dA2;
       zero(dA);
+      zero(dA2);
       {
         frag<T> og[KS];
 #pragma unroll
@@ -1252,32 +1254,26 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
           for (int u = 0; u < PS / 2; ++u) ods[u] = ld_nat<T>(s_dsu, LDD, c, 16 * (half * (PS / 2) + u) + 8 * g);
           __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-          for (int u = 0; u < PS / 2; ++u)
+          for (int u = 0; u < PS / 2; ++u) {
             if (half * (PS / 2) + u >= sfirst) mma(dA, ods[u], ftt[half * (PS / 2) + u]);
+            if (half == 0 && u < KS) mma(dA2, og[u], fvu[u]);   // og is zero where no reverse state exists
+          }
         }
-#pragma unroll
-        for (int s = 0; s < KS; ++s) mma(dA, og[s], fvu[s]);   // og is zero where no reverse state exists
       }
       acc_t dz;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) dz[r] = dA[r] * aK[r] * (1.f - aK[r]);
-      frag<T> oqt[2][NT], ogt[2][NT];
+      for (int r = 0; r < 16; ++r) dz[r] = (dA[r] + dA2[r]) * aK[r] * (1.f - aK[r]);
+      frag<T> oqt[2][NT];
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-          oqt[s2][nt] = ld_free<T, true>(s_qu, LDK, 32 * nt, HD, 16 * s2, c, g);
-          ogt[s2][nt] = has_g ? ld_free<T, true>(s_g, LDK, 32 * nt, HD, 16 * s2, c, g) : zero_frag<T>();
-        }
+        for (int nt = 0; nt < NT; ++nt) oqt[s2][nt] = ld_free<T, true>(s_qu, LDK, 32 * nt, HD, 16 * s2, c, g);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
-        const frag<T> fdz = chain<T>(dz, s2), fa = chain<T>(aK, s2);
+        const frag<T> fdz = chain<T>(dz, s2);
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-          mma(dku[nt], oqt[s2][nt], fdz);
-          mma(dvu[nt], ogt[s2][nt], fa);
-        }
+        for (int nt = 0; nt < NT; ++nt) mma(dku[nt], oqt[s2][nt], fdz);
       }
     }
 #undef CASTLE_BQ2_LOAD_A
@@ -1289,24 +1285,13 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
       st.load_flat(qc + (int64_t)qb * QB * HD); st.store(e_qc, LDK);
     }
     __syncthreads();   // e2: epilogue tiles and dT shared
-#pragma unroll
-    for (int s = 0; s < PS; ++s) {
-      if (s < sfirst) continue;
-      // B operand: source j = jw + c on lanes, queries i = 16 s .. in natural order, from dT[i][j]
-      const frag<T> fdt = ld_free<T, false>(e_dt, LDT, jw, QB, 16 * s, c, g);
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-        mma(dvu[nt], ld_free<T, false>(e_qc, LDK, 32 * nt, HD, 16 * s, c, g), fdt);
-    }
-    if (i < L) {
-      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dku, b, h) + (int64_t)i * a.dku.sl, dku, c0 * kLn2, g, a.s.rotary ? i : -1);
-      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvu, b, h) + (int64_t)i * a.dvu.sl, dvu, kLn2, g, a.s.rotary ? i : -1);
-    }
+    if (i < L) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dku, b, h) + (int64_t)i * a.dku.sl, dku, c0 * kLn2, g, a.s.rotary ? i : -1);
   } else {
     acc_t dqc[NT];     // [n rows, i lanes]
+    acc_t dvu[NT];     // [n rows, j lanes]: this role's rows taken as lookahead sources
     acc_t dtacc[PT];   // [j rows (pair local), i lanes]
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) zero(dqc[nt]);
+    for (int nt = 0; nt < NT; ++nt) { zero(dqc[nt]); zero(dvu[nt]); }
 #pragma unroll
     for (int jt = 0; jt < PT; ++jt) zero(dtacc[jt]);
     // this role stages the reverse state
@@ -1351,19 +1336,23 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
       }
       __syncthreads();   // 3
       if (!live) continue;
-      {
-        frag<T> oat[2][PT];
 #pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2)
+      for (int s2 = 0; s2 < 2; ++s2) {   // one 16-key step at a time keeps the operand registers few
+        frag<T> oat[PT], ogt[NT];
 #pragma unroll
-          for (int jt = 0; jt < PT; ++jt)
-            if (jt <= pw) oat[s2][jt] = ld_nat<T>(s_at, LDA, 32 * jt + c, 16 * s2 + 8 * g);
+        for (int jt = 0; jt < PT; ++jt)
+          if (jt <= pw) oat[jt] = ld_nat<T>(s_at, LDA, 32 * jt + c, 16 * s2 + 8 * g);
+        // dVu += G'^T A for the rows taken as sources: A^T[j][k] of this wave's own rows
+        const frag<T> fa = ld_nat<T>(s_at, LDA, jw + c, 16 * s2 + 8 * g);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+          ogt[nt] = has_g ? ld_free<T, false>(s_g, LDK, 32 * nt, HD, 16 * s2, c, g) : zero_frag<T>();
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2)
+        for (int jt = 0; jt < PT; ++jt)
+          if (jt <= pw) mma(dtacc[jt], oat[jt], bdsu[s2]);
 #pragma unroll
-          for (int jt = 0; jt < PT; ++jt)
-            if (jt <= pw) mma(dtacc[jt], oat[s2][jt], bdsu[s2]);
+        for (int nt = 0; nt < NT; ++nt) mma(dvu[nt], ogt[nt], fa);   // ogt is zero where no reverse state exists
       }
     }
 #undef CASTLE_BQ2_LOAD_B
@@ -1395,7 +1384,19 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
           mma(dqc[nt], ld_free<T, true>(e_vu, LDK, 32 * nt, HD, 32 * jt + 16 * s2, c, g), fdt);
       }
     }
-    if (i < L) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqc, b, h) + (int64_t)i * a.dqc.sl, dqc, c0, g, a.s.rotary ? i : -1);
+#pragma unroll
+    for (int s = 0; s < PS; ++s) {
+      if (s < sfirst) continue;
+      // B operand: source j = jw + c on lanes, queries i = 16 s .. in natural order, from dT[i][j]
+      const frag<T> fdt = ld_free<T, false>(e_dt, LDT, jw, QB, 16 * s, c, g);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+        mma(dvu[nt], ld_free<T, false>(e_qc, LDK, 32 * nt, HD, 16 * s, c, g), fdt);
+    }
+    if (i < L) {
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqc, b, h) + (int64_t)i * a.dqc.sl, dqc, c0, g, a.s.rotary ? i : -1);
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvu, b, h) + (int64_t)i * a.dvu.sl, dvu, kLn2, g, a.s.rotary ? i : -1);
+    }
   }
 }
 

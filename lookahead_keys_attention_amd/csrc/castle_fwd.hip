@@ -92,51 +92,50 @@ template <typename T, typename TI, int HD>
 __global__ __launch_bounds__(kThreads) void tqv_kernel(FwdArgs a) {
   constexpr int KS = HD / 16;
   constexpr int TB = kNB / 32;
-  const int I = blockIdx.x, bh = blockIdx.y, b = bh / a.s.H, h = bh % a.s.H;
+  static_assert(TB * TB == kThreads / 64, "one 32x32 tile of the block per wave");
+  const int I = blockIdx.x, bh = blockIdx.y;
   const int lane = lane_id(), c = lane & 31, g = lane >> 5;
-  const float c1 = a.s.scale * kLog2e;
   const T* qc = prep_ptr<T>(a.ws.qc_p, bh, a.s.Lp, HD);   // pre-scaled by c1
   const T* vu = prep_ptr<T>(a.ws.vu_p, bh, a.s.Lp, HD);
   T* tb = reinterpret_cast<T*>(a.ws.t_blk) + (int64_t)bh * a.s.Lp * kNB;
   T* ttb = reinterpret_cast<T*>(a.ws.tt_blk) + (int64_t)bh * a.s.Lp * kNB;
-  for (int t = wave_id(); t < TB * TB; t += kThreads / 64) {
-    const int it = t / TB, jt = t % TB;
-    const int64_t i = (int64_t)I * kNB + 32 * it + c;   // A-operand row
-    const int64_t j = (int64_t)I * kNB + 32 * jt + c;   // B-operand row
-    acc_t acc;
-    zero(acc);
+  T* ttx = reinterpret_cast<T*>(a.ws.ttx_blk) + (int64_t)bh * a.s.Lp * kNB;
+  const int it = wave_id() / TB, jt = wave_id() % TB;
+  const int64_t i = (int64_t)I * kNB + 32 * it + c;   // A-operand row
+  const int64_t j = (int64_t)I * kNB + 32 * jt + c;   // B-operand row
+  // cross quarter of a pair of blocks, (Qc'_{I+1} Vu_I^T)^T for even I: same sources, the queries
+  // of the next block, no mask (every query is later).  All operand loads are issued together.
+  const bool cross = (I & 1) == 0 && I + 1 < a.s.nblk;
+  frag<T> fq[KS], fv[KS], fx[KS];
 #pragma unroll
-    for (int s = 0; s < KS; ++s)
-      mma(acc, ldg_nat<T>(qc, HD, i, 16 * s + 8 * g, true), ldg_nat<T>(vu, HD, j, 16 * s + 8 * g, true));
-    // acc[r] = (Qc' Vu^T)[il = 32 it + acc_row][jl = 32 jt + c]; stored as T' = tril(.)
-    const int jl = 32 * jt + c;
+  for (int s = 0; s < KS; ++s) {
+    fq[s] = ldg_nat<T>(qc, HD, i, 16 * s + 8 * g, true);
+    fv[s] = ldg_nat<T>(vu, HD, j, 16 * s + 8 * g, true);
+    fx[s] = ldg_nat<T>(qc, HD, i + kNB, 16 * s + 8 * g, cross);
+  }
+  acc_t acc, accx;
+  zero(acc);
+  zero(accx);
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int il = 32 * it + acc_row(r, g);
-      acc[r] = jl > il ? 0.f : acc[r];
-      tb[((int64_t)I * kNB + il) * kNB + jl] = (T)acc[r];
-    }
+  for (int s = 0; s < KS; ++s) {
+    mma(acc, fq[s], fv[s]);
+    mma(accx, fx[s], fv[s]);
+  }
+  // acc[r] = (Qc' Vu^T)[il = 32 it + acc_row][jl = 32 jt + c]; stored as T' = tril(.)
+  const int jl = 32 * jt + c;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int il = 32 * it + acc_row(r, g);
+    acc[r] = jl > il ? 0.f : acc[r];
+    tb[((int64_t)I * kNB + il) * kNB + jl] = (T)acc[r];
+  }
+#pragma unroll
+  for (int q = 0; q < 4; ++q)
+    st4<T>(ttb + ((int64_t)I * kNB + jl) * kNB + 32 * it + 8 * q + 4 * g, pack4<T>(acc, q));
+  if (cross) {
 #pragma unroll
     for (int q = 0; q < 4; ++q)
-      st4<T>(ttb + ((int64_t)I * kNB + jl) * kNB + 32 * it + 8 * q + 4 * g, pack4<T>(acc, q));
-  }
-  // cross quarter of a pair of blocks: (Qc'_{I+1} Vu_I^T)^T for even I, no mask (every query is later)
-  if ((I & 1) == 0 && I + 1 < a.s.nblk) {
-    T* ttx = reinterpret_cast<T*>(a.ws.ttx_blk) + (int64_t)bh * a.s.Lp * kNB;
-    for (int t = wave_id(); t < TB * TB; t += kThreads / 64) {
-      const int it = t / TB, jt = t % TB;
-      const int64_t i = (int64_t)(I + 1) * kNB + 32 * it + c;
-      const int64_t j = (int64_t)I * kNB + 32 * jt + c;
-      acc_t acc;
-      zero(acc);
-#pragma unroll
-      for (int s = 0; s < KS; ++s)
-        mma(acc, ldg_nat<T>(qc, HD, i, 16 * s + 8 * g, true), ldg_nat<T>(vu, HD, j, 16 * s + 8 * g, true));
-      const int jl = 32 * jt + c;
-#pragma unroll
-      for (int q = 0; q < 4; ++q)
-        st4<T>(ttx + ((int64_t)I * kNB + jl) * kNB + 32 * it + 8 * q + 4 * g, pack4<T>(acc, q));
-    }
+      st4<T>(ttx + ((int64_t)I * kNB + jl) * kNB + 32 * it + 8 * q + 4 * g, pack4<T>(accx, q));
   }
 }
 
