@@ -3,16 +3,16 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-decode] [--no-lm] [--no-cpu]
 
-Workload (BASELINE config 2): one Castle layer (dim 512, 8 heads, dim_head 64), bf16,
+Workload (benchmark configuration 2): one Castle layer (dim 512, 8 heads, dim_head 64), bf16,
 x and the upstream gradient ~ N(0,1) of shape (4, 4096, 512), seeded random-init weights;
 one step = forward + backward of the layer (projection GEMMs included), inputs resident in
 HBM.  Prints ONE JSON line:
   value        layer TFLOP/s = (19*B*H*L^2*d core flop + projection GEMM flop) / step time
   core         the same for the attention core alone, from per-kernel HIP-event times
   roofline     the longest-running kernel against the bf16 MFMA peak (2.5 PFLOP/s)
-  decode       BASELINE config 4 (B32, prefill 2048, 512 cached steps): tokens/s and the decode
+  decode       benchmark configuration 4 (B32, prefill 2048, 512 cached steps): tokens/s and the decode
                stream kernel against the HBM peak (8 TB/s)
-  lm           BASELINE config 5 (12 x [Castle + MLP], tied embedding, (16, 1024) tokens, bf16): one
+  lm           benchmark configuration 5 (12 x [Castle + MLP], tied embedding, (16, 1024) tokens, bf16): one
                forward + loss + backward, and greedy generation through prefill + cached decode
   cpu_baseline the CPU oracle (dense PyTorch restatement of the reference's non-Triton path)
                on a bounded sample of the same workload, host cores stated

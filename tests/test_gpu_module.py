@@ -1,5 +1,5 @@
 """Module-level parity on the GPU: the reference's GPU tests re-stated for the native path
-(tests/test_lookahead.py:67-143, 185-222, 225-282 of the reference) and the BASELINE configs at
+(tests/test_lookahead.py:67-143, 185-222, 225-282 of the reference) and the benchmark configurations at
 their full sizes, checked through the oracle on sampled heads and through size-independent
 properties (parallel == cached sequential, causality / prefix invariance)."""
 import pytest
@@ -110,7 +110,7 @@ def test_multi_token_with_cache_is_rejected():
 
 
 def test_config1_readme_fp32_parallel_vs_sequential():
-    # BASELINE config 1: Castle(512, 8, 64), x (2,128,512) fp32, parallel vs 128 cached steps, atol 1e-3
+    # benchmark configuration 1: Castle(512, 8, 64), x (2,128,512) fp32, parallel vs 128 cached steps, atol 1e-3
     m = make(512, 8, 64, seed=0).eval()
     x = torch.randn(2, 128, 512, generator=torch.Generator().manual_seed(0))
     with torch.no_grad():
@@ -141,7 +141,7 @@ def _head_oracle_check(proj, dmerged, merged, dproj, heads, d, b, h):
 
 
 def test_config2_bf16_full_size_sampled_heads():
-    # BASELINE config 2: dim 512, H8, d64, B4, L4096, bf16, forward + backward
+    # benchmark configuration 2: dim 512, H8, d64, B4, L4096, bf16, forward + backward
     from lookahead_keys_attention_amd import ops
 
     m = make(512, 8, 64, dtype=torch.bfloat16, seed=0)
@@ -161,7 +161,7 @@ def test_config2_bf16_full_size_sampled_heads():
 
 
 def test_config3_bf16_long_context_forward_backward():
-    # BASELINE config 3: dim 2048, H16, d128, B1, L16384, bf16, forward + backward at full size.
+    # benchmark configuration 3: dim 2048, H16, d128, B1, L16384, bf16, forward + backward at full size.
     # The dense oracle at L=16384 is out of reach on CPU, so the full-size run is checked through
     # size-independent properties: (i) prefix invariance of the forward output; (iii) the backward
     # pass is linear in dO, and positions whose dO is zero (and that no later position with a
@@ -205,7 +205,7 @@ def test_config3_bf16_long_context_forward_backward():
 
 
 def test_config4_bf16_decode_after_prefill():
-    # BASELINE config 4: B32, prefill 2048 through the parallel path, then cached steps
+    # benchmark configuration 4: B32, prefill 2048 through the parallel path, then cached steps
     m = make(512, 8, 64, dtype=torch.bfloat16, seed=0).eval()
     g = torch.Generator().manual_seed(0)
     steps = 4

@@ -235,7 +235,7 @@ def test_decode_step_with_an_out_of_range_device_count_writes_nothing():
 
 @pytest.mark.gpu
 def test_config5_language_model_step_bf16():
-    """BASELINE config 5: 12 x [Castle(512, 8 heads, 64) + MLP], tied embedding, (16, 1024) tokens,
+    """benchmark configuration 5: 12 x [Castle(512, 8 heads, 64) + MLP], tied embedding, (16, 1024) tokens,
     forward + loss + backward."""
     torch.manual_seed(0)
     model = CastleLM(num_tokens=VOCAB, dim=512, depth=12, heads=8, dim_head=64, use_triton=True,

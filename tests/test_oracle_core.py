@@ -167,7 +167,7 @@ def test_module_rejects_multi_token_with_cache():
 
 
 def test_readme_config_parallel_vs_sequential_fp32():
-    # BASELINE config 1: Castle(512, 8, 64), x (2,128,512) fp32, atol 1e-3
+    # benchmark configuration 1: Castle(512, 8, 64), x (2,128,512) fp32, atol 1e-3
     p = O.default_init(512, 8, 64, seed=0)
     x = torch.randn(2, 128, 512, generator=torch.Generator().manual_seed(0))
     full = O.module_forward(x, p, 8)
