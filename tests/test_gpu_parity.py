@@ -159,6 +159,53 @@ def test_backward_without_score_tiles(monkeypatch):
         assert_close(leaf.grad, r, torch.bfloat16, name, 2e-2)
 
 
+def test_two_streams_run_the_operator_side_by_side():
+    """Every launch goes to the caller's stream and every call owns its workspace: two forward +
+    backward passes enqueued on two streams without synchronising in between give, bit for bit,
+    what each gives alone on the default stream."""
+    cases = [(2, 2, 640, 64, torch.bfloat16, 5), (1, 4, 384, 32, torch.bfloat16, 6)]
+    alone = []
+    for B, Hh, L, d, dtype, seed in cases:
+        ops, dout = rand_ops(B, Hh, L, d, dtype, seed=seed)
+        leaves = [t.to(DEV).requires_grad_() for t in ops]
+        out = H().castle_attention_hip(*leaves, d ** -0.5)
+        out.backward(dout.to(DEV))
+        alone.append((out.detach().clone(), [leaf.grad.clone() for leaf in leaves]))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(device=DEV) for _ in cases]
+    together = []
+    for (B, Hh, L, d, dtype, seed), stream in zip(cases, streams):
+        ops, dout = rand_ops(B, Hh, L, d, dtype, seed=seed)
+        leaves = [t.to(DEV).requires_grad_() for t in ops]
+        dout = dout.to(DEV)
+        torch.cuda.synchronize()
+        together.append((leaves, dout, stream))
+    results = []
+    for leaves, dout, stream in together:      # enqueue both before waiting for either
+        with torch.cuda.stream(stream):
+            out = H().castle_attention_hip(*leaves, leaves[0].shape[-1] ** -0.5)
+            out.backward(dout)
+            results.append(out)
+    torch.cuda.synchronize()
+    for (want_out, want_grads), out, (leaves, _, _) in zip(alone, results, together):
+        assert torch.equal(out, want_out)
+        for leaf, want in zip(leaves, want_grads):
+            assert torch.equal(leaf.grad, want)
+
+
+def test_forward_and_backward_are_deterministic():
+    """No atomics anywhere: the same inputs give the same bits, call after call."""
+    ops, dout = rand_ops(2, 3, 1000, 64, torch.bfloat16, seed=9)
+    runs = []
+    for _ in range(3):
+        leaves = [t.to(DEV).requires_grad_() for t in ops]
+        out = H().castle_attention_hip(*leaves, 0.125)
+        out.backward(dout.to(DEV))
+        runs.append([out.detach()] + [leaf.grad for leaf in leaves])
+    for other in runs[1:]:
+        assert all(torch.equal(a, b) for a, b in zip(runs[0], other))
+
+
 def test_lookahead_keys_carry_no_gradient():
     ops, dout = rand_ops(1, 1, 40, 16, torch.float32, seed=5)
     leaves = [t.to(DEV).requires_grad_() for t in ops]
