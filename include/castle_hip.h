@@ -82,11 +82,10 @@ int castle_fwd(const castle_view4* qc, const castle_view4* kc, const castle_view
                void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Bytes of extra device workspace castle_bwd needs: reverse state snapshots, delta, a copy of dout in
- * the compute type and, for the
- * 16-bit element types at d <= 64, the dS / dSu score-gradient tiles its first kernel hands to its
- * second (2 * B * H * Lp * Lp elements, Lp = L rounded up to 128; left out, and the score chain recomputed
- * instead, when they would exceed 16 GiB or the byte count in the environment variable
- * CASTLE_MAX_SCORE_TILE_BYTES). */
+ * the compute type and, for the 16-bit element types, the dS / dSu score-gradient tiles its first
+ * kernel hands to its second (2 * B * H * Lp * Lp elements, Lp = L rounded up to 128; left out, and
+ * the score chain recomputed instead, when they would exceed 40 GiB or the byte count in the
+ * environment variable CASTLE_MAX_SCORE_TILE_BYTES). */
 int64_t castle_bwd_workspace_bytes(int B, int H, int L, int d, int dtype);
 
 /* Parallel backward.  Same operands as castle_fwd plus the forward output `out`, the

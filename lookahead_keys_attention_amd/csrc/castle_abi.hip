@@ -36,7 +36,7 @@ int64_t align_up(int64_t x, int64_t a) { return (x + a - 1) / a * a; }
 
 // upper limit of the dS / dSu tile buffers (they grow with B*H*L^2); beyond it the backward
 // falls back to recomputing the score chain in its second kernel
-constexpr int64_t kMaxScoreTileBytes = (int64_t)16 << 30;
+constexpr int64_t kMaxScoreTileBytes = (int64_t)40 << 30;
 // CASTLE_MAX_SCORE_TILE_BYTES in the environment overrides the limit (0 = never use the tiles)
 int64_t max_score_tile_bytes() {
   const char* e = getenv("CASTLE_MAX_SCORE_TILE_BYTES");
@@ -57,8 +57,8 @@ Geometry geometry(int B, int H, int L, int d, int es) {
   g.lse_bytes = align_up(BH * g.Lp * 4, 256);
   g.tblk_bytes = align_up(BH * g.Lp * kNB * es, 256);
   g.snap_bytes = align_up(BH * castle::snap_rows(g.nblk) * d * es, 256);
-  // dS / dSu tiles between the two backward kernels: only the 16-bit, d <= 64 path uses them
-  g.mat_bytes = (es == 2 && d <= 64) ? align_up(BH * g.Lp * g.Lp * es, 256) : 0;
+  // dS / dSu tiles between the two backward kernels: the 16-bit paths use them
+  g.mat_bytes = es == 2 ? align_up(BH * g.Lp * g.Lp * es, 256) : 0;
   if (2 * g.mat_bytes > max_score_tile_bytes()) g.mat_bytes = 0;   // too long: the query kernel recomputes the scores instead
   g.off_lse = 0;
   g.off_t = g.off_lse + g.lse_bytes;

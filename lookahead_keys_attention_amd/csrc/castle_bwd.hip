@@ -184,7 +184,9 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   if (PF) CASTLE_BK_LOAD(a.s.nblk - 1);
   for (int I = a.s.nblk - 1; I >= I0; --I) {
     const bool active = I >= Iw;
-    if (DO_QG && active && I <= a.s.nblk - 2) {   // reverse state as of block I
+    // reverse state as of block I; the tile-consuming query kernel only reads those behind a pair
+    // of blocks (odd I), the recomputing one all of them
+    if (DO_QG && active && I <= a.s.nblk - 2 && (a.ds_mat == nullptr || (I & 1))) {
       store_snap_tile<T, HD, NT>(gsnap + (gsnap_off(I) + kw0) * HD, G, c, g);
     }
     if (I > Iw) {
@@ -298,6 +300,18 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
         sc[r] = p;
         ds[r] = dsv;
         dsu[r] = -dsv * sp;
+      }
+      if constexpr (DO_KV && sizeof(T) == 2) {
+        if (a.ds_mat != nullptr) {   // hand the tile to the tile-consuming query kernel: element (k, i) at (i/16)*512 + k*16 + i%16
+          T* ds_mat = reinterpret_cast<T*>(a.ds_mat) + (int64_t)bh * a.s.Lp * a.s.Lp;
+          T* dsu_mat = reinterpret_cast<T*>(a.dsu_mat) + (int64_t)bh * a.s.Lp * a.s.Lp;
+          const int64_t tile = ((int64_t)(kw0 / 32) * (a.s.Lp / 32) + i0 / 32) * 1024 + c * 16 + 4 * g;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {   // registers 4q .. 4q+3: queries 8q + 4g .. + 3 of the tile
+            st4<T>(ds_mat + tile + (q / 2) * 512 + 8 * (q % 2), pack4<T>(ds, q));
+            st4<T>(dsu_mat + tile + (q / 2) * 512 + 8 * (q % 2), pack4<T>(dsu, q));
+          }
+        }
       }
       {
         frag<T> odt[2][NT], oqt[2][NT], ott[2][BT];
@@ -1076,10 +1090,12 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
 template <typename T> constexpr int kLdD = 128 + 8;   // dS / dSu tiles [key][128 queries]
 template <typename T> constexpr int kLdA = kCK + 8;   // gate tile [128 sources][key]
 template <typename T> constexpr int kLdT2 = 128 + 4;  // dT of the row pair [128 queries][128 sources]
+template <typename T> constexpr int kLdTT = 128 + 8;  // T'^T rows of the pair [128 sources][128 queries] (d = 128 only)
 template <typename T, int HD> constexpr int bwd_query2_lds_bytes() {
   int b = 4 * a16((int)sizeof(T) * kCK * lds_ld<T>(HD));          // kc, qu, ub, g
   b += a16((int)sizeof(T) * 128 * kLdA<T>);                       // A^T [j][k]
   b += 2 * a16((int)sizeof(T) * kCK * kLdD<T>);                   // dS, dSu [k][i]
+  if (HD > 64) b += a16((int)sizeof(T) * 128 * kLdTT<T>) + a16((int)sizeof(T) * 128 * lds_ld<T>(HD));   // T'^T and vu rows
   int e = 2 * a16((int)sizeof(T) * 128 * lds_ld<T>(HD)) + a16((int)sizeof(T) * 128 * kLdT2<T>);
   return b > e ? b : e;
 }
@@ -1114,16 +1130,22 @@ struct TileStage {
 //   dA[k,j]  = sum_{i in pair, i >= j} dSu[i,k] T'[i,j] + G'[k] . vu_j
 //   dQc[i]  += sum_k dSu[i,k] U[k]  (keys before the pair)  + sum_{j in pair, j <= i} dT[i,j] vu_j
 //   dVu[j]  += sum_k A[k,j] G'[k] + sum_{i in pair, i >= j} dT[i,j] qc'_i,   dT[i,j] = sum_k dSu[i,k] A[k,j]
-template <typename T, typename TI, int HD>
+// PART selects the outputs of a launch: 0 = all (d <= 64); at d = 128, where the accumulators of
+// all outputs do not fit the register file, 1 = dQc and 2 = dKu, dVu (gate and dT are formed in
+// both).  At d = 128 the T'^T and vu rows of the pair also sit in LDS instead of registers.
+template <typename T, typename TI, int HD, int PART>
 __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) {
-  static_assert(sizeof(T) == 2 && HD <= 64 && kCK == 32, "tile consumer: 16-bit operands, d <= 64");
+  static_assert(sizeof(T) == 2 && kCK == 32, "tile consumer: 16-bit operands");
+  static_assert((PART == 0) == (HD <= 64), "one launch up to d = 64, two at d = 128");
+  constexpr bool DO_Q = PART != 2, DO_S = PART != 1;
+  constexpr bool LDS_ROWS = HD > 64;   // T'^T / vu rows of the pair in LDS, not in registers
   constexpr int KS = HD / 16;
   constexpr int HDP = HD < 32 ? 32 : HD;
   constexpr int NT = HDP / 32;
   constexpr int QB = 128;
   constexpr int PT = QB / 32;    // 32-row tiles across the pair
   constexpr int PS = QB / 16;    // 16-deep steps across the pair
-  constexpr int LDK = lds_ld<T>(HD), LDT = kLdT2<T>, LDA = kLdA<T>, LDD = kLdD<T>;
+  constexpr int LDK = lds_ld<T>(HD), LDT = kLdT2<T>, LDA = kLdA<T>, LDD = kLdD<T>, LDTT = kLdTT<T>;
 
   Carver cv{castle_smem};
   T* s_kc = cv.take<T>(kCK * LDK);
@@ -1133,6 +1155,8 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
   T* s_at = cv.take<T>(QB * LDA);    // gate, [source j][key k]
   T* s_ds = cv.take<T>(kCK * LDD);   // dS,  [key k][query i]
   T* s_dsu = cv.take<T>(kCK * LDD);  // dSu, [key k][query i]
+  T* s_tt = LDS_ROWS ? cv.take<T>(QB * LDTT) : nullptr;   // T'^T [source j][query i of the pair]
+  T* s_vu = LDS_ROWS ? cv.take<T>(QB * LDK) : nullptr;    // vu rows of the pair
   // the epilogue reuses the same memory
   Carver ce{castle_smem};
   T* e_vu = ce.take<T>(QB * LDK);
@@ -1154,12 +1178,14 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
   const int i = i0w + c;                      // this lane's row
   const int blk0 = 2 * qb, blk1 = 2 * qb + 1;
   const int sfirst = jw / 16;                 // first step covering queries i >= j
-  const bool has_g = blk1 <= a.s.nblk - 2;    // a reverse state exists behind the pair
+  const bool has_g = DO_S && blk1 <= a.s.nblk - 2;    // a reverse state exists behind the pair (and is needed)
 
   const T* qc = prep_ptr<T>(a.ws.qc_p, bh, a.s.Lp, HD);
   const T* vu = prep_ptr<T>(a.ws.vu_p, bh, a.s.Lp, HD);
   const T* usnap = reinterpret_cast<const T*>(a.ws.usnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
   const T* gsnap = reinterpret_cast<const T*>(a.gsnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
+  const T* ttb = reinterpret_cast<const T*>(a.ws.tt_blk) + (int64_t)bh * a.s.Lp * kNB;
+  const T* ttx = reinterpret_cast<const T*>(a.ws.ttx_blk) + (int64_t)bh * a.s.Lp * kNB;
   const int64_t tile_row = (int64_t)(a.s.Lp / 32) * 1024;   // elements between the tiles of consecutive key groups
   const T* dsm = reinterpret_cast<const T*>(a.ds_mat) + (int64_t)bh * a.s.Lp * a.s.Lp + (int64_t)qb * 4 * 1024;
   const T* dsum = reinterpret_cast<const T*>(a.dsu_mat) + (int64_t)bh * a.s.Lp * a.s.Lp + (int64_t)qb * 4 * 1024;
@@ -1167,38 +1193,58 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
   if (kend > a.s.Lp) kend = a.s.Lp;
   TileStage<T> pds, pdsu;   // every thread: one piece of each
 
+  if constexpr (LDS_ROWS && DO_S) {
+    // rows j of the pair: T'^T[j][i] over the pair's queries (own block from tt_blk; for the first
+    // block the second block's queries from the cross quarter), and vu_j.  Columns a row never
+    // uses (queries before its block) are left unwritten.
+    constexpr int VH = kNB / 8;   // 16-byte pieces per half row
+    for (int p = threadIdx.x; p < QB * 2 * VH; p += 2 * kThreads) {
+      const int j = p / (2 * VH), half = (p / VH) & 1, v = p % VH;
+      const bool first = j < kNB;
+      if (!first && half == 0) continue;
+      const T* src = (first && half == 1) ? ttx : ttb;
+      *reinterpret_cast<frag_mem<T>*>(s_tt + j * LDTT + half * kNB + v * 8) =
+          *reinterpret_cast<const frag_mem<T>*>(src + ((int64_t)qb * QB + j) * kNB + v * 8);
+    }
+    RowStage<T, T, QB, HD, 2 * kThreads> st;
+    st.load_flat(vu + (int64_t)qb * QB * HD);
+    st.store(s_vu, LDK);
+    // visible after the first barrier of the chunk loop; first used behind its third
+  }
+
   if (source_role) {
     const T* kc = prep_ptr<T>(a.ws.kc_p, bh, a.s.Lp, HD);
     const T* qu = prep_ptr<T>(a.ws.qu_p, bh, a.s.Lp, HD);
     const T* ku = prep_ptr<T>(a.ws.ku_p, bh, a.s.Lp, HD);
-    const T* ttb = reinterpret_cast<const T*>(a.ws.tt_blk) + (int64_t)bh * a.s.Lp * kNB;
-    const T* ttx = reinterpret_cast<const T*>(a.ws.ttx_blk) + (int64_t)bh * a.s.Lp * kNB;
     // T'^T rows of this wave across the queries of the pair: its own block from tt_blk, and for a
     // wave of the first block the second block from the cross quarter
-    frag<T> fku[KS], fvu[KS], ftt[PS];
+    constexpr int NREG = (LDS_ROWS || !DO_S) ? 1 : PS;   // register copies only up to d = 64
+    constexpr int NVU = (LDS_ROWS || !DO_S) ? 1 : KS;
+    frag<T> fku[KS], fvu[NVU], ftt[NREG];
 #pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      fku[s] = ldg_nat_scaled<T, T>(ku, HD, i, 16 * s + 8 * g, true, -c1);
-      fvu[s] = ldg_nat<T>(vu, HD, i, 16 * s + 8 * g, true);
+    for (int s = 0; s < KS; ++s) fku[s] = ldg_nat_scaled<T, T>(ku, HD, i, 16 * s + 8 * g, true, -c1);
+    if constexpr (DO_S && !LDS_ROWS) {
+#pragma unroll
+      for (int s = 0; s < KS; ++s) fvu[s] = ldg_nat<T>(vu, HD, i, 16 * s + 8 * g, true);
+#pragma unroll
+      for (int s = 0; s < PS; ++s) {
+        const bool own = (s < PS / 2) == (pw < 2);   // queries of step s lie in this wave's own block
+        const T* src = own ? ttb : ttx;
+        ftt[s] = ldg_nat<T>(src, kNB, i, 16 * (s % (PS / 2)) + 8 * g, s >= sfirst);
+      }
     }
+    acc_t dku[DO_S ? NT : 1];   // [n rows, j lanes]
 #pragma unroll
-    for (int s = 0; s < PS; ++s) {
-      const bool own = (s < PS / 2) == (pw < 2);   // queries of step s lie in this wave's own block
-      const T* src = own ? ttb : ttx;
-      ftt[s] = ldg_nat<T>(src, kNB, i, 16 * (s % (PS / 2)) + 8 * g, s >= sfirst);
-    }
-    acc_t dku[NT];   // [n rows, j lanes]
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) zero(dku[nt]);
+    for (int nt = 0; nt < (DO_S ? NT : 1); ++nt) zero(dku[nt]);
 
     // this role stages kc, qu and the lookahead state
     RowStage<T, T, kCK, HD> pkc, pqu;
     SnapStage<T, kCK, HD> pu;
 #define CASTLE_BQ2_LOAD_A(K0)                                                            \
   do {                                                                                   \
-    pkc.load_flat(kc + (int64_t)(K0) * HD, tid);                                         \
+    if (DO_Q) pkc.load_flat(kc + (int64_t)(K0) * HD, tid);                               \
     pqu.load_flat(qu + (int64_t)(K0) * HD, tid);                                         \
-    if ((K0) / kNB < blk0) pu.load(usnap + (usnap_off(blk0) + (K0)) * HD, tid);          \
+    if (DO_Q && (K0) / kNB < blk0) pu.load(usnap + (usnap_off(blk0) + (K0)) * HD, tid);  \
     pds.load(dsm + (int64_t)((K0) / 32) * tile_row);                                     \
     pdsu.load(dsum + (int64_t)((K0) / 32) * tile_row);                                   \
   } while (0)
@@ -1206,9 +1252,9 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
     for (int k0 = 0; k0 < kend; k0 += kCK) {
       const int Kb = k0 / kNB;
       __syncthreads();   // 1: tiles free
-      pkc.store(s_kc, LDK, tid);
+      if (DO_Q) pkc.store(s_kc, LDK, tid);
       pqu.store(s_qu, LDK, tid);
-      if (Kb < blk0) pu.store(s_ub, LDK, tid);
+      if (DO_Q && Kb < blk0) pu.store(s_ub, LDK, tid);
       pds.store(s_ds);
       pdsu.store(s_dsu);
       if (k0 + kCK < kend) CASTLE_BQ2_LOAD_A(k0 + kCK);   // in flight while this chunk is processed
@@ -1218,13 +1264,15 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
       acc_t aK;
       zero(aK);
       if (live) {
-        {
-          frag<T> oqu[KS];
 #pragma unroll
-          for (int s = 0; s < KS; ++s) oqu[s] = ld_nat<T>(s_qu, LDK, c, 16 * s + 8 * g);
+        for (int s0 = 0; s0 < KS; s0 += 4) {   // operand fragments in batches of four
+          frag<T> oqu[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) oqu[u] = ld_nat<T>(s_qu, LDK, c, 16 * (s0 + u) + 8 * g);
           __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-          for (int s = 0; s < KS; ++s) mma(aK, oqu[s], fku[s]);
+          for (int u = 0; u < 4; ++u)
+            if (s0 + u < KS) mma(aK, oqu[u], fku[s0 + u]);
         }
 #pragma unroll
         for (int r = 0; r < 16; ++r) aK[r] = fast_rcp(1.f + fast_exp2(aK[r]));
@@ -1238,12 +1286,12 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
 #pragma unroll
       for (int q = 0; q < 4; ++q) st4<T>(s_at + (jw + c) * LDA + 8 * q + 4 * g, pack4<T>(aK, q));
       __syncthreads();   // 3: gate shared
-      if (!live) continue;
+      if (!live || !DO_S) continue;
       // dA in two accumulators (two dependent MFMA chains instead of one of up to twelve)
       acc_t dA, dA2;
       zero(dA);
       zero(dA2);
-      {
+      if constexpr (!LDS_ROWS) {
         frag<T> og[KS];
 #pragma unroll
         for (int s = 0; s < KS; ++s) og[s] = has_g ? ld_nat<T>(s_g, LDK, c, 16 * s + 8 * g) : zero_frag<T>();
@@ -1255,43 +1303,80 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
           __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
           for (int u = 0; u < PS / 2; ++u) {
-            if (half * (PS / 2) + u >= sfirst) mma(dA, ods[u], ftt[half * (PS / 2) + u]);
-            if (half == 0 && u < KS) mma(dA2, og[u], fvu[u]);   // og is zero where no reverse state exists
+            if (half * (PS / 2) + u >= sfirst) mma(dA, ods[u], ftt[NREG == 1 ? 0 : half * (PS / 2) + u]);
+            if (half == 0 && u < KS) mma(dA2, og[u], fvu[NVU == 1 ? 0 : u]);   // og is zero where no reverse state exists
           }
+        }
+      } else {
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {   // dSu^T T'
+          frag<T> ods[PS / 2], ott[PS / 2];
+#pragma unroll
+          for (int u = 0; u < PS / 2; ++u) {
+            ods[u] = ld_nat<T>(s_dsu, LDD, c, 16 * (half * (PS / 2) + u) + 8 * g);
+            ott[u] = ld_nat<T>(s_tt, LDTT, jw + c, 16 * (half * (PS / 2) + u) + 8 * g);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int u = 0; u < PS / 2; ++u)
+            if (half * (PS / 2) + u >= sfirst) mma(dA, ods[u], ott[u]);
+        }
+#pragma unroll
+        for (int s0 = 0; s0 < KS; s0 += 4) {   // G' Vu^T; og is zero where no reverse state exists
+          frag<T> og[4], ovu[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            og[u] = has_g ? ld_nat<T>(s_g, LDK, c, 16 * (s0 + u) + 8 * g) : zero_frag<T>();
+            ovu[u] = ld_nat<T>(s_vu, LDK, jw + c, 16 * (s0 + u) + 8 * g);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            if (s0 + u < KS) mma(dA2, og[u], ovu[u]);
         }
       }
       acc_t dz;
 #pragma unroll
       for (int r = 0; r < 16; ++r) dz[r] = (dA[r] + dA2[r]) * aK[r] * (1.f - aK[r]);
-      frag<T> oqt[2][NT];
+      {
+        constexpr int SB = LDS_ROWS ? 1 : 2;
 #pragma unroll
-      for (int s2 = 0; s2 < 2; ++s2)
+        for (int s0 = 0; s0 < 2; s0 += SB) {
+          frag<T> oqt[SB][NT];
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) oqt[s2][nt] = ld_free<T, true>(s_qu, LDK, 32 * nt, HD, 16 * s2, c, g);
-      __builtin_amdgcn_sched_barrier(0);
+          for (int u = 0; u < SB; ++u)
 #pragma unroll
-      for (int s2 = 0; s2 < 2; ++s2) {
-        const frag<T> fdz = chain<T>(dz, s2);
+            for (int nt = 0; nt < NT; ++nt) oqt[u][nt] = ld_free<T, true>(s_qu, LDK, 32 * nt, HD, 16 * (s0 + u), c, g);
+          __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) mma(dku[nt], oqt[s2][nt], fdz);
+          for (int u = 0; u < SB; ++u) {
+            const frag<T> fdz = chain<T>(dz, s0 + u);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) mma(dku[DO_S ? nt : 0], oqt[u][nt], fdz);
+          }
+        }
       }
     }
 #undef CASTLE_BQ2_LOAD_A
-    // ---- epilogue: in-pair term dvu += dT^T Qc' ----------------------------------------------
+    // ---- epilogue (the other role's): only the shared staging ---------------------------------
     __syncthreads();   // e1: chunk tiles dead
     {
       RowStage<T, T, QB, HD, 2 * kThreads> st;
-      st.load_flat(vu + (int64_t)qb * QB * HD); st.store(e_vu, LDK);
-      st.load_flat(qc + (int64_t)qb * QB * HD); st.store(e_qc, LDK);
+      if (DO_Q) { st.load_flat(vu + (int64_t)qb * QB * HD); st.store(e_vu, LDK); }
+      if (DO_S) { st.load_flat(qc + (int64_t)qb * QB * HD); st.store(e_qc, LDK); }
     }
     __syncthreads();   // e2: epilogue tiles and dT shared
-    if (i < L) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dku, b, h) + (int64_t)i * a.dku.sl, dku, c0 * kLn2, g, a.s.rotary ? i : -1);
+    if constexpr (DO_S) {
+      if (i < L) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dku, b, h) + (int64_t)i * a.dku.sl, dku, c0 * kLn2, g, a.s.rotary ? i : -1);
+    }
   } else {
-    acc_t dqc[NT];     // [n rows, i lanes]
-    acc_t dvu[NT];     // [n rows, j lanes]: this role's rows taken as lookahead sources
-    acc_t dtacc[PT];   // [j rows (pair local), i lanes]
+    acc_t dqc[DO_Q ? NT : 1];   // [n rows, i lanes]
+    acc_t dvu[DO_S ? NT : 1];   // [n rows, j lanes]: this role's rows taken as lookahead sources
+    acc_t dtacc[PT];            // [j rows (pair local), i lanes]
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) { zero(dqc[nt]); zero(dvu[nt]); }
+    for (int nt = 0; nt < (DO_Q ? NT : 1); ++nt) zero(dqc[nt]);
+#pragma unroll
+    for (int nt = 0; nt < (DO_S ? NT : 1); ++nt) zero(dvu[nt]);
 #pragma unroll
     for (int jt = 0; jt < PT; ++jt) zero(dtacc[jt]);
     // this role stages the reverse state
@@ -1314,25 +1399,34 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
       const bool live = k0 <= i0w;
       frag<T> bdsu[2];
       if (live) {
-        frag<T> bds[2], okt[2][NT], out[2][NT];
+        constexpr int SB = LDS_ROWS ? 1 : 2;   // 16-key steps whose operand fragments are requested together
 #pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2) {
-          bds[s2] = ld_free<T, false>(s_ds, LDD, jw, 1 << 30, 16 * s2, c, g);
-          bdsu[s2] = ld_free<T, false>(s_dsu, LDD, jw, 1 << 30, 16 * s2, c, g);
+        for (int s0 = 0; s0 < 2; s0 += SB) {
+          frag<T> bds[SB], okt[SB][NT], out[SB][NT];
 #pragma unroll
-          for (int nt = 0; nt < NT; ++nt) {
-            okt[s2][nt] = ld_free<T, false>(s_kc, LDK, 32 * nt, HD, 16 * s2, c, g);
-            out[s2][nt] = ld_free<T, false>(s_ub, LDK, 32 * nt, HD, 16 * s2, c, g);
+          for (int u = 0; u < SB; ++u) {
+            const int s2 = s0 + u;
+            bdsu[s2] = ld_free<T, false>(s_dsu, LDD, jw, 1 << 30, 16 * s2, c, g);
+            if constexpr (DO_Q) {
+              bds[u] = ld_free<T, false>(s_ds, LDD, jw, 1 << 30, 16 * s2, c, g);
+#pragma unroll
+              for (int nt = 0; nt < NT; ++nt) {
+                okt[u][nt] = ld_free<T, false>(s_kc, LDK, 32 * nt, HD, 16 * s2, c, g);
+                out[u][nt] = ld_free<T, false>(s_ub, LDK, 32 * nt, HD, 16 * s2, c, g);
+              }
+            }
+          }
+          if constexpr (DO_Q) {
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < SB; ++u)
+#pragma unroll
+              for (int nt = 0; nt < NT; ++nt) {
+                mma(dqc[nt], okt[u][nt], bds[u]);
+                if (Kb < blk0) mma(dqc[nt], out[u][nt], bdsu[s0 + u]);
+              }
           }
         }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2)
-#pragma unroll
-          for (int nt = 0; nt < NT; ++nt) {
-            mma(dqc[nt], okt[s2][nt], bds[s2]);
-            if (Kb < blk0) mma(dqc[nt], out[s2][nt], bdsu[s2]);
-          }
       }
       __syncthreads();   // 3
       if (!live) continue;
@@ -1344,24 +1438,28 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
           if (jt <= pw) oat[jt] = ld_nat<T>(s_at, LDA, 32 * jt + c, 16 * s2 + 8 * g);
         // dVu += G'^T A for the rows taken as sources: A^T[j][k] of this wave's own rows
         const frag<T> fa = ld_nat<T>(s_at, LDA, jw + c, 16 * s2 + 8 * g);
+        if constexpr (DO_S) {
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-          ogt[nt] = has_g ? ld_free<T, false>(s_g, LDK, 32 * nt, HD, 16 * s2, c, g) : zero_frag<T>();
+          for (int nt = 0; nt < NT; ++nt)
+            ogt[nt] = has_g ? ld_free<T, false>(s_g, LDK, 32 * nt, HD, 16 * s2, c, g) : zero_frag<T>();
+        }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int jt = 0; jt < PT; ++jt)
           if (jt <= pw) mma(dtacc[jt], oat[jt], bdsu[s2]);
+        if constexpr (DO_S) {
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) mma(dvu[nt], ogt[nt], fa);   // ogt is zero where no reverse state exists
+          for (int nt = 0; nt < NT; ++nt) mma(dvu[nt], ogt[nt], fa);   // ogt is zero where no reverse state exists
+        }
       }
     }
 #undef CASTLE_BQ2_LOAD_B
-    // ---- epilogue: dT = tril(dTacc) over the pair:  dqc += dT Vu ------------------------------
+    // ---- epilogue: dT = tril(dTacc) over the pair:  dqc += dT Vu,  dvu += dT^T Qc' ------------
     __syncthreads();   // e1
     {
       RowStage<T, T, QB, HD, 2 * kThreads> st;
-      st.load_flat(vu + (int64_t)qb * QB * HD); st.store(e_vu, LDK);
-      st.load_flat(qc + (int64_t)qb * QB * HD); st.store(e_qc, LDK);
+      if (DO_Q) { st.load_flat(vu + (int64_t)qb * QB * HD); st.store(e_vu, LDK); }
+      if (DO_S) { st.load_flat(qc + (int64_t)qb * QB * HD); st.store(e_qc, LDK); }
     }
     // dT^T[j rows, i lanes] masked to j <= i, shared as dT[i][j] for the source-side product
 #pragma unroll
@@ -1369,33 +1467,39 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
 #pragma unroll
       for (int r = 0; r < 16; ++r)
         if (32 * jt + acc_row(r, g) > jw + c) dtacc[jt][r] = 0.f;
+      if constexpr (DO_S) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) st4<T>(e_dt + (jw + c) * LDT + 32 * jt + 8 * q + 4 * g, pack4<T>(dtacc[jt], q));
-    }
-    __syncthreads();   // e2
-#pragma unroll
-    for (int jt = 0; jt < PT; ++jt) {
-      if (jt > pw) continue;
-#pragma unroll
-      for (int s2 = 0; s2 < 2; ++s2) {
-        const frag<T> fdt = chain<T>(dtacc[jt], s2);
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-          mma(dqc[nt], ld_free<T, true>(e_vu, LDK, 32 * nt, HD, 32 * jt + 16 * s2, c, g), fdt);
+        for (int q = 0; q < 4; ++q) st4<T>(e_dt + (jw + c) * LDT + 32 * jt + 8 * q + 4 * g, pack4<T>(dtacc[jt], q));
       }
     }
+    __syncthreads();   // e2
+    if constexpr (DO_Q) {
 #pragma unroll
-    for (int s = 0; s < PS; ++s) {
-      if (s < sfirst) continue;
-      // B operand: source j = jw + c on lanes, queries i = 16 s .. in natural order, from dT[i][j]
-      const frag<T> fdt = ld_free<T, false>(e_dt, LDT, jw, QB, 16 * s, c, g);
+      for (int jt = 0; jt < PT; ++jt) {
+        if (jt > pw) continue;
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-        mma(dvu[nt], ld_free<T, false>(e_qc, LDK, 32 * nt, HD, 16 * s, c, g), fdt);
+        for (int s2 = 0; s2 < 2; ++s2) {
+          const frag<T> fdt = chain<T>(dtacc[jt], s2);
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt)
+            mma(dqc[nt], ld_free<T, true>(e_vu, LDK, 32 * nt, HD, 32 * jt + 16 * s2, c, g), fdt);
+        }
+      }
+    }
+    if constexpr (DO_S) {
+#pragma unroll
+      for (int s = 0; s < PS; ++s) {
+        if (s < sfirst) continue;
+        // B operand: source j = jw + c on lanes, queries i = 16 s .. in natural order, from dT[i][j]
+        const frag<T> fdt = ld_free<T, false>(e_dt, LDT, jw, QB, 16 * s, c, g);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+          mma(dvu[nt], ld_free<T, false>(e_qc, LDK, 32 * nt, HD, 16 * s, c, g), fdt);
+      }
     }
     if (i < L) {
-      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqc, b, h) + (int64_t)i * a.dqc.sl, dqc, c0, g, a.s.rotary ? i : -1);
-      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvu, b, h) + (int64_t)i * a.dvu.sl, dvu, kLn2, g, a.s.rotary ? i : -1);
+      if constexpr (DO_Q) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqc, b, h) + (int64_t)i * a.dqc.sl, dqc, c0, g, a.s.rotary ? i : -1);
+      if constexpr (DO_S) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvu, b, h) + (int64_t)i * a.dvu.sl, dvu, kLn2, g, a.s.rotary ? i : -1);
     }
   }
 }
@@ -1419,12 +1523,21 @@ template <typename T, typename TI, int HD> static int launch_bwd_t(const BwdArgs
   if (key_lds > kMaxLds || query_lds > kMaxLds) return -2;
   constexpr bool SPLIT = HD > 64;   // two passes per kernel, half of the outputs each
   constexpr bool TWO_ROLE = sizeof(T) == 2 && HD <= 64;
+  constexpr bool TILES = sizeof(T) == 2;   // the query-stationary kernel can read dS / dSu tiles
   if constexpr (TWO_ROLE) {
     static bool configured2 = false;
     if (!configured2) {
       if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_key2_kernel<T, TI, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_key2_lds_bytes<T, HD>()) != hipSuccess) return -3;
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_query2_kernel<T, TI, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_query2_lds_bytes<T, HD>()) != hipSuccess) return -3;
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_query2_kernel<T, TI, HD, 0>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_query2_lds_bytes<T, HD>()) != hipSuccess) return -3;
       configured2 = true;
+    }
+  } else if constexpr (TILES) {
+    static_assert(bwd_query2_lds_bytes<T, HD>() <= kMaxLds, "tile consumer does not fit the LDS");
+    static bool configured3 = false;
+    if (!configured3) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_query2_kernel<T, TI, HD, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_query2_lds_bytes<T, HD>()) != hipSuccess) return -3;
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_query2_kernel<T, TI, HD, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_query2_lds_bytes<T, HD>()) != hipSuccess) return -3;
+      configured3 = true;
     }
   }
   int rc = 0;
@@ -1455,18 +1568,26 @@ template <typename T, typename TI, int HD> static int launch_bwd_t(const BwdArgs
   }
   {
     ProfScope ps(kSlotBwdQuery, stream);
-    if constexpr (SPLIT) {
-      hipLaunchKernelGGL((bwd_query_kernel<T, TI, HD, 1>), grid, block, query_lds, stream, a);
-      hipLaunchKernelGGL((bwd_query_kernel<T, TI, HD, 2>), grid, block, query_lds, stream, a);
-    } else if constexpr (TWO_ROLE) {
-      if (a.ds_mat != nullptr) {
+    bool done = false;
+    if constexpr (TILES) {
+      if (a.ds_mat != nullptr) {   // the key kernel left the dS / dSu tiles
         constexpr int query2_lds = bwd_query2_lds_bytes<T, HD>();
-        hipLaunchKernelGGL((bwd_query2_kernel<T, TI, HD>), grid, dim3(2 * kThreads), query2_lds, stream, a);
-      } else {   // no room for the dS / dSu tiles (long sequences): the recomputing kernel
+        if constexpr (SPLIT) {
+          hipLaunchKernelGGL((bwd_query2_kernel<T, TI, HD, 1>), grid, dim3(2 * kThreads), query2_lds, stream, a);
+          hipLaunchKernelGGL((bwd_query2_kernel<T, TI, HD, 2>), grid, dim3(2 * kThreads), query2_lds, stream, a);
+        } else {
+          hipLaunchKernelGGL((bwd_query2_kernel<T, TI, HD, 0>), grid, dim3(2 * kThreads), query2_lds, stream, a);
+        }
+        done = true;
+      }
+    }
+    if (!done) {   // fp32, or no room for the tiles (long sequences): the recomputing kernel
+      if constexpr (SPLIT) {
+        hipLaunchKernelGGL((bwd_query_kernel<T, TI, HD, 1>), grid, block, query_lds, stream, a);
+        hipLaunchKernelGGL((bwd_query_kernel<T, TI, HD, 2>), grid, block, query_lds, stream, a);
+      } else {
         hipLaunchKernelGGL((bwd_query_kernel<T, TI, HD, 0>), grid, block, query_lds, stream, a);
       }
-    } else {
-      hipLaunchKernelGGL((bwd_query_kernel<T, TI, HD, 0>), grid, block, query_lds, stream, a);
     }
   }
   return hipGetLastError() == hipSuccess ? 0 : -3;
