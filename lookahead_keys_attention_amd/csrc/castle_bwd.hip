@@ -113,9 +113,12 @@ template <typename T, int HD> constexpr int bwd_key_lds_bytes() {
 
 // PART selects the outputs of a launch: 0 = all (d <= 64); 1 = dVc, dKc; 2 = dQu and the reverse
 // state (gsnap).  At d = 128 the four accumulator sets do not fit the register file together, so
-// the kernel runs once with PART 1 and once with PART 2 (the score tiles are recomputed).
-template <typename T, typename TI, int HD, int PART>
+// the kernel runs once with PART 1 and once with PART 2.  The PART 1 launch hands dS / dSu to the
+// query-stationary kernel as tiles when there is room for them; a PART 2 launch with TILES_IN
+// (after it) reads dSu from those tiles instead of evaluating the score chain a second time.
+template <typename T, typename TI, int HD, int PART, bool TILES_IN = false>
 __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
+  static_assert(!TILES_IN || (PART == 2 && sizeof(T) == 2), "only the dQu / reverse-state pass reads tiles");
   constexpr bool DO_KV = PART != 2, DO_QG = PART != 1;
   constexpr int KS = HD / 16;
   constexpr int HDP = HD < 32 ? 32 : HD;
@@ -154,14 +157,21 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   const float* lse = a.ws.lse + (int64_t)bh * a.s.Lp;
   const float* delta = a.delta + (int64_t)bh * a.s.Lp;
 
-  frag<T> fkc[KS], fvc[KS], fqu[KS], fub[KS];
+  constexpr int NSC = TILES_IN ? 1 : KS;   // the score-chain operands are not needed when dSu is read
+  frag<T> fkc[NSC], fvc[NSC], fqu[KS], fub[NSC];
 #pragma unroll
-  for (int s = 0; s < KS; ++s) {
-    fkc[s] = ldg_nat<T>(kc, HD, k, 16 * s + 8 * g, true);
-    fvc[s] = ldg_nat<T>(vc, HD, k, 16 * s + 8 * g, true);
-    fqu[s] = ldg_nat_scaled<T, T>(qu, HD, k, 16 * s + 8 * g, true, -c1);
-    fub[s] = zero_frag<T>();
+  for (int s = 0; s < KS; ++s) fqu[s] = ldg_nat_scaled<T, T>(qu, HD, k, 16 * s + 8 * g, true, -c1);
+  if constexpr (!TILES_IN) {
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      fkc[s] = ldg_nat<T>(kc, HD, k, 16 * s + 8 * g, true);
+      fvc[s] = ldg_nat<T>(vc, HD, k, 16 * s + 8 * g, true);
+      fub[s] = zero_frag<T>();
+    }
   }
+  const T* dsu_tiles = TILES_IN ? reinterpret_cast<const T*>(a.dsu_mat) + (int64_t)bh * a.s.Lp * a.s.Lp +
+                                      (int64_t)(kw0 / 32) * (a.s.Lp / 32) * 1024 + c * 16 + 8 * g
+                                : nullptr;
   acc_t dvc[NT], dkc[NT], dqu[NT], G[NT];   // [n rows, k lanes]
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) { zero(dvc[nt]); zero(dkc[nt]); zero(dqu[nt]); zero(G[nt]); }
@@ -173,14 +183,14 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   do {                                                       \
     const int64_t r_ = (int64_t)(I_) * kNB;                  \
     pqc.load_flat(qc + r_ * HD);                            \
-    pdo.load_flat(dout + r_ * HD);                        \
+    if (!TILES_IN) pdo.load_flat(dout + r_ * HD);           \
     pku.load_flat(ku + r_ * HD);                            \
     pvu.load_flat(vu + r_ * HD);                            \
     ptb.load(tb, kNB, r_, (int64_t)1 << 40);                 \
   } while (0)
 
   const int I0 = (kb * 128) / kNB;
-  constexpr bool PF = HD <= 64;   // d = 128 has no registers to spare for a block in flight
+  constexpr bool PF = HD <= 64 || TILES_IN;   // the full d = 128 passes have no registers to spare for a block in flight
   if (PF) CASTLE_BK_LOAD(a.s.nblk - 1);
   for (int I = a.s.nblk - 1; I >= I0; --I) {
     const bool active = I >= Iw;
@@ -189,20 +199,35 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
     if (DO_QG && active && I <= a.s.nblk - 2 && (a.ds_mat == nullptr || (I & 1))) {
       store_snap_tile<T, HD, NT>(gsnap + (gsnap_off(I) + kw0) * HD, G, c, g);
     }
-    if (I > Iw) {
+    if constexpr (!TILES_IN) {
+      if (I > Iw) {
 #pragma unroll
-      for (int s = 0; s < KS; ++s) fub[s] = ldg_snap_nat<T>(usnap + (usnap_off(I) + kw0) * HD, c, 16 * s + 8 * g);
+        for (int s = 0; s < KS; ++s) fub[s] = ldg_snap_nat<T>(usnap + (usnap_off(I) + kw0) * HD, c, 16 * s + 8 * g);
+      }
+    }
+    // dSu fragments of the block's sub-tiles straight from the tiles (natural order: lane = key,
+    // 8 consecutive queries), requested here and used behind the gate
+    frag<T> tdsu[TILES_IN ? BT : 1][2];
+    if constexpr (TILES_IN) {
+#pragma unroll
+      for (int it = 0; it < BT; ++it) {
+        const int i0 = I * kNB + 32 * it;
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2)
+          tdsu[it][s2] = (active && i0 + 31 >= kw0) ? *reinterpret_cast<const frag_mem<T>*>(dsu_tiles + (int64_t)(i0 / 32) * 1024 + s2 * 512)
+                                                   : zero_frag<T>();
+      }
     }
     __syncthreads();
     const int64_t r0 = (int64_t)I * kNB;
     if (!PF) CASTLE_BK_LOAD(I);
     pqc.store(s_qc, LDK);
-    pdo.store(s_do, LDK);
+    if (!TILES_IN) pdo.store(s_do, LDK);
     pku.store(s_ku, LDK);
     pvu.store_halves(s_vu, LDU);
     ptb.store_halves(s_t, LDT);
     if (PF && I > I0) CASTLE_BK_LOAD(I - 1);   // in flight while this block is processed
-    if (threadIdx.x < kNB) {
+    if (!TILES_IN && threadIdx.x < kNB) {
       const int64_t i = r0 + threadIdx.x;
       s_lse[threadIdx.x] = i < L ? lse[i] * kLog2e : INFINITY;
       s_delta[threadIdx.x] = i < L ? delta[i] : 0.f;
@@ -254,6 +279,28 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
     for (int it = 0; it < BT; ++it) {
       const int i0 = I * kNB + 32 * it;
       if (i0 + 31 < kw0) continue;   // every query precedes every key of this wave
+      if constexpr (TILES_IN) {
+        frag<T> oqt[2][NT], ott[2][BT];
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+          const int ic = 32 * it + 16 * s2;
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) oqt[s2][nt] = ld_free<T, false>(s_qc, LDK, 32 * nt, HD, ic, c, g);
+#pragma unroll
+          for (int jt = 0; jt < BT; ++jt)
+            if (jt <= it) ott[s2][jt] = ld_free<T, false>(s_t, LDT, 32 * jt, kNB, ic, c, g);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) mma(G[nt], oqt[s2][nt], tdsu[it][s2]);
+#pragma unroll
+          for (int jt = 0; jt < BT; ++jt)
+            if (jt <= it) mma(dA[jt], ott[s2][jt], tdsu[it][s2]);
+        }
+        continue;
+      }
       acc_t sc, su, dp;
       zero(sc); zero(su); zero(dp);
       {
@@ -1537,6 +1584,7 @@ template <typename T, typename TI, int HD> static int launch_bwd_t(const BwdArgs
     if (!configured3) {
       if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_query2_kernel<T, TI, HD, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_query2_lds_bytes<T, HD>()) != hipSuccess) return -3;
       if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_query2_kernel<T, TI, HD, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_query2_lds_bytes<T, HD>()) != hipSuccess) return -3;
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_key_kernel<T, TI, HD, 2, true>), hipFuncAttributeMaxDynamicSharedMemorySize, key_lds) != hipSuccess) return -3;
       configured3 = true;
     }
   }
@@ -1557,8 +1605,15 @@ template <typename T, typename TI, int HD> static int launch_bwd_t(const BwdArgs
   {
     ProfScope ps(kSlotBwdKey, stream);
     if constexpr (SPLIT) {
-      hipLaunchKernelGGL((bwd_key_kernel<T, TI, HD, 2>), grid, block, key_lds, stream, a);
-      hipLaunchKernelGGL((bwd_key_kernel<T, TI, HD, 1>), grid, block, key_lds, stream, a);
+      hipLaunchKernelGGL((bwd_key_kernel<T, TI, HD, 1>), grid, block, key_lds, stream, a);   // also writes the tiles
+      bool from_tiles = false;
+      if constexpr (TILES) {
+        if (a.ds_mat != nullptr) {
+          hipLaunchKernelGGL((bwd_key_kernel<T, TI, HD, 2, true>), grid, block, key_lds, stream, a);
+          from_tiles = true;
+        }
+      }
+      if (!from_tiles) hipLaunchKernelGGL((bwd_key_kernel<T, TI, HD, 2>), grid, block, key_lds, stream, a);
     } else if constexpr (TWO_ROLE) {
       constexpr int key2_lds = bwd_key2_lds_bytes<T, HD>();
       hipLaunchKernelGGL((bwd_key2_kernel<T, TI, HD>), grid, dim3(2 * kThreads), key2_lds, stream, a);
