@@ -41,7 +41,7 @@ template <typename T, int HD> constexpr int attn_lds_bytes() {
   return (int)sizeof(T) * (4 * kNB * lds_ld<T>(HD) + vtile_elems<T, HD>() + kNB * lds_ld<T>(128));
 }
 // register prefetch of the next tile is affordable for 16-bit operands up to d = 64
-template <typename T, int HD> constexpr bool use_prefetch() { return sizeof(T) == 2 && HD <= 64; }
+template <typename T, int HD> constexpr bool use_prefetch() { return sizeof(T) == 2; }
 
 template <typename T> __device__ __forceinline__ const T* head_ptr(const View4& v, int b, int h) {
   return reinterpret_cast<const T*>(v.ptr) + (int64_t)b * v.sb + (int64_t)h * v.sh;
