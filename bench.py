@@ -107,6 +107,51 @@ def bench_layer(steps, warmup):
     }
 
 
+def bench_long_context(steps=3, warmup=2):
+    """Benchmark configuration 3: one Castle layer forward+backward, dim 2048, 16 heads, dim_head 128,
+    batch 1, seq 16384, bf16.  Opt-in (--long-context): about 40 GB of workspace."""
+    import torch
+
+    from lookahead_keys_attention_amd import Castle, _native
+
+    dev = torch.device("cuda:0")
+    B, L, dim, H, d = 1, 16384, 2048, 16, 128
+    torch.manual_seed(0)
+    model = Castle(dim, heads=H, dim_head=d, use_triton=True).to(dev).bfloat16()
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(B, L, dim, generator=g).bfloat16().to(dev).requires_grad_()
+    gy = torch.randn(B, L, dim, generator=g).bfloat16().to(dev)
+
+    def step():
+        model.zero_grad(set_to_none=True)
+        x.grad = None
+        model(x).backward(gy)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    _native.profile_enable(True)
+    step()
+    records = _native.profile_read()
+    _native.profile_enable(False)
+    per = {}
+    for name, t in records:   # the d = 128 backward launches each kernel twice: summed per slot
+        per[name] = per.get(name, 0.0) + t
+    _, core, _ = cfg2_flops(B, H, L, d, dim)
+    core_ms = sum(per.values())
+    return {"workload": "config 3: one Castle layer forward+backward, dim 2048, 16 heads, dim_head 128, batch 1, "
+                        "seq 16384, bf16 tensors",
+            "ms_per_step": round(ms, 3), "core_ms": round(core_ms, 3),
+            "core_tflops": round(core / (core_ms * 1e-3) / 1e12, 2),
+            "frac_of_peak": round(core / (core_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
+            "kernels_ms": {k: round(v, 3) for k, v in per.items()}}
+
+
 def bench_decode(n_steps=512, prefill=2048):
     import torch
 
@@ -245,6 +290,8 @@ def main():
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-lm", action="store_true")
+    ap.add_argument("--long-context", action="store_true",
+                    help="also time benchmark configuration 3 (seq 16384, dim_head 128; ~40 GB of workspace)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device-to-device copy four times (reference for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters to bytes)")
@@ -297,6 +344,8 @@ def main():
         line["decode"] = bench_decode()
     if not args.no_lm:
         line["lm"] = bench_lm()
+    if args.long_context:
+        line["long_context"] = bench_long_context()
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline()
     print(json.dumps(line))
