@@ -108,6 +108,7 @@ template <typename T, int HD> constexpr int bwd_key_lds_bytes() {
   b += a16((int)sizeof(T) * kNB * lds_ld_chain<T>(HD));         // vu
   b += a16((int)sizeof(T) * kNB * lds_ld_chain<T>(kNB));        // T
   b += 2 * a16(4 * kNB);                                        // lse, delta
+  if (HD > 64) b += 2 * a16((int)sizeof(T) * 128 * lds_ld<T>(HD));   // kc, vc rows of the workgroup (d = 128: not in registers)
   return b;
 }
 
@@ -134,6 +135,11 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   T* s_t = cv.take<T>(kNB * LDT);
   float* s_lse = cv.take<float>(kNB);
   float* s_delta = cv.take<float>(kNB);
+  // At d = 128 the score chain takes the kc / vc rows of the workgroup's keys from LDS instead of
+  // holding them in registers: that is what leaves room for the register prefetch of the next block.
+  constexpr bool KV_LDS = HD > 64 && !TILES_IN;
+  T* s_kcw = KV_LDS ? cv.take<T>(128 * LDK) : nullptr;
+  T* s_vcw = KV_LDS ? cv.take<T>(128 * LDK) : nullptr;
 
   int kb, bh;   // key group 0 meets every query block: rank order = kb
   work_item(a.s.B * a.s.H, kb, bh);
@@ -158,15 +164,23 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   const float* delta = a.delta + (int64_t)bh * a.s.Lp;
 
   constexpr int NSC = TILES_IN ? 1 : KS;   // the score-chain operands are not needed when dSu is read
-  frag<T> fkc[NSC], fvc[NSC], fqu[KS], fub[NSC];
+  constexpr int NKV = (TILES_IN || KV_LDS) ? 1 : KS;
+  frag<T> fkc[NKV], fvc[NKV], fqu[KS], fub[NSC];
 #pragma unroll
   for (int s = 0; s < KS; ++s) fqu[s] = ldg_nat_scaled<T, T>(qu, HD, k, 16 * s + 8 * g, true, -c1);
   if constexpr (!TILES_IN) {
 #pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      fkc[s] = ldg_nat<T>(kc, HD, k, 16 * s + 8 * g, true);
-      fvc[s] = ldg_nat<T>(vc, HD, k, 16 * s + 8 * g, true);
-      fub[s] = zero_frag<T>();
+    for (int s = 0; s < KS; ++s) fub[s] = zero_frag<T>();
+    if constexpr (KV_LDS) {   // visible after the first barrier of the block loop
+      RowStage<T, T, 128, HD> st;
+      st.load_flat(kc + (int64_t)kb * 128 * HD); st.store(s_kcw, LDK);
+      st.load_flat(vc + (int64_t)kb * 128 * HD); st.store(s_vcw, LDK);
+    } else {
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        fkc[s] = ldg_nat<T>(kc, HD, k, 16 * s + 8 * g, true);
+        fvc[s] = ldg_nat<T>(vc, HD, k, 16 * s + 8 * g, true);
+      }
     }
   }
   const T* dsu_tiles = TILES_IN ? reinterpret_cast<const T*>(a.dsu_mat) + (int64_t)bh * a.s.Lp * a.s.Lp +
@@ -190,7 +204,7 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   } while (0)
 
   const int I0 = (kb * 128) / kNB;
-  constexpr bool PF = HD <= 64 || TILES_IN;   // the full d = 128 passes have no registers to spare for a block in flight
+  constexpr bool PF = true;   // every variant keeps the next block in flight in registers
   if (PF) CASTLE_BK_LOAD(a.s.nblk - 1);
   for (int I = a.s.nblk - 1; I >= I0; --I) {
     const bool active = I >= Iw;
@@ -318,8 +332,13 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
-          mma(sc, oq[s], fkc[s]);
-          mma(dp, od[s], fvc[s]);
+          if constexpr (KV_LDS) {
+            mma(sc, oq[s], ld_nat<T>(s_kcw, LDK, 32 * wave + c, 16 * s + 8 * g));
+            mma(dp, od[s], ld_nat<T>(s_vcw, LDK, 32 * wave + c, 16 * s + 8 * g));
+          } else {
+            mma(sc, oq[s], fkc[s]);
+            mma(dp, od[s], fvc[s]);
+          }
         }
         if (I > Iw) {
 #pragma unroll
