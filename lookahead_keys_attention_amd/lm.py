@@ -192,6 +192,10 @@ class CastleLM(nn.Module):
         self.__dict__["_kept_decoder"] = decoder   # not a module attribute: never part of the state
         return decoder
 
+    def release_decoder(self):
+        """Drops the graph (and the cache buffers it was captured on) kept from the last `sample` call."""
+        self.__dict__.pop("_kept_decoder", None)
+
     def _native_on_gpu(self, device) -> bool:
         return device.type == "cuda" and all(attention.use_triton for attention, _ in self.layers)
 

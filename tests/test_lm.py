@@ -199,6 +199,8 @@ def test_sampler_reuses_its_captured_graph_for_a_new_prompt():
         model.to_logits.weight = torch.nn.Parameter(model.to_logits.weight.clone())
     model.sample(tokens(2, 30, seed=3).cuda(), seq_len=50, temperature=0.0, graph=True)
     assert model._kept_decoder is not kept
+    model.release_decoder()
+    assert "_kept_decoder" not in model.__dict__
 
 
 @pytest.mark.gpu
