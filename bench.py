@@ -34,7 +34,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 1 GiB copy
 # (profiles/castle_cfg2_cfg4_pmc_hbm_traffic.txt).  Recorded values, not measured by this script.
-MEASURED_TRAFFIC_BYTES = {"scan": 724.0e6, "attn": 737.7e6, "bwd_key": 2363.5e6, "bwd_query": 1912.9e6, "decode_stream": 378.9e6}
+MEASURED_TRAFFIC_BYTES = {"scan": 722.2e6, "attn": 735.6e6, "bwd_key": 2362.4e6, "bwd_query": 1917.0e6, "decode_stream": 378.0e6}
 
 # algorithmic contractions (unit: B*H*L^2*d flop = 2*d flop per causal pair) attributed to each kernel
 KERNEL_UNITS = {"tqv": 0.0, "scan": 2.0, "attn": 3.0, "delta": 0.0, "bwd_key": 9.0, "bwd_query": 4.0}
