@@ -1574,7 +1574,8 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
 template <typename T, typename TI, int HD, int PART> static int launch_bwd_part(const BwdArgs& a, hipStream_t stream) {
   const int BH = a.s.B * a.s.H;
   constexpr int key_lds = bwd_key_lds_bytes<T, HD>(), query_lds = bwd_query_lds_bytes<T, HD>();
-  static bool configured = false;   // raising the dynamic-LDS limit is idempotent, so a race is harmless
+  static PerDeviceOnce once;
+  bool& configured = once.flag();
   if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_key_kernel<T, TI, HD, PART>), hipFuncAttributeMaxDynamicSharedMemorySize, key_lds) != hipSuccess) return -3;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_query_kernel<T, TI, HD, PART>), hipFuncAttributeMaxDynamicSharedMemorySize, query_lds) != hipSuccess) return -3;
@@ -1591,7 +1592,8 @@ template <typename T, typename TI, int HD> static int launch_bwd_t(const BwdArgs
   constexpr bool TWO_ROLE = sizeof(T) == 2 && HD <= 64;
   constexpr bool TILES = sizeof(T) == 2;   // the query-stationary kernel can read dS / dSu tiles
   if constexpr (TWO_ROLE) {
-    static bool configured2 = false;
+    static PerDeviceOnce once2;
+    bool& configured2 = once2.flag();
     if (!configured2) {
       if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_key2_kernel<T, TI, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_key2_lds_bytes<T, HD>()) != hipSuccess) return -3;
       if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_query2_kernel<T, TI, HD, 0>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_query2_lds_bytes<T, HD>()) != hipSuccess) return -3;
@@ -1599,7 +1601,8 @@ template <typename T, typename TI, int HD> static int launch_bwd_t(const BwdArgs
     }
   } else if constexpr (TILES) {
     static_assert(bwd_query2_lds_bytes<T, HD>() <= kMaxLds, "tile consumer does not fit the LDS");
-    static bool configured3 = false;
+    static PerDeviceOnce once3;
+    bool& configured3 = once3.flag();
     if (!configured3) {
       if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_query2_kernel<T, TI, HD, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_query2_lds_bytes<T, HD>()) != hipSuccess) return -3;
       if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_query2_kernel<T, TI, HD, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_query2_lds_bytes<T, HD>()) != hipSuccess) return -3;

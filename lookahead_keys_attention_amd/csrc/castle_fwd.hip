@@ -437,7 +437,8 @@ template <typename T, typename TI, int HD> static int launch_fwd_t(const FwdArgs
   const int BH = a.s.B * a.s.H;
   constexpr int scan_lds = scan_lds_bytes<T, HD>(), attn_lds = attn_lds_bytes<T, HD>();
   if (attn_lds > kMaxLds) return -2;   // this (dtype, head dim) pair does not fit the 160 KB LDS
-  static bool configured = false;      // raising the dynamic-LDS limit is idempotent, so a race is harmless
+  static PerDeviceOnce once;
+  bool& configured = once.flag();
   if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(&scan_kernel<T, TI, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, scan_lds) != hipSuccess) return -3;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_kernel<T, TI, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, attn_lds) != hipSuccess) return -3;

@@ -18,6 +18,17 @@
 
 namespace castle {
 
+// "Done once per device" flag for host-side kernel configuration (the dynamic-LDS limit of a
+// kernel is a per-device attribute).  Racing callers at worst configure twice, which is harmless.
+struct PerDeviceOnce {
+  bool done[64] = {};
+  bool& flag() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+    return done[dev];
+  }
+};
+
 typedef __bf16 bf16_t;
 typedef _Float16 fp16_t;
 template <typename T, int N> using vec = T __attribute__((ext_vector_type(N)));
