@@ -23,7 +23,7 @@
 extern "C" {
 #endif
 
-#define CASTLE_ABI_VERSION 3
+#define CASTLE_ABI_VERSION 4
 
 /* element types of the tensors (accumulation is always fp32) */
 #define CASTLE_F32 0
@@ -50,6 +50,7 @@ extern "C" {
 #define CASTLE_ERR_LAUNCH (-3)     /* HIP reported a launch / configuration error */
 #define CASTLE_ERR_WORKSPACE (-4)  /* workspace NULL, misaligned or too small */
 #define CASTLE_ERR_ARG (-5)        /* NULL pointer, misaligned pointer or stride */
+#define CASTLE_ERR_SCRATCH (-6)    /* castle_decode_step_static: partial results exceed the static scratch */
 
 /* A (B, H, L, d) tensor view: element strides for b, h and l; the d axis has stride 1.
  * ptr must be 16-byte aligned and every stride a multiple of 16 bytes / sizeof(element). */
@@ -106,14 +107,14 @@ int castle_bwd(const castle_view4* qc, const castle_view4* kc, const castle_view
 int64_t castle_decode_workspace_bytes(int B, int H, int d, int t_max);
 
 /* One cached decode step (lookahead_keys_attention.py:166-203), in place.
- * U, qu_cache, kc_cache, vc_cache: (B,H,capacity,d) buffers holding t valid rows,
- * capacity > t.  The call updates U rows 0..t-1 in place (U_k += sigmoid(s qu_k.ku) vu),
+ * U, qu_cache, kc_cache, vc_cache: (B,H,capacity,d) buffers holding t valid rows;
+ * t >= capacity is rejected (CASTLE_ERR_SHAPE) because row t is written.  The call updates U rows 0..t-1 in place (U_k += sigmoid(s qu_k.ku) vu),
  * writes row t of all four (U_t = 0, qu, kc, vc of the new token) and writes
  * out (B,H,1,d) = softmax_k(s qc.kc_k - silu(s qc.U_k)) vc_k over k = 0..t.
  * qc..vu: the new token's (B,H,1,d) operands (stride_l unused).  After the call the cache
  * holds t+1 rows.  d in {16,32,64,128}.  flags: 0 or CASTLE_FLAG_ROTARY. */
 int castle_decode_step(const castle_view4* U, const castle_view4* qu_cache,
-                       const castle_view4* kc_cache, const castle_view4* vc_cache, int t,
+                       const castle_view4* kc_cache, const castle_view4* vc_cache, int t, int capacity,
                        const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
                        const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
                        int B, int H, int d, int dtype, float scale, int flags,
@@ -135,6 +136,26 @@ int castle_decode_step_device_count(const castle_view4* U, const castle_view4* q
                                     int B, int H, int d, int dtype, float scale, int flags,
                                     const castle_view4* out,
                                     void* workspace, int64_t workspace_bytes, void* stream);
+
+/* The cached step for callers that cannot allocate or bring a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same kernels and results as castle_decode_step (t_device == NULL: row count t from
+ * the host) or castle_decode_step_device_count (t_device != NULL: t is ignored), but the partial
+ * results of the split pass live in a 4 MiB array that is part of the library's device code, one
+ * copy per GPU, held until the process ends.  The call allocates nothing and clears nothing (every
+ * partial that is read was written by the same call).  B * H * splits * (d + 2) * 4 bytes must fit
+ * the array (splits <= 64, about 640 / (B*H) for small batches: e.g. B*H up to 8065 heads at
+ * d = 128), else CASTLE_ERR_SCRATCH.  All calls on one GPU share that GPU's array: calls that
+ * overlap on one GPU (different streams, or graph replays running side by side) race.  The first
+ * call on a device looks the array's address up (hipGetSymbolAddress); make that call outside
+ * stream capture. */
+int castle_decode_step_static(const castle_view4* U, const castle_view4* qu_cache,
+                              const castle_view4* kc_cache, const castle_view4* vc_cache,
+                              int t, const int32_t* t_device, int capacity,
+                              const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
+                              const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
+                              int B, int H, int d, int dtype, float scale, int flags,
+                              const castle_view4* out, void* stream);
 
 /* Rotary position embedding of one tensor, out of place: out[b,h,l,:] = R(first_position + l) x[b,h,l,:]
  * (the rotation CASTLE_FLAG_ROTARY applies inside the kernels; lookahead_keys_attention.py:112).  Used to

@@ -14,7 +14,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libcastle_hip.so")
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 DTYPE_CODES = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
 SUPPORTED_HEAD_DIMS = (16, 32, 64, 128)
 FLAG_BF16_OPERANDS = 1   # keep bf16 MFMA operands for bf16 tensors (default: fp16 operands)
@@ -30,6 +30,7 @@ EXPORTED_SYMBOLS = (
     "castle_decode_workspace_bytes",
     "castle_decode_step",
     "castle_decode_step_device_count",
+    "castle_decode_step_static",
     "castle_rope",
     "castle_profile_enable",
     "castle_profile_read",
@@ -73,7 +74,9 @@ def _declare(lib):
     lib.castle_profile_read.restype = i
     lib.castle_profile_read.argtypes = [ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_float), i]
     lib.castle_decode_step.restype = i
-    lib.castle_decode_step.argtypes = [_VP] * 4 + [i] + [_VP] * 6 + [i, i, i, i, f, i, _VP, vp, i64, vp]
+    lib.castle_decode_step.argtypes = [_VP] * 4 + [i, i] + [_VP] * 6 + [i, i, i, i, f, i, _VP, vp, i64, vp]
+    lib.castle_decode_step_static.restype = i
+    lib.castle_decode_step_static.argtypes = [_VP] * 4 + [i, vp, i] + [_VP] * 6 + [i, i, i, i, f, i, _VP, vp]
     lib.castle_decode_step_device_count.restype = i
     lib.castle_decode_step_device_count.argtypes = [_VP] * 4 + [vp, i] + [_VP] * 6 + [i, i, i, i, f, i, _VP, vp, i64, vp]
     lib.castle_rope.restype = i

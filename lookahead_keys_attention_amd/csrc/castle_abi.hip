@@ -15,6 +15,7 @@ int launch_bwd(const BwdArgs& a, int dtype, bool bf16_operands, hipStream_t stre
 int launch_decode(const DecodeArgs& a, int dtype, hipStream_t stream);
 int launch_rope(const View4& src, const View4& dst, int B, int H, int L, int d, int dtype, int pos0, hipStream_t stream);
 int decode_pick_splits(int BH, int t);
+int decode_static_scratch(float** ptr);
 }  // namespace castle
 
 namespace {
@@ -131,6 +132,7 @@ const char* castle_error_string(int code) {
     case CASTLE_ERR_LAUNCH: return "HIP launch or configuration error";
     case CASTLE_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
     case CASTLE_ERR_ARG: return "NULL or misaligned tensor view";
+    case CASTLE_ERR_SCRATCH: return "problem too large for the static scratch of the entry point that allocates nothing";
     default: return "unknown error";
   }
 }
@@ -226,26 +228,35 @@ static int decode_step_common(const castle_view4* U, const castle_view4* qu_cach
                               const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
                               int B, int H, int d, int dtype, float scale, int flags,
                               const castle_view4* out,
-                              void* workspace, int64_t workspace_bytes, void* stream) {
+                              void* workspace, int64_t workspace_bytes, bool static_scratch, void* stream) {
   const int es = elem_size(dtype);
   if (es == 0) return CASTLE_ERR_DTYPE;
   if (B <= 0 || H <= 0 || t < 0 || capacity <= 0 || !head_dim_ok(d) || (int64_t)B * H > 65535) return CASTLE_ERR_SHAPE;
+  if (t_device == nullptr && t >= capacity) return CASTLE_ERR_SHAPE;   // row t would be written past the buffers
   const castle_view4* caches[] = {U, qu_cache, kc_cache, vc_cache};
   for (const castle_view4* v : caches)
     if (!view_ok(v, es, true)) return CASTLE_ERR_ARG;
   const castle_view4* tok[] = {qc, kc, vc, qu, ku, vu, out};
   for (const castle_view4* v : tok)
     if (!view_ok(v, es, false)) return CASTLE_ERR_ARG;
-  if (workspace == nullptr || reinterpret_cast<uintptr_t>(workspace) % 256 != 0 ||
-      workspace_bytes < castle_decode_workspace_bytes(B, H, d, t))
+  // with a device-side count the split must not depend on it: sized for a full cache
+  const int splits = castle::decode_pick_splits(B * H, t_device != nullptr ? capacity : t);
+  if (static_scratch) {
+    // the per-GPU array replaces the caller's workspace; nothing is allocated on this path
+    if ((int64_t)B * H * splits * (d + 2) * 4 > castle::kDecodeStaticScratchBytes) return CASTLE_ERR_SCRATCH;
+    float* p = nullptr;
+    if (castle::decode_static_scratch(&p) != 0) return CASTLE_ERR_LAUNCH;
+    workspace = p;
+  } else if (workspace == nullptr || reinterpret_cast<uintptr_t>(workspace) % 256 != 0 ||
+             workspace_bytes < castle_decode_workspace_bytes(B, H, d, t)) {
     return CASTLE_ERR_WORKSPACE;
+  }
 
   castle::DecodeArgs a;
   a.B = B; a.H = H; a.d = d; a.t = t; a.scale = scale;
   a.t_dev = t_device; a.capacity = capacity;
   a.rotary = (flags & CASTLE_FLAG_ROTARY) != 0;
-  // with a device-side count the split must not depend on it: sized for a full cache
-  a.splits = castle::decode_pick_splits(B * H, t_device != nullptr ? capacity : t);
+  a.splits = splits;
   a.U = to_view(U); a.qu_cache = to_view(qu_cache); a.kc_cache = to_view(kc_cache); a.vc_cache = to_view(vc_cache);
   a.qc = to_view(qc); a.kc = to_view(kc); a.vc = to_view(vc);
   a.qu = to_view(qu); a.ku = to_view(ku); a.vu = to_view(vu);
@@ -255,14 +266,26 @@ static int decode_step_common(const castle_view4* U, const castle_view4* qu_cach
 }
 
 int castle_decode_step(const castle_view4* U, const castle_view4* qu_cache,
-                       const castle_view4* kc_cache, const castle_view4* vc_cache, int t,
+                       const castle_view4* kc_cache, const castle_view4* vc_cache, int t, int capacity,
                        const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
                        const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
                        int B, int H, int d, int dtype, float scale, int flags,
                        const castle_view4* out,
                        void* workspace, int64_t workspace_bytes, void* stream) {
-  return decode_step_common(U, qu_cache, kc_cache, vc_cache, t, nullptr, 0x7fffffff, qc, kc, vc, qu, ku, vu,
-                            B, H, d, dtype, scale, flags, out, workspace, workspace_bytes, stream);
+  return decode_step_common(U, qu_cache, kc_cache, vc_cache, t, nullptr, capacity, qc, kc, vc, qu, ku, vu,
+                            B, H, d, dtype, scale, flags, out, workspace, workspace_bytes, false, stream);
+}
+
+int castle_decode_step_static(const castle_view4* U, const castle_view4* qu_cache,
+                              const castle_view4* kc_cache, const castle_view4* vc_cache,
+                              int t, const int32_t* t_device, int capacity,
+                              const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
+                              const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
+                              int B, int H, int d, int dtype, float scale, int flags,
+                              const castle_view4* out, void* stream) {
+  if (t_device != nullptr && reinterpret_cast<uintptr_t>(t_device) % 4 != 0) return CASTLE_ERR_ARG;
+  return decode_step_common(U, qu_cache, kc_cache, vc_cache, t_device != nullptr ? 0 : t, t_device, capacity,
+                            qc, kc, vc, qu, ku, vu, B, H, d, dtype, scale, flags, out, nullptr, 0, true, stream);
 }
 
 int castle_decode_step_device_count(const castle_view4* U, const castle_view4* qu_cache,
@@ -275,7 +298,7 @@ int castle_decode_step_device_count(const castle_view4* U, const castle_view4* q
                                     void* workspace, int64_t workspace_bytes, void* stream) {
   if (t_device == nullptr || reinterpret_cast<uintptr_t>(t_device) % 4 != 0) return CASTLE_ERR_ARG;
   return decode_step_common(U, qu_cache, kc_cache, vc_cache, 0, t_device, capacity, qc, kc, vc, qu, ku, vu,
-                            B, H, d, dtype, scale, flags, out, workspace, workspace_bytes, stream);
+                            B, H, d, dtype, scale, flags, out, workspace, workspace_bytes, false, stream);
 }
 
 int castle_rope(const castle_view4* x, const castle_view4* out, int B, int H, int L, int d, int dtype,

@@ -11,6 +11,7 @@
 #include "castle_tiles.h"
 #include "castle_params.h"
 #include "castle_profile.h"
+#include <mutex>
 
 namespace castle {
 
@@ -291,6 +292,28 @@ int launch_rope(const View4& src, const View4& dst, int B, int H, int L, int d, 
     case 2: return launch_rope_d<fp16_t>(src, dst, B, H, L, d, pos0, stream);
     default: return -1;
   }
+}
+
+// ---------------------------------------------------------------------------
+// Partial-result buffer of the entry point that allocates nothing: one array per GPU, part of the
+// loaded code object, alive until the process ends.  Host code never uses the array's name as an
+// address (on the host it is only a stand-in for the symbol): the device address is looked up
+// once per device and handed to the kernels like any other workspace pointer.
+static __device__ __align__(256) unsigned char scratch[kDecodeStaticScratchBytes];
+
+int decode_static_scratch(float** ptr) {
+  static std::mutex mu;
+  static void* per_device[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return -3;
+  std::lock_guard<std::mutex> lock(mu);
+  if (per_device[dev] == nullptr) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) return -3;
+    per_device[dev] = p;
+  }
+  *ptr = static_cast<float*>(per_device[dev]);
+  return 0;
 }
 
 // rows of one (b, h) handled per workgroup iteration, needed by the host to size `splits`

@@ -55,6 +55,9 @@ struct BwdArgs {
   void* dsu_mat;  // dSu
 };
 
+// size of the per-GPU partial-result array behind castle_decode_step_static
+constexpr int64_t kDecodeStaticScratchBytes = (int64_t)4 << 20;
+
 struct DecodeArgs {
   int B, H, d;
   int t;            // rows already in the cache (used when t_dev is NULL)

@@ -179,7 +179,7 @@ def castle_decode_step_hip(U, qu_cache, kc_cache, vc_cache, t, qc, kc, vc, qu, k
     views = [N.view4(x) for x in (U, qu_cache, kc_cache, vc_cache)]
     tviews = [N.view4(x) for x in toks]
     with torch.cuda.device(U.device):
-        rc = N.lib().castle_decode_step(*views, int(t), *tviews, B, H, d, code, float(scale),
+        rc = N.lib().castle_decode_step(*views, int(t), int(cap), *tviews, B, H, d, code, float(scale),
                                         N.FLAG_ROTARY if rotary else 0, N.view4(out),
                                         workspace.data_ptr(), workspace.numel(), N.stream_ptr(U.device))
     N.check(rc, "castle_decode_step")
@@ -223,7 +223,7 @@ def castle_decode_step_packed(cache_views, capacity, t, proj, heads, scale, out,
         if t_device is None:
             if not (0 <= t < capacity):
                 raise ValueError(f"cache capacity {capacity} cannot take row {t}")
-            rc = N.lib().castle_decode_step(*cache_views, int(t), qc, kc, vc, qu, ku, vu, B, heads, d,
+            rc = N.lib().castle_decode_step(*cache_views, int(t), int(capacity), qc, kc, vc, qu, ku, vu, B, heads, d,
                                             N.dtype_code(proj.dtype), float(scale), flags, vout,
                                             workspace.data_ptr(), workspace.numel(), N.stream_ptr(proj.device))
         else:
