@@ -8,11 +8,16 @@ module (lookahead_keys_attention.py:41-214), so it can replace it where the refe
     forward(x, cache=None, return_next_cache=None) -> out | (out, Cache)
 
 `use_triton` keeps its name for drop-in compatibility and selects the native kernels:
-  None  -> native HIP kernels when a GPU is present (reference: lookahead_keys_attention.py:58)
-  True  -> native HIP kernels; anything that prevents them raises
+  None  -> native HIP kernels when a GPU is present and the library is built (the reference
+           resolves None the same way, lookahead_keys_attention.py:58); such a module handed CPU
+           tensors uses the dense formulation, as the reference does when `not qc.is_cuda`
+           (lookahead_keys_attention.py:120)
+  True  -> native HIP kernels; anything that prevents them raises (missing library, CPU tensors)
   False -> the dense PyTorch formulation (the reference's own non-Triton path), any device
 On the native path both the parallel pass (seq_len > 1) and the cached single-token step
-run in HIP; nothing silently falls back.
+run in HIP.  The native step is inference-only; a single-token call that autograd would have to
+differentiate (grad mode on and the projection requires grad) takes the dense step instead, which
+is differentiable like the reference's (lookahead_keys_attention.py:166-203).
 
 Decode cache.  `Cache(U, qu_cache, kc_cache, vc_cache)` holds four (B, H, n, d) tensors as in
 the reference (lookahead_keys_attention.py:26).  Caches made by the native path are views into
@@ -87,12 +92,26 @@ def rotate_half_pairs(t, positions, theta=10000.0):
     return (x * cos + rot * sin).to(t.dtype)
 
 
+class RotaryFrequencies(nn.Module):
+    """Holds `freqs` = theta^(-2i/d), i = 0 .. d/2 - 1, as a frozen parameter: the one entry the
+    reference's third-party rotary module contributes to a state_dict (`rotary_emb.freqs`), so
+    checkpoints interchange with strict loading.  It is held for that purpose only: the kernels and
+    the dense path both evaluate the closed form in fp32 (a `.bfloat16()` model would otherwise
+    rotate by bf16-rounded frequencies on one path and exact ones on the other)."""
+
+    def __init__(self, dim, theta=10000.0):
+        super().__init__()
+        freqs = theta ** (-torch.arange(0, dim, 2, dtype=torch.float32) / dim)
+        self.freqs = nn.Parameter(freqs, requires_grad=False)
+
+
 class Castle(nn.Module):
     def __init__(self, dim, heads=8, dim_head=64, use_triton=None, rotary_emb=False, prenorm=False):
         super().__init__()
         self.dim, self.heads, self.dim_head = dim, heads, dim_head
+        self._explicit_native = use_triton is True
         if use_triton is None:
-            use_triton = torch.cuda.is_available()
+            use_triton = torch.cuda.is_available() and _native.is_built()
         if use_triton and not _native.is_built():
             raise AssertionError(
                 "native kernels requested but libcastle_hip.so is not built "
@@ -101,7 +120,10 @@ class Castle(nn.Module):
         self.use_triton = bool(use_triton)
         self.scale = dim_head ** -0.5
         self.norm = nn.RMSNorm(dim) if prenorm else nn.Identity()
-        self.rotary_emb = bool(rotary_emb)
+        # same state_dict entry as the reference's RotaryEmbedding(dim=dim_head) submodule
+        # (lookahead_keys_attention.py:71-73): `rotary_emb.freqs`, shape (dim_head / 2,)
+        self.use_rotary = bool(rotary_emb)
+        self.rotary_emb = RotaryFrequencies(dim_head) if rotary_emb else None
         inner = heads * dim_head
         self.to_all_qkv = nn.Linear(dim, inner * 6, bias=False)
         self.combine_heads = nn.Linear(inner, dim, bias=False)
@@ -125,12 +147,16 @@ class Castle(nn.Module):
         proj = self.to_all_qkv(self.norm(x))
         native = self.use_triton
         if native and not x.is_cuda:
-            raise RuntimeError("Castle(use_triton=True) runs HIP kernels and needs GPU tensors; "
-                               "construct with use_triton=False for the PyTorch formulation")
+            if self._explicit_native:
+                raise RuntimeError("Castle(use_triton=True) runs HIP kernels and needs GPU tensors; "
+                                   "construct with use_triton=False for the PyTorch formulation")
+            native = False   # auto-selected kernels, CPU tensors: the dense formulation (lookahead_keys_attention.py:120)
         if not single:
             assert cache is None, "must be inferencing single tokens if receiving cache"
             merged, next_cache = (self._parallel_native if native else self._parallel_dense)(proj, return_next_cache)
         else:
+            if native and torch.is_grad_enabled() and proj.requires_grad:
+                native = False   # the native step records no autograd graph; the dense step does
             merged, next_cache = (self._step_native if native else self._step_dense)(proj, cache)
         y = self.combine_heads(merged)
         return (y, next_cache) if return_next_cache else y
@@ -143,13 +169,13 @@ class Castle(nn.Module):
         if want_cache:
             store = _CacheStore(B, H, d, _reserve_rows(n), proj.dtype, proj.device)
         U_view = store.buffers[0][:, :, :n] if want_cache else None
-        res = ops.castle_attention_packed(proj, H, self.scale, want_cache, U_view, rotary=self.rotary_emb)
+        res = ops.castle_attention_packed(proj, H, self.scale, want_cache, U_view, rotary=self.use_rotary)
         merged = res[0] if want_cache else res
         qu, _, _, _, kc, vc = self._split(proj)
         if not want_cache:
             return merged, None
         with torch.no_grad():
-            if self.rotary_emb:   # the cache holds the rotated qu / kc rows
+            if self.use_rotary:   # the cache holds the rotated qu / kc rows
                 ops.castle_rope_hip(qu, store.buffers[1][:, :, :n])
                 ops.castle_rope_hip(kc, store.buffers[2][:, :, :n])
             else:
@@ -181,10 +207,10 @@ class Castle(nn.Module):
         out = torch.empty((B, 1, H, d), dtype=proj.dtype, device=proj.device)
         if proj.is_contiguous() and proj.data_ptr() % 16 == 0:
             ops.castle_decode_step_packed(store.views, store.capacity, t, proj, H, self.scale, out, store.workspace,
-                                          rotary=self.rotary_emb)
+                                          rotary=self.use_rotary)
         else:
             ops.castle_decode_step_hip(*store.buffers, t, qc, kc, vc, qu, ku, vu, self.scale,
-                                       out.permute(0, 2, 1, 3), store.workspace, rotary=self.rotary_emb)
+                                       out.permute(0, 2, 1, 3), store.workspace, rotary=self.use_rotary)
         store.length = t + 1
         return out.view(B, 1, H * d), store.as_cache()
 
@@ -198,14 +224,14 @@ class Castle(nn.Module):
         proj = self.to_all_qkv(self.norm(x))
         out = torch.empty((B, 1, self.heads, self.dim_head), dtype=proj.dtype, device=proj.device)
         ops.castle_decode_step_packed(store.views, store.capacity, 0, proj, self.heads, self.scale, out,
-                                      store.workspace, rotary=self.rotary_emb, t_device=t_device)
+                                      store.workspace, rotary=self.use_rotary, t_device=t_device)
         return self.combine_heads(out.view(B, 1, self.heads * self.dim_head))
 
     # -- dense PyTorch formulation (use_triton=False) -------------------------
     def _parallel_dense(self, proj, want_cache):
         B, n, _ = proj.shape
         qu, ku, vu, qc, kc, vc = self._split(proj)
-        if self.rotary_emb:
+        if self.use_rotary:
             qc, kc, qu, ku, vu = self._rotate((qc, kc, qu, ku, vu), 0, n, proj.device)
         s = self.scale
         future = torch.ones(n, n, dtype=torch.bool, device=proj.device).triu(1)
@@ -225,7 +251,7 @@ class Castle(nn.Module):
             cache = (empty,) * 4
         U, qu_hist, kc_hist, vc_hist = cache
         t = kc_hist.shape[-2]
-        if self.rotary_emb:
+        if self.use_rotary:
             qc, kc, qu, ku, vu = self._rotate((qc, kc, qu, ku, vu), t, 1, proj.device)
         s = self.scale
         gate = torch.sigmoid((qu_hist * s) @ ku.mT)

@@ -23,8 +23,15 @@ How each function is pinned (tests/test_oracle_*.py):
   lm_forward         composition of module_forward with library routines (embedding,
                      rms_norm, gelu, cross_entropy): parallel == cached sequential,
                      causality, and loss = ln(vocabulary) for zero logits weights.
-Rotary embedding (LKA:71-73,106-112) depends on a third-party package that is
-not present; it is not restated here: parity unpinned for rotary_emb=True.
+  rope               rotary embedding written as a complex multiplication; pinned by its
+                     closed-form properties (tests/test_oracle_core.py): position 0 is the
+                     identity, norms are kept, R(p) R(q) = R(p + q), the dot product of two
+                     rotated rows depends on the position difference only, and pair i at
+                     position p turns by exactly p * 10000^(-2i/d) radians.  The reference
+                     delegates rotary embedding to `rotary-embedding-torch>=0.8.9`
+                     (LKA:13,73,112; pyproject.toml:29), which is absent: agreement with
+                     THAT package is parity unpinned; this is the published RoPE formula
+                     over interleaved pairs, which is what that package documents.
 """
 from __future__ import annotations
 
@@ -70,6 +77,22 @@ def parallel_core(qc, kc, vc, qu, ku, vu, scale, want_U=False):
     if not want_U:
         return out
     return out, torch.matmul(A, vu)                              # LKA:161-163
+
+
+# --------------------------------------------------------------------------
+# rotary position embedding                                      LKA:71-73,106-112
+# --------------------------------------------------------------------------
+def rope(t, positions, theta=10000.0):
+    """Rows of t (..., n, d) rotated by their absolute positions (n,): the pair
+    (t[2i], t[2i+1]) is read as the complex number t[2i] + 1j t[2i+1] and multiplied by
+    exp(1j * position * theta^(-2i/d)).  LKA:112 applies this to qc, kc, qu, ku, vu with
+    offset = number of cached rows."""
+    d = t.shape[-1]
+    z = torch.view_as_complex(t.double().reshape(*t.shape[:-1], d // 2, 2).contiguous())
+    freq = torch.tensor([theta ** (-2.0 * i / d) for i in range(d // 2)], dtype=torch.float64)
+    turn = torch.polar(torch.ones(len(positions), d // 2, dtype=torch.float64),
+                       positions.double()[:, None] * freq[None, :])
+    return torch.view_as_real(z * turn).reshape(t.shape).to(t.dtype)
 
 
 # --------------------------------------------------------------------------

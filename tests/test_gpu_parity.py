@@ -105,39 +105,35 @@ def test_bf16_operand_flag_forward_and_backward(L, d, monkeypatch):
 @pytest.mark.parametrize("B,Hh,L,d,dtype", [(1, 2, 200, 64, torch.float32), (2, 2, 300, 64, torch.bfloat16),
                                             (1, 2, 130, 32, torch.float16), (1, 1, 260, 128, torch.bfloat16)])
 def test_rotary_inside_the_kernels(B, Hh, L, d, dtype):
-    """FLAG_ROTARY: rotating inside the kernels == the operator on operands rotated beforehand
-    (fp32 rotation, the formula of castle.rotate_half_pairs), forward, final lookahead keys and the
-    gradients with respect to the UN-rotated operands (chain rule through the rotation)."""
-    from lookahead_keys_attention_amd.castle import rotate_half_pairs
-
+    """FLAG_ROTARY: rotating inside the kernels == the operator on operands rotated beforehand by
+    the oracle's rotary embedding (complex multiplication, fp64), forward, final lookahead keys and
+    the gradients with respect to the UN-rotated operands (chain rule through the rotation)."""
     ops, dout = rand_ops(B, Hh, L, d, dtype, seed=5 * L + d)
     s = d ** -0.5
     leaves = [t.to(DEV).requires_grad_() for t in ops]
     out, U = H().castle_attention_hip(*leaves, s, True, rotary=True)
     out.backward(dout.to(DEV))
     pos = torch.arange(L)
-    rot = [t.double() if idx == 2 else rotate_half_pairs(t.float(), pos).double() for idx, t in enumerate(ops)]
+    rot = [t.double() if idx == 2 else O.rope(t.double(), pos) for idx, t in enumerate(ops)]
     ref_out, ref_U = O.parallel_core(*rot, s, want_U=True)
     assert_close(out, ref_out, dtype, "out", 1e-3)
     assert_close(U, ref_U, dtype, "U", 1e-3)
     # gradients: closed forms with respect to the rotated operands, rotated back (transpose = -angle)
     g_rot = O.closed_form_grads(*rot, s, dout.double())
-    inv = lambda g: rotate_half_pairs(g.float(), -pos).double()
+    inv = lambda g: O.rope(g, -pos)
     for idx, (name, leaf) in enumerate(zip(NAMES, leaves)):
         want = g_rot[idx] if idx == 2 else inv(g_rot[idx])
         assert_close(leaf.grad, want, dtype, name, 2e-2)
 
 
 def test_rope_entry_point_matches_formula():
-    from lookahead_keys_attention_amd.castle import rotate_half_pairs
-
     x = torch.randn(2, 3, 77, 64, generator=torch.Generator().manual_seed(2))
     for dtype, tol in ((torch.float32, 1e-4), (torch.bfloat16, 2e-2)):
         xs = x.to(dtype).to(DEV)
         out = torch.empty_like(xs)
         H().castle_rope_hip(xs, out, first_position=11)
-        want = rotate_half_pairs(x.to(dtype).float(), torch.arange(11, 11 + 77))
-        assert (out.float().cpu() - want).abs().max() <= tol
+        want = O.rope(x.to(dtype).double(), torch.arange(11, 11 + 77))
+        assert (out.double().cpu() - want).abs().max() <= tol
 
 
 def test_backward_without_score_tiles(monkeypatch):

@@ -88,3 +88,49 @@ def test_plain_tuple_cache_is_accepted_on_dense_path():
         y1, _ = m(x[:, 4:], cache=tuple(cache))
         y2, _ = m(x[:, 4:], cache=cache)
     assert torch.equal(y1, y2)
+
+
+def test_rotary_state_dict_entry_matches_the_reference_module():
+    # the reference holds RotaryEmbedding(dim=dim_head) as `rotary_emb` (lookahead_keys_attention.py:71-73),
+    # whose only state entry is the frozen frequency vector theta^(-2i/d)
+    m = Castle(32, heads=2, dim_head=16, use_triton=False, rotary_emb=True)
+    sd = m.state_dict()
+    assert set(sd) == {"to_all_qkv.weight", "combine_heads.weight", "rotary_emb.freqs"}
+    expect = 1.0 / (10000.0 ** (torch.arange(0, 16, 2).float() / 16))
+    assert torch.allclose(sd["rotary_emb.freqs"], expect, rtol=1e-6, atol=0)
+    assert not m.rotary_emb.freqs.requires_grad
+    other = Castle(32, heads=2, dim_head=16, use_triton=False, rotary_emb=True)
+    other.load_state_dict(sd, strict=True)
+    assert "rotary_emb.freqs" not in Castle(32, heads=2, dim_head=16, use_triton=False).state_dict()
+
+
+def test_auto_selected_kernels_fall_back_to_dense_on_cpu_tensors(monkeypatch):
+    # use_triton=None resolves like the reference (lookahead_keys_attention.py:58) and a CPU tensor
+    # then takes the dense path (lookahead_keys_attention.py:120); only an explicit True insists
+    monkeypatch.setattr(torch.cuda, "is_available", lambda: True)
+    torch.manual_seed(4)
+    auto = Castle(32, heads=2, dim_head=16)
+    assert auto.use_triton is True
+    dense = Castle(32, heads=2, dim_head=16, use_triton=False)
+    dense.load_state_dict(auto.state_dict())
+    x = torch.randn(1, 6, 32)
+    with torch.no_grad():
+        assert torch.equal(auto(x), dense(x))
+    from lookahead_keys_attention_amd import _native
+    monkeypatch.setattr(_native, "is_built", lambda: False)
+    assert Castle(32, heads=2, dim_head=16).use_triton is False      # no library: not selected
+    with pytest.raises(AssertionError):
+        Castle(32, heads=2, dim_head=16, use_triton=True)
+
+
+def test_single_token_call_is_differentiable_when_grad_is_needed():
+    # lookahead_keys_attention.py:166-203 is plain differentiable PyTorch; a module whose native step
+    # is inference-only must not return an output cut off from its parameters
+    torch.manual_seed(5)
+    m = Castle(32, heads=2, dim_head=16, use_triton=False)
+    x = torch.randn(1, 3, 32)
+    with torch.no_grad():
+        _, cache = m(x[:, :2], return_next_cache=True)
+    y, _ = m(x[:, 2:], cache=cache)
+    y.sum().backward()
+    assert m.to_all_qkv.weight.grad is not None and m.to_all_qkv.weight.grad.abs().sum() > 0

@@ -176,3 +176,41 @@ def test_readme_config_parallel_vs_sequential_fp32():
         y, cache = O.module_forward(x[:, t:t + 1], p, 8, cache=cache)
         ys.append(y)
     assert torch.allclose(torch.cat(ys, 1), full, atol=1e-3)
+
+
+def test_rope_closed_form_properties():
+    """The oracle's rotary embedding against what the mathematics fixes (no formula retyped):
+    identity at position 0; norm preserving; additive in the position; the dot product of two
+    rotated rows depends on the position difference only; pair i at position p turns by exactly
+    p * 10000^(-2i/d) radians (checked through the angle of a unit vector)."""
+    g = torch.Generator().manual_seed(9)
+    d, n = 16, 7
+    x = torch.randn(2, n, d, generator=g, dtype=torch.float64)
+    y = torch.randn(2, n, d, generator=g, dtype=torch.float64)
+    pos = torch.tensor([0, 1, 2, 5, 9, 30, 1000])
+    r = O.rope(x, pos)
+    assert torch.equal(r[:, 0], x[:, 0])
+    assert torch.allclose(r.norm(dim=-1), x.norm(dim=-1), atol=1e-12)
+    assert torch.allclose(O.rope(O.rope(x, pos), pos + 3), O.rope(x, 2 * pos + 3), atol=1e-9)
+    assert torch.allclose(O.rope(O.rope(x, pos), -pos), x, atol=1e-9)
+    dots = (O.rope(x, pos + 4) * O.rope(y, pos + 1)).sum(-1)
+    assert torch.allclose(dots, (O.rope(x, pos + 103) * O.rope(y, pos + 100)).sum(-1), atol=1e-8)
+    e = torch.zeros(1, 1, d, dtype=torch.float64)
+    e[..., 0::2] = 1.0                                   # every pair is the unit vector (1, 0)
+    turned = O.rope(e, torch.tensor([3]))
+    angle = torch.atan2(turned[0, 0, 1::2], turned[0, 0, 0::2])
+    want = torch.tensor([math.remainder(3.0 * 10000.0 ** (-2.0 * i / d), 2 * math.pi) for i in range(d // 2)], dtype=torch.float64)
+    assert torch.allclose(angle, want, atol=1e-12)
+    # interleaved pairs: only elements 2i and 2i+1 mix
+    one = torch.zeros(1, 1, d, dtype=torch.float64)
+    one[..., 4] = 1.0
+    out = O.rope(one, torch.tensor([2]))
+    assert (out[0, 0].abs() > 1e-9).nonzero().flatten().tolist() == [4, 5]
+
+
+def test_dense_module_rotation_equals_oracle_rope():
+    from lookahead_keys_attention_amd.castle import rotate_half_pairs
+
+    x = torch.randn(2, 3, 40, 32, generator=torch.Generator().manual_seed(4))
+    pos = torch.arange(5, 45)
+    assert torch.allclose(rotate_half_pairs(x, pos).double(), O.rope(x.double(), pos), atol=1e-4)
