@@ -42,6 +42,10 @@ extern "C" {
  * appends the rotated qu, kc rows.  The final lookahead keys U are those of the rotated operands. */
 #define CASTLE_FLAG_BF16_OPERANDS 1
 #define CASTLE_FLAG_ROTARY 2
+/* castle_bwd / castle_bwd_workspace_bytes only: do not hand dS / dSu tiles from the first backward
+ * kernel to the second (2 * B * H * Lp * Lp elements of workspace); the second kernel recomputes
+ * the score chain instead.  Slower, for callers short of memory. */
+#define CASTLE_FLAG_RECOMPUTE_SCORES 4
 
 /* error codes */
 #define CASTLE_OK 0
@@ -85,9 +89,10 @@ int castle_fwd(const castle_view4* qc, const castle_view4* kc, const castle_view
 /* Bytes of extra device workspace castle_bwd needs: reverse state snapshots, delta, a copy of dout in
  * the compute type and, for the 16-bit element types, the dS / dSu score-gradient tiles its first
  * kernel hands to its second (2 * B * H * Lp * Lp elements, Lp = L rounded up to 128; left out, and
- * the score chain recomputed instead, when they would exceed 40 GiB or the byte count in the
- * environment variable CASTLE_MAX_SCORE_TILE_BYTES). */
-int64_t castle_bwd_workspace_bytes(int B, int H, int L, int d, int dtype);
+ * the score chain recomputed instead, under CASTLE_FLAG_RECOMPUTE_SCORES or when they would exceed
+ * 40 GiB, or the byte count found in the environment variable CASTLE_MAX_SCORE_TILE_BYTES when
+ * the library first needed it).  `flags`: those the castle_bwd call will get. */
+int64_t castle_bwd_workspace_bytes(int B, int H, int L, int d, int dtype, int flags);
 
 /* Parallel backward.  Same operands as castle_fwd plus the forward output `out`, the
  * upstream gradient `dout` and the forward workspace as castle_fwd left it.  Writes the six

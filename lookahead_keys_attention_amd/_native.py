@@ -19,6 +19,7 @@ DTYPE_CODES = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
 SUPPORTED_HEAD_DIMS = (16, 32, 64, 128)
 FLAG_BF16_OPERANDS = 1   # keep bf16 MFMA operands for bf16 tensors (default: fp16 operands)
 FLAG_ROTARY = 2          # rotary position embedding of qc, kc, qu, ku, vu inside the kernels
+FLAG_RECOMPUTE_SCORES = 4   # backward without the dS / dSu tile hand-over (less workspace, slower)
 
 EXPORTED_SYMBOLS = (
     "castle_abi_version",
@@ -62,7 +63,7 @@ def _declare(lib):
     lib.castle_fwd_workspace_bytes.restype = i64
     lib.castle_fwd_workspace_bytes.argtypes = [i, i, i, i, i]
     lib.castle_bwd_workspace_bytes.restype = i64
-    lib.castle_bwd_workspace_bytes.argtypes = [i, i, i, i, i]
+    lib.castle_bwd_workspace_bytes.argtypes = [i, i, i, i, i, i]
     lib.castle_decode_workspace_bytes.restype = i64
     lib.castle_decode_workspace_bytes.argtypes = [i, i, i, i]
     lib.castle_fwd.restype = i

@@ -39,18 +39,25 @@ int64_t align_up(int64_t x, int64_t a) { return (x + a - 1) / a * a; }
 // falls back to recomputing the score chain in its second kernel
 constexpr int64_t kMaxScoreTileBytes = (int64_t)40 << 30;
 // CASTLE_MAX_SCORE_TILE_BYTES in the environment overrides the limit (0 = never use the tiles)
+// (read once, when the library first needs it, so that castle_bwd_workspace_bytes and castle_bwd
+// cannot disagree)
 int64_t max_score_tile_bytes() {
-  const char* e = getenv("CASTLE_MAX_SCORE_TILE_BYTES");
-  return e != nullptr ? strtoll(e, nullptr, 10) : kMaxScoreTileBytes;
+  static const int64_t limit = [] {
+    const char* e = getenv("CASTLE_MAX_SCORE_TILE_BYTES");
+    return e != nullptr ? strtoll(e, nullptr, 10) : kMaxScoreTileBytes;
+  }();
+  return limit;
 }
 
 struct Geometry {
   int Lp, nblk;
   int64_t lse_bytes, tblk_bytes, snap_bytes, mat_bytes, op_bytes;
   int64_t off_lse, off_t, off_tt, off_ttx, off_snap, off_ops, total;
+  int64_t bwd_total;
 };
+constexpr int64_t kHeaderBytes = 256 + 4 * castle::kAmaxBlocks;   // header + partial maxima, forward and backward alike
 
-Geometry geometry(int B, int H, int L, int d, int es) {
+Geometry geometry(int B, int H, int L, int d, int es, int flags = 0) {
   Geometry g;
   g.Lp = (int)align_up(L, 128);
   g.nblk = g.Lp / kNB;
@@ -60,8 +67,9 @@ Geometry geometry(int B, int H, int L, int d, int es) {
   g.snap_bytes = align_up(BH * castle::snap_rows(g.nblk) * d * es, 256);
   // dS / dSu tiles between the two backward kernels: the 16-bit paths use them
   g.mat_bytes = es == 2 ? align_up(BH * g.Lp * g.Lp * es, 256) : 0;
-  if (2 * g.mat_bytes > max_score_tile_bytes()) g.mat_bytes = 0;   // too long: the query kernel recomputes the scores instead
-  g.off_lse = 0;
+  // too long, or the caller asks for it: the query kernel recomputes the scores instead
+  if (2 * g.mat_bytes > max_score_tile_bytes() || (flags & CASTLE_FLAG_RECOMPUTE_SCORES)) g.mat_bytes = 0;
+  g.off_lse = kHeaderBytes;
   g.off_t = g.off_lse + g.lse_bytes;
   g.off_tt = g.off_t + g.tblk_bytes;
   g.off_ttx = g.off_tt + g.tblk_bytes;
@@ -69,6 +77,8 @@ Geometry geometry(int B, int H, int L, int d, int es) {
   g.op_bytes = align_up(BH * g.Lp * d * es, 256);   // one operand in the compute type, padded to Lp rows
   g.off_ops = g.off_snap + g.snap_bytes;
   g.total = g.off_ops + 6 * g.op_bytes;
+  // header, reverse-state snapshots, delta, dO copy, dS / dSu tiles
+  g.bwd_total = kHeaderBytes + g.snap_bytes + g.lse_bytes + g.op_bytes + 2 * g.mat_bytes;
   return g;
 }
 
@@ -104,6 +114,8 @@ int check_core(int B, int H, int L, int d, int dtype) {
 castle::FwdWorkspace carve(void* base, const Geometry& g) {
   char* p = static_cast<char*>(base);
   castle::FwdWorkspace w;
+  w.hdr = reinterpret_cast<castle::WsHeader*>(p);
+  w.amax_part = reinterpret_cast<float*>(p + 256);
   w.lse = reinterpret_cast<float*>(p + g.off_lse);
   w.t_blk = p + g.off_t;
   w.tt_blk = p + g.off_tt;
@@ -171,11 +183,11 @@ int castle_fwd(const castle_view4* qc, const castle_view4* kc, const castle_view
   return castle::launch_fwd(a, dtype, (flags & CASTLE_FLAG_BF16_OPERANDS) != 0, static_cast<hipStream_t>(stream));
 }
 
-int64_t castle_bwd_workspace_bytes(int B, int H, int L, int d, int dtype) {
+int64_t castle_bwd_workspace_bytes(int B, int H, int L, int d, int dtype, int flags) {
   const int rc = check_core(B, H, L, d, dtype);
   if (rc != CASTLE_OK) return rc;
-  const Geometry g = geometry(B, H, L, d, elem_size(dtype));
-  return g.snap_bytes + g.lse_bytes + g.op_bytes + 2 * g.mat_bytes;   // reverse-state snapshots, delta, dO copy, dS / dSu tiles
+  const Geometry g = geometry(B, H, L, d, elem_size(dtype), flags);
+  return g.bwd_total;
 }
 
 int castle_bwd(const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
@@ -192,11 +204,11 @@ int castle_bwd(const castle_view4* qc, const castle_view4* kc, const castle_view
   const castle_view4* in[] = {qc, kc, vc, qu, ku, vu, out, dout, dqc, dkc, dvc, dqu, dku, dvu};
   for (const castle_view4* v : in)
     if (!view_ok(v, es, true)) return CASTLE_ERR_ARG;
-  const Geometry g = geometry(B, H, L, d, es);
+  const Geometry g = geometry(B, H, L, d, es, flags);
   if (fwd_workspace == nullptr || reinterpret_cast<uintptr_t>(fwd_workspace) % 256 != 0 || fwd_workspace_bytes < g.total)
     return CASTLE_ERR_WORKSPACE;
   if (bwd_workspace == nullptr || reinterpret_cast<uintptr_t>(bwd_workspace) % 256 != 0 ||
-      bwd_workspace_bytes < g.snap_bytes + g.lse_bytes + g.op_bytes + 2 * g.mat_bytes)
+      bwd_workspace_bytes < g.bwd_total)
     return CASTLE_ERR_WORKSPACE;
 
   castle::BwdArgs a;
@@ -208,11 +220,15 @@ int castle_bwd(const castle_view4* qc, const castle_view4* kc, const castle_view
   a.dqc = to_view(dqc); a.dkc = to_view(dkc); a.dvc = to_view(dvc);
   a.dqu = to_view(dqu); a.dku = to_view(dku); a.dvu = to_view(dvu);
   a.ws = carve(const_cast<void*>(fwd_workspace), g);
-  a.gsnap = bwd_workspace;
-  a.delta = reinterpret_cast<float*>(static_cast<char*>(bwd_workspace) + g.snap_bytes);
-  a.dout_p = static_cast<char*>(bwd_workspace) + g.snap_bytes + g.lse_bytes;
-  a.ds_mat = g.mat_bytes ? static_cast<char*>(bwd_workspace) + g.snap_bytes + g.lse_bytes + g.op_bytes : nullptr;
-  a.dsu_mat = g.mat_bytes ? static_cast<char*>(bwd_workspace) + g.snap_bytes + g.lse_bytes + g.op_bytes + g.mat_bytes : nullptr;
+  char* bw = static_cast<char*>(bwd_workspace);
+  a.bhdr = reinterpret_cast<castle::BwdHeader*>(bw);
+  a.amax_part = reinterpret_cast<float*>(bw + 256);
+  bw += kHeaderBytes;
+  a.gsnap = bw;
+  a.delta = reinterpret_cast<float*>(bw + g.snap_bytes);
+  a.dout_p = bw + g.snap_bytes + g.lse_bytes;
+  a.ds_mat = g.mat_bytes ? bw + g.snap_bytes + g.lse_bytes + g.op_bytes : nullptr;
+  a.dsu_mat = g.mat_bytes ? bw + g.snap_bytes + g.lse_bytes + g.op_bytes + g.mat_bytes : nullptr;
   return castle::launch_bwd(a, dtype, (flags & CASTLE_FLAG_BF16_OPERANDS) != 0, static_cast<hipStream_t>(stream));
 }
 

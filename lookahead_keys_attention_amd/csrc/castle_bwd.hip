@@ -84,6 +84,15 @@ __global__ __launch_bounds__(kThreads) void delta_kernel(BwdArgs a) {
   const int bh = blockIdx.y, b = bh / a.s.H, h = bh % a.s.H;
   const int grp = threadIdx.x / LPR, sub = threadIdx.x % LPR;
   const int64_t i = (int64_t)blockIdx.x * RPB + grp;
+  // 16-bit operands: the whole backward runs on dO * gs, gs the power of two that puts max|dO| into
+  // [16, 32), so that neither tiny nor huge upstream gradients leave the fp16 range on their way
+  // through dS, dSu, dZ and the reverse state; the gradient stores multiply by 1 / gs
+  float gs = 1.f;
+  if constexpr (sizeof(T) == 2) gs = pow2_placing(amax_from_partials(a.amax_part), 4);
+  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
+    a.bhdr->grad_scale = gs;
+    a.bhdr->grad_unscale = 1.f / gs;
+  }
   if (i >= a.s.Lp) return;
   float acc = 0.f;
   vt d;
@@ -95,10 +104,13 @@ __global__ __launch_bounds__(kThreads) void delta_kernel(BwdArgs a) {
 #pragma unroll
     for (int e = 0; e < V; ++e) acc = __builtin_fmaf((float)o[e], (float)d[e], acc);
   }
-  *reinterpret_cast<vec<T, V>*>(reinterpret_cast<T*>(a.dout_p) + ((int64_t)bh * a.s.Lp + i) * HD + sub * V) = cvt_vec<T, TI, V>(d);
+  vec<float, V> ds = __builtin_convertvector(d, vec<float, V>);
+#pragma unroll
+  for (int e = 0; e < V; ++e) ds[e] *= gs;
+  *reinterpret_cast<vec<T, V>*>(reinterpret_cast<T*>(a.dout_p) + ((int64_t)bh * a.s.Lp + i) * HD + sub * V) = __builtin_convertvector(ds, vec<T, V>);
 #pragma unroll
   for (int o = 1; o < LPR; o <<= 1) acc += __shfl_xor(acc, o);
-  if (sub == 0) a.delta[(int64_t)bh * a.s.Lp + i] = acc;
+  if (sub == 0) a.delta[(int64_t)bh * a.s.Lp + i] = acc * gs;
 }
 
 // ---------------------------------------------------------------------------
@@ -147,6 +159,7 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   const int lane = lane_id(), wave = wave_id(), c = lane & 31, g = lane >> 5;
   const int L = a.s.L;
   const float c0 = a.s.scale, c1 = a.s.scale * kLog2e;
+  const float su_mul = a.ws.hdr->su_mul, gun = a.bhdr->grad_unscale;
   const int kw0 = kb * 128 + 32 * wave;
   const int k = kw0 + c;
   const int Iw = kw0 / kNB;
@@ -355,17 +368,18 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int il = 32 * it + acc_row(r, g);
-        const float sg = fast_rcp(1.f + fast_exp2(-su[r]));
-        const float x = __builtin_fmaf(-su[r], sg, sc[r]);
+        const float sut = su[r] * su_mul;                 // log2(e) * Su
+        const float sg = fast_rcp(1.f + fast_exp2(-sut));
+        const float x = __builtin_fmaf(-sut, sg, sc[r]);
         float p = fast_exp2(x - s_lse[il]);
         if (diag && I * kNB + il < k) p = 0.f;
         const float dsv = p * (dp[r] - s_delta[il]);
-        const float y = su[r] * kLn2;                     // true Su
+        const float y = sut * kLn2;                       // true Su
         const float t = __builtin_fmaf(-y, sg, y);        // y (1 - sigmoid)
         const float sp = __builtin_fmaf(sg, t, sg);       // silu'(y)
         sc[r] = p;
         ds[r] = dsv;
-        dsu[r] = -dsv * sp;
+        dsu[r] = -dsv * sp * su_mul;                      // gradient of the product built from vu * vu_scale
       }
       if constexpr (DO_KV && sizeof(T) == 2) {
         if (a.ds_mat != nullptr) {   // hand the tile to the tile-consuming query kernel: element (k, i) at (i/16)*512 + k*16 + i%16
@@ -439,10 +453,10 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
 #undef CASTLE_BK_LOAD
   if (k < L) {
     if constexpr (DO_KV) {
-      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dkc, b, h) + (int64_t)k * a.dkc.sl, dkc, kLn2, g, a.s.rotary ? k : -1);
-      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvc, b, h) + (int64_t)k * a.dvc.sl, dvc, 1.f, g);
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dkc, b, h) + (int64_t)k * a.dkc.sl, dkc, kLn2 * gun, g, a.s.rotary ? k : -1);
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvc, b, h) + (int64_t)k * a.dvc.sl, dvc, gun, g);
     }
-    if constexpr (DO_QG) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqu, b, h) + (int64_t)k * a.dqu.sl, dqu, c0 * kLn2, g, a.s.rotary ? k : -1);
+    if constexpr (DO_QG) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqu, b, h) + (int64_t)k * a.dqu.sl, dqu, c0 * kLn2 * gun, g, a.s.rotary ? k : -1);
   }
 }
 
@@ -497,6 +511,7 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_key2_kernel(BwdArgs a) {
   const int pw = wave & 3;
   const int L = a.s.L;
   const float c0 = a.s.scale, c1 = a.s.scale * kLog2e;
+  const float su_mul = a.ws.hdr->su_mul, gun = a.bhdr->grad_unscale;
   const int kw0 = kb * 128 + 32 * pw;
   const int k = kw0 + c;
   const int Iw = kw0 / kNB;
@@ -669,15 +684,16 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_key2_kernel(BwdArgs a) {
           }
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            const float sg = fast_rcp(1.f + fast_exp2(-su[r]));
-            const float p = fast_exp2(__builtin_fmaf(-su[r], sg, sc[r]));   // sc carries -lse
+            const float sut = su[r] * su_mul;                 // log2(e) * Su
+            const float sg = fast_rcp(1.f + fast_exp2(-sut));
+            const float p = fast_exp2(__builtin_fmaf(-sut, sg, sc[r]));   // sc carries -lse
             const float dsv = p * dp[r];                      // dp carries -delta
-            const float y = su[r] * kLn2;                     // true Su
+            const float y = sut * kLn2;                       // true Su
             const float t = __builtin_fmaf(-y, sg, y);        // y (1 - sigmoid)
             const float sp = __builtin_fmaf(sg, t, sg);       // silu'(y)
             sc[r] = p;
             ds[r] = dsv;
-            dsu[r] = -dsv * sp;
+            dsu[r] = -dsv * sp * su_mul;                      // gradient of the product built from vu * vu_scale
           }
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
@@ -796,9 +812,9 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_key2_kernel(BwdArgs a) {
     if (I0 >= Iw) CASTLE_BK2_DQU(I0);
 #undef CASTLE_BK2_DQU
     if (k < L) {
-      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dkc, b, h) + (int64_t)k * a.dkc.sl, dkc, kLn2, g, a.s.rotary ? k : -1);
-      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvc, b, h) + (int64_t)k * a.dvc.sl, dvc, 1.f, g);
-      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqu, b, h) + (int64_t)k * a.dqu.sl, dqu, c0 * kLn2, g, a.s.rotary ? k : -1);
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dkc, b, h) + (int64_t)k * a.dkc.sl, dkc, kLn2 * gun, g, a.s.rotary ? k : -1);
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvc, b, h) + (int64_t)k * a.dvc.sl, dvc, gun, g);
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqu, b, h) + (int64_t)k * a.dqu.sl, dqu, c0 * kLn2 * gun, g, a.s.rotary ? k : -1);
     }
   }
 #undef CASTLE_BK2_STAGE_DECL
@@ -851,6 +867,7 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
   const int lane = lane_id(), wave = wave_id(), c = lane & 31, g = lane >> 5;
   const int L = a.s.L;
   const float c0 = a.s.scale, c1 = a.s.scale * kLog2e;
+  const float su_mul = a.ws.hdr->su_mul, gun = a.bhdr->grad_unscale, vu_scale = a.ws.hdr->vu_scale;
   const int i0w = qb * QB + 32 * wave;
   const int i = i0w + c;                      // this lane's row: a query in phase 1, a source in phase 2
   const int Ifirst = (qb * QB) / kNB;
@@ -997,16 +1014,17 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
       const bool diag = ks + 31 > i0w;   // sub-tile reaches the diagonal
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const float sg = fast_rcp(1.f + fast_exp2(-su[r]));
-        const float x = __builtin_fmaf(-su[r], sg, sc[r]);
+        const float sut = su[r] * su_mul;                 // log2(e) * Su
+        const float sg = fast_rcp(1.f + fast_exp2(-sut));
+        const float x = __builtin_fmaf(-sut, sg, sc[r]);
         float p = fast_exp2(x - lse2);
         if (diag && ks + acc_row(r, g) > i) p = 0.f;
         const float dsv = p * (dp[r] - dlt);
-        const float y = su[r] * kLn2;                     // true Su
+        const float y = sut * kLn2;                       // true Su
         const float t = __builtin_fmaf(-y, sg, y);
         const float sp = __builtin_fmaf(sg, t, sg);
         ds[r] = dsv;
-        dsu[r] = -dsv * sp;
+        dsu[r] = -dsv * sp * su_mul;                      // gradient of the product built from vu * vu_scale
       }
       if constexpr (DO_S) {
 #pragma unroll
@@ -1140,10 +1158,10 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
       mma(dvu[nt], ld_free<T, false>(e_qcw, LDK, 32 * nt, HD, 16 * s, c, g), fdt);
   }
   if (i < L) {
-    if constexpr (DO_Q) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqc, b, h) + (int64_t)i * a.dqc.sl, dqc, c0, g, a.s.rotary ? i : -1);
+    if constexpr (DO_Q) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqc, b, h) + (int64_t)i * a.dqc.sl, dqc, c0 * gun, g, a.s.rotary ? i : -1);
     if constexpr (DO_S) {
-      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dku, b, h) + (int64_t)i * a.dku.sl, dku, c0 * kLn2, g, a.s.rotary ? i : -1);
-      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvu, b, h) + (int64_t)i * a.dvu.sl, dvu, kLn2, g, a.s.rotary ? i : -1);
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dku, b, h) + (int64_t)i * a.dku.sl, dku, c0 * kLn2 * gun, g, a.s.rotary ? i : -1);
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvu, b, h) + (int64_t)i * a.dvu.sl, dvu, kLn2 * gun * vu_scale, g, a.s.rotary ? i : -1);
     }
   }
 }
@@ -1239,6 +1257,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
   const int tid = threadIdx.x & (kThreads - 1);   // thread index inside the role
   const int L = a.s.L;
   const float c0 = a.s.scale, c1 = a.s.scale * kLog2e;
+  const float gun = a.bhdr->grad_unscale, vu_scale = a.ws.hdr->vu_scale;
   const int jw = 32 * pw;                     // rows of this wave pair inside the 128-row exchange tiles
   const int i0w = qb * QB + jw;
   const int i = i0w + c;                      // this lane's row
@@ -1433,7 +1452,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
     }
     __syncthreads();   // e2: epilogue tiles and dT shared
     if constexpr (DO_S) {
-      if (i < L) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dku, b, h) + (int64_t)i * a.dku.sl, dku, c0 * kLn2, g, a.s.rotary ? i : -1);
+      if (i < L) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dku, b, h) + (int64_t)i * a.dku.sl, dku, c0 * kLn2 * gun, g, a.s.rotary ? i : -1);
     }
   } else {
     acc_t dqc[DO_Q ? NT : 1];   // [n rows, i lanes]
@@ -1564,15 +1583,15 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
       }
     }
     if (i < L) {
-      if constexpr (DO_Q) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqc, b, h) + (int64_t)i * a.dqc.sl, dqc, c0, g, a.s.rotary ? i : -1);
-      if constexpr (DO_S) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvu, b, h) + (int64_t)i * a.dvu.sl, dvu, kLn2, g, a.s.rotary ? i : -1);
+      if constexpr (DO_Q) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqc, b, h) + (int64_t)i * a.dqc.sl, dqc, c0 * gun, g, a.s.rotary ? i : -1);
+      if constexpr (DO_S) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvu, b, h) + (int64_t)i * a.dvu.sl, dvu, kLn2 * gun * vu_scale, g, a.s.rotary ? i : -1);
     }
   }
 }
 
 // ---------------------------------------------------------------------------
-template <typename T, typename TI, int HD, int PART> static int launch_bwd_part(const BwdArgs& a, hipStream_t stream) {
-  const int BH = a.s.B * a.s.H;
+// raises the dynamic-LDS limit of the single-role kernels (once per device); launches nothing
+template <typename T, typename TI, int HD, int PART> static int configure_single_role_kernels() {
   constexpr int key_lds = bwd_key_lds_bytes<T, HD>(), query_lds = bwd_query_lds_bytes<T, HD>();
   static PerDeviceOnce once;
   bool& configured = once.flag();
@@ -1612,16 +1631,19 @@ template <typename T, typename TI, int HD> static int launch_bwd_t(const BwdArgs
   }
   int rc = 0;
   if constexpr (SPLIT) {
-    rc = launch_bwd_part<T, TI, HD, 1>(a, stream);
-    if (rc == 0) rc = launch_bwd_part<T, TI, HD, 2>(a, stream);
+    rc = configure_single_role_kernels<T, TI, HD, 1>();
+    if (rc == 0) rc = configure_single_role_kernels<T, TI, HD, 2>();
   } else {
-    rc = launch_bwd_part<T, TI, HD, 0>(a, stream);
+    rc = configure_single_role_kernels<T, TI, HD, 0>();
   }
   if (rc != 0) return rc;
   constexpr int RPB = kThreads / (HD / elem_traits<T>::vec16);
   const dim3 grid(a.s.Lp / 128 * BH), block(kThreads);
   {
     ProfScope ps(kSlotDelta, stream);
+    if constexpr (sizeof(T) == 2)
+      hipLaunchKernelGGL((amax_kernel<TI, HD>), dim3(kAmaxBlocks), dim3(kThreads), 0, stream, a.dout, a.s.H, a.s.L,
+                         (int64_t)BH * a.s.L, a.amax_part, (int*)nullptr);
     hipLaunchKernelGGL((delta_kernel<T, TI, HD>), dim3((a.s.Lp + RPB - 1) / RPB, BH), block, 0, stream, a);
   }
   {

@@ -72,6 +72,21 @@ __global__ __launch_bounds__(kThreads) void prep_kernel(FwdArgs a) {
     case 4: src = a.ku; dstv = a.ws.ku_p; break;
     default: src = a.vu; dstv = a.ws.vu_p; break;
   }
+  if constexpr (sizeof(T) == 2) {
+    if (blockIdx.z == 5) {   // vu is brought into the range that keeps every lookahead state finite in fp16
+      mul = vu_scale_for(amax_from_partials(a.ws.amax_part), a.s.L);
+      if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
+        a.ws.hdr->vu_scale = mul;
+        a.ws.hdr->su_mul = 1.f / mul;
+      }
+    }
+  } else {
+    if (blockIdx.z == 5 && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
+      a.ws.hdr->status = 0;
+      a.ws.hdr->vu_scale = 1.f;
+      a.ws.hdr->su_mul = 1.f;
+    }
+  }
   vec<float, V> f;
 #pragma unroll
   for (int e = 0; e < V; ++e) f[e] = 0.f;
@@ -83,6 +98,17 @@ __global__ __launch_bounds__(kThreads) void prep_kernel(FwdArgs a) {
   }
 #pragma unroll
   for (int e = 0; e < V; ++e) f[e] *= mul;
+  if constexpr (__is_same(T, fp16_t) && !__is_same(TI, fp16_t)) {
+    // wider input type: values beyond the fp16 range are clamped (and reported in the header)
+    bool clamped = false;
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      const float y = __builtin_amdgcn_fmed3f(f[e], -kHalfMax, kHalfMax);
+      clamped |= y != f[e] && f[e] == f[e];
+      f[e] = y;
+    }
+    if (clamped) atomicOr(&a.ws.hdr->status, 1);
+  }
   T* dst = reinterpret_cast<T*>(dstv) + ((int64_t)bh * a.s.Lp + row) * HD + cv * V;
   *reinterpret_cast<vec<T, V>*>(dst) = __builtin_convertvector(f, vec<T, V>);
 }
@@ -120,6 +146,17 @@ __global__ __launch_bounds__(kThreads) void tqv_kernel(FwdArgs a) {
   for (int s = 0; s < KS; ++s) {
     mma(acc, fq[s], fv[s]);
     mma(accx, fx[s], fv[s]);
+  }
+  if constexpr (__is_same(T, fp16_t)) {   // T' beyond the fp16 range is clamped (and reported in the header)
+    bool clamped = false;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float y = __builtin_amdgcn_fmed3f(acc[r], -kHalfMax, kHalfMax), yx = __builtin_amdgcn_fmed3f(accx[r], -kHalfMax, kHalfMax);
+      clamped |= (y != acc[r] && acc[r] == acc[r]) || (yx != accx[r] && accx[r] == accx[r]);
+      acc[r] = y;
+      accx[r] = yx;
+    }
+    if (clamped) atomicOr(&a.ws.hdr->status, 2);
   }
   // acc[r] = (Qc' Vu^T)[il = 32 it + acc_row][jl = 32 jt + c]; stored as T' = tril(.)
   const int jl = 32 * jt + c;
@@ -224,6 +261,11 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(FwdArgs a) {
   }
   if (a.U.ptr != nullptr && k < L) {
     TI* dst = head_ptr_mut<TI>(a.U, b, h) + (int64_t)k * a.U.sl;
+    const float su_mul = a.ws.hdr->su_mul;   // the state was built from vu * vu_scale
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) st[nt][r] *= su_mul;
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -259,6 +301,7 @@ __global__ __launch_bounds__(kThreads, (sizeof(T) == 2 && HD <= 64) ? 2 : 1) voi
   const int lane = lane_id(), wave = wave_id(), c = lane & 31, g = lane >> 5;
   const int L = a.s.L;
   const float c1 = a.s.scale * kLog2e;
+  const float su_mul = a.ws.hdr->su_mul;   // Su = su_mul * (the product built from vu * vu_scale)
   const int i0w = qb * QB + 32 * wave;
   const int i = i0w + c;
   const int Ifirst = (qb * QB) / kNB;
@@ -377,8 +420,9 @@ __global__ __launch_bounds__(kThreads, (sizeof(T) == 2 && HD <= 64) ? 2 : 1) voi
         float mx = -INFINITY;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const float sg = fast_rcp(1.f + fast_exp2(-su[r]));
-          sc[r] = __builtin_fmaf(-su[r], sg, sc[r]);
+          const float sut = su[r] * su_mul;
+          const float sg = fast_rcp(1.f + fast_exp2(-sut));
+          sc[r] = __builtin_fmaf(-sut, sg, sc[r]);
         }
         if (k0 + 31 > i0w) {   // tile touches the diagonal: causal mask
 #pragma unroll
@@ -447,6 +491,9 @@ template <typename T, typename TI, int HD> static int launch_fwd_t(const FwdArgs
   {
     ProfScope ps(kSlotTqv, stream);
     constexpr int PIECES_PER_ROW = HD / elem_traits<T>::vec16;
+    if constexpr (sizeof(T) == 2)
+      hipLaunchKernelGGL((amax_kernel<TI, HD>), dim3(kAmaxBlocks), dim3(kThreads), 0, stream, a.vu, a.s.H, a.s.L,
+                         (int64_t)BH * a.s.L, a.ws.amax_part, &a.ws.hdr->status);
     hipLaunchKernelGGL((prep_kernel<T, TI, HD>), dim3((a.s.Lp * PIECES_PER_ROW + kThreads - 1) / kThreads, BH, 6), dim3(kThreads), 0, stream, a);
     hipLaunchKernelGGL((tqv_kernel<T, TI, HD>), dim3(a.s.nblk, BH), dim3(kThreads), 0, stream, a);
   }

@@ -18,8 +18,27 @@ struct CoreShape {
   int rotary;   // 1: qc, kc, qu, ku, vu are rotated by their row position (RoPE) inside the kernels
 };
 
+// Header of the forward workspace (its first 256 bytes), written on the device by the forward pass.
+// The kernels work on vu_s = vu * vu_scale (a power of two <= 1 chosen from max|vu| so that no
+// lookahead state can leave the fp16 range: L * max|vu_s| <= 2^15); the scores use
+// Su = su_mul * Su_s with su_mul = 1 / vu_scale.  For fp32 tensors both are 1.
+struct WsHeader {
+  int status;       // bit 0: an input element was clamped to the fp16 range; bit 1: a T' element was
+  float vu_scale;
+  float su_mul;
+};
+constexpr int kAmaxBlocks = 256;   // partial maxima written by amax_kernel
+// the same for the backward pass: the kernels work on dO * grad_scale (a power of two that puts
+// max|dO| into [16, 32)) and multiply the gradients by grad_unscale = 1 / grad_scale when storing
+struct BwdHeader {
+  float grad_scale;
+  float grad_unscale;
+};
+
 // Workspace written by the forward pass and read again by the backward pass.
 struct FwdWorkspace {
+  WsHeader* hdr;
+  float* amax_part;   // [kAmaxBlocks] partial maxima of |vu|
   void* t_blk;    // [B*H][Lp][kNB]  T[i][j_local]  = tril(Qc_I Vu_I^T), unscaled
   void* tt_blk;   // [B*H][Lp][kNB]  T^T per block: [j][i_local]
   void* ttx_blk;  // [B*H][Lp][kNB]  rows j of even blocks I: (Qc'_{I+1} Vu_I^T)^T [j][i_local of block I+1]; odd blocks unused
@@ -44,6 +63,8 @@ struct BwdArgs {
   View4 qc, kc, vc, qu, ku, vu, out, dout;
   View4 dqc, dkc, dvc, dqu, dku, dvu;
   FwdWorkspace ws;
+  BwdHeader* bhdr;
+  float* amax_part;   // [kAmaxBlocks] partial maxima of |dO|
   void* gsnap;    // [B*H][snap_rows(nblk)][d]  reverse state at block ends
   float* delta;   // [B*H][Lp]  rowsum(dO * O)
   // Score-gradient tiles handed from the key-stationary to the query-stationary kernel (16-bit

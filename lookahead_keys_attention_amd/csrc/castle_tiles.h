@@ -15,6 +15,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include "castle_params.h"
 
 namespace castle {
 
@@ -561,6 +562,64 @@ __device__ __forceinline__ vec<float, 2> rope_rot(float x0, float x1, float pos,
     (X0) = y_[0];                                                              \
     (X1) = y_[1];                                                              \
   } while (0)
+
+// ---- range control ------------------------------------------------------------------------
+// Partial maxima of |x| over a (B, H, L, HD) view: kAmaxBlocks workgroups, one partial each.  The
+// consumers reduce the partials themselves (amax_from_partials), so no atomics and no clearing.
+template <typename TI, int HD>
+__global__ __launch_bounds__(kThreads) void amax_kernel(View4 x, int H, int L, int64_t rows, float* part, int* status) {
+  constexpr int V = elem_traits<TI>::vec16;
+  constexpr int VPR = HD / V;
+  if (status != nullptr && blockIdx.x == 0 && threadIdx.x == 0) *status = 0;
+  float m = 0.f;
+  const int64_t pieces = rows * VPR;
+  for (int64_t p = (int64_t)blockIdx.x * kThreads + threadIdx.x; p < pieces; p += (int64_t)gridDim.x * kThreads) {
+    const int64_t row = p / VPR;
+    const int cv = (int)(p % VPR);
+    const int64_t bh = row / L, l = row % L;
+    const TI* src = reinterpret_cast<const TI*>(x.ptr) + (bh / H) * x.sb + (bh % H) * x.sh + l * x.sl + cv * V;
+    const vec<float, V> f = __builtin_convertvector(*reinterpret_cast<const vec<TI, V>*>(src), vec<float, V>);
+#pragma unroll
+    for (int e = 0; e < V; ++e) m = fmaxf(m, fabsf(f[e]));   // fmaxf drops NaNs
+  }
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) m = fmaxf(m, __shfl_xor(m, o));
+  __shared__ float s_m[kThreads / 64];
+  if ((threadIdx.x & 63) == 0) s_m[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int w = 1; w < kThreads / 64; ++w) m = fmaxf(m, s_m[w]);
+    part[blockIdx.x] = fminf(m, 3.0e38f);   // an infinite input counts as the largest finite value
+  }
+}
+// max of the partials, by every thread of a wave (64 lanes x 4 partials)
+__device__ __forceinline__ float amax_from_partials(const float* part) {
+  static_assert(kAmaxBlocks == 256, "one load of four partials per lane");
+  const vec<float, 4> v = *reinterpret_cast<const vec<float, 4>*>(part + 4 * lane_id());
+  float m = fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]));
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) m = fmaxf(m, __shfl_xor(m, o));
+  return m;
+}
+// the power of two 2^k with  2^lo <= x * 2^k < 2^(lo+1)  (1 for x == 0)
+__device__ __forceinline__ float pow2_placing(float x, int lo) {
+  if (!(x > 0.f)) return 1.f;
+  int e;
+  (void)frexpf(x, &e);   // x = f * 2^e, f in [0.5, 1)
+  int k = lo + 1 - e;
+  k = k < -100 ? -100 : (k > 100 ? 100 : k);
+  return ldexpf(1.f, k);
+}
+// vu_scale: the largest power of two <= 1 with  L * max|vu| * scale <= 2^15
+__device__ __forceinline__ float vu_scale_for(float amax_vu, int L) {
+  const float bound = amax_vu * (float)L;
+  if (!(bound > 32768.f)) return 1.f;
+  int e;
+  (void)frexpf(bound, &e);   // bound < 2^e
+  return ldexpf(1.f, 15 - e);
+}
+constexpr float kHalfMax = 65504.f;
 
 // head bh of an operand copy in the compute type ([B*H][Lp][HD] contiguous, rows >= L zero)
 template <typename T> __device__ __forceinline__ const T* prep_ptr(const void* base, int bh, int Lp, int HD) {

@@ -23,6 +23,10 @@ from . import _native as N
 # flags handed to castle_fwd / castle_bwd (0, or _native.FLAG_BF16_OPERANDS); read when the
 # forward runs and remembered for its backward.  The `rotary` arguments below add FLAG_ROTARY.
 DEFAULT_FLAGS = 0
+# Debugging aid: when True every parallel forward waits for its kernels and raises if they had to
+# clamp a value to the fp16 range (an input element of a bf16 tensor beyond +-65504, or a T' entry):
+# the result is then that of the clamped operands.  Off by default because it synchronises.
+CHECK_RANGE = False
 
 
 def _require_gpu(t: torch.Tensor, what: str):
@@ -50,14 +54,25 @@ def _fwd_raw(qc, kc, vc, qu, ku, vu, scale, out, U, flags=0):
     with torch.cuda.device(qc.device):
         rc = lib.castle_fwd(*views, B, H, L, d, code, float(scale), int(flags), vo, vU, ws.data_ptr(), nbytes, N.stream_ptr(qc.device))
     N.check(rc, "castle_fwd")
+    if CHECK_RANGE:
+        status = range_status(ws)
+        if status:
+            raise RuntimeError(f"castle_fwd clamped values to the fp16 range (status bits {status:#x}: "
+                               "1 = input element, 2 = T' = s qc.vu entry)")
     return ws
+
+
+def range_status(ws: torch.Tensor) -> int:
+    """Status word the forward kernels leave at the start of their workspace (synchronises):
+    bit 0 = an input element was clamped to +-65504, bit 1 = an entry of T' = s qc.vu was."""
+    return int(ws[:4].view(torch.int32).item())
 
 
 def _bwd_raw(qc, kc, vc, qu, ku, vu, out, dout, scale, grads, ws, flags=0):
     B, H, L, d = qc.shape
     code = N.dtype_code(qc.dtype)
     lib = N.lib()
-    nbytes = N.check(lib.castle_bwd_workspace_bytes(B, H, L, d, code), "castle_bwd_workspace_bytes")
+    nbytes = N.check(lib.castle_bwd_workspace_bytes(B, H, L, d, code, int(flags)), "castle_bwd_workspace_bytes")
     bws = torch.empty(nbytes, dtype=torch.uint8, device=qc.device)
     views = [N.view4(t) for t in (qc, kc, vc, qu, ku, vu, out, dout)]
     gviews = [N.view4(t) for t in grads]

@@ -22,7 +22,12 @@ How each function is pinned (tests/test_oracle_*.py):
                      sequential, causality) with default-initialised weights.
   lm_forward         composition of module_forward with library routines (embedding,
                      rms_norm, gelu, cross_entropy): parallel == cached sequential,
-                     causality, and loss = ln(vocabulary) for zero logits weights.
+                     causality, loss = ln(vocabulary) for zero logits weights, and the
+                     wiring cases a missing residual or a misplaced norm would fail: with
+                     every attention and feed-forward output projection zeroed the logits
+                     are rms_norm(embedding) @ W exactly; with only the feed-forward ones
+                     zeroed the hidden state is embedding + sum of the layers' attention
+                     outputs, each computed by module_forward on the running state.
   rope               rotary embedding written as a complex multiplication; pinned by its
                      closed-form properties (tests/test_oracle_core.py): position 0 is the
                      identity, norms are kept, R(p) R(q) = R(p + q), the dot product of two
@@ -143,7 +148,10 @@ def split_projection(proj, heads):
 
 
 def module_forward(x, params, heads, cache=None, return_next_cache=None):
-    """Functional restatement of Castle.forward without rotary (LKA:82-214)."""
+    """Functional restatement of Castle.forward (LKA:82-214).  A `rotary_emb.freqs` entry in
+    `params` (the state entry of the reference's rotary submodule, LKA:71-73) switches the rotary
+    embedding on: qc, kc, qu, ku, vu are rotated by their absolute positions, offset by the number
+    of cached rows (LKA:106-112); the rotation is `rope` above, not the third-party module."""
     w_qkv, w_out = params["to_all_qkv.weight"], params["combine_heads.weight"]
     d = w_qkv.shape[0] // (6 * heads)
     scale = d ** -0.5                                            # LKA:63
@@ -154,6 +162,10 @@ def module_forward(x, params, heads, cache=None, return_next_cache=None):
     if "norm.weight" in params:                                  # LKA:67,95 (RMSNorm, eps=None)
         x = F.rms_norm(x, (x.shape[-1],), params["norm.weight"])
     qu, ku, vu, qc, kc, vc = split_projection(x @ w_qkv.t(), heads)   # LKA:99-104
+    if "rotary_emb.freqs" in params:                             # LKA:106-112
+        offset = cache[2].shape[-2] if cache is not None else 0
+        pos = torch.arange(offset, offset + n)
+        qc, kc, qu, ku, vu = (rope(t, pos) for t in (qc, kc, qu, ku, vu))
     nxt = None
     if not single:
         assert cache is None, "must be inferencing single tokens if receiving cache"   # LKA:117
@@ -171,7 +183,7 @@ def module_forward(x, params, heads, cache=None, return_next_cache=None):
 
 def lm_forward(tokens, params, heads, depth, return_loss=False, cache=None, return_next_cache=False):
     """Functional restatement of the reference's language model around the layer
-    (train_triton.py:141-175), without rotary: embedding, `depth` x [h += castle(h); h += ff(h)]
+    (train_triton.py:141-175): embedding, `depth` x [h += castle(h); h += ff(h)]
     with ff = RMSNorm, Linear(4x), GELU, Linear (train_triton.py:103-108), final RMSNorm, logits,
     and the shift-by-one cross entropy (train_triton.py:143-144,172-175).
     params: state-dict style keys of the module tree (token_emb.weight, layers.<i>.0.<castle key>,

@@ -46,9 +46,10 @@ def test_workspace_sizes(lib):
     # B4 H8 L4096 d64 bf16: lse + three T arrays (T', T'^T, cross quarter) + snapshots (64 * nblk*(nblk-1)/2 rows per head) + six operand copies
     n = lib.castle_fwd_workspace_bytes(4, 8, 4096, 64, 1)
     BH, Lp, nblk = 32, 4096, 64
-    expect = BH * Lp * 4 + 3 * BH * Lp * 64 * 2 + BH * 64 * nblk * (nblk - 1) // 2 * 64 * 2 + 6 * BH * Lp * 64 * 2
+    header = 256 + 4 * 256   # status / scale header + partial maxima
+    expect = header + BH * Lp * 4 + 3 * BH * Lp * 64 * 2 + BH * 64 * nblk * (nblk - 1) // 2 * 64 * 2 + 6 * BH * Lp * 64 * 2
     assert n == expect
-    assert lib.castle_bwd_workspace_bytes(4, 8, 4096, 64, 1) == BH * 64 * nblk * (nblk - 1) // 2 * 64 * 2 + BH * Lp * 4 + BH * Lp * 64 * 2 + 2 * BH * Lp * Lp * 2
+    assert lib.castle_bwd_workspace_bytes(4, 8, 4096, 64, 1, 0) == header + BH * 64 * nblk * (nblk - 1) // 2 * 64 * 2 + BH * Lp * 4 + BH * Lp * 64 * 2 + 2 * BH * Lp * Lp * 2
     # ragged L rounds up to 128 rows
     assert lib.castle_fwd_workspace_bytes(1, 1, 129, 64, 0) == lib.castle_fwd_workspace_bytes(1, 1, 256, 64, 0)
     assert lib.castle_decode_workspace_bytes(32, 8, 64, 4096) > 0

@@ -205,32 +205,50 @@ def test_config3_bf16_long_context_forward_backward():
 
 
 def test_config4_bf16_decode_after_prefill():
-    # benchmark configuration 4: B32, prefill 2048 through the parallel path, then cached steps
+    """benchmark configuration 4 at full size: B32, prefill 2048 through the parallel path, then all
+    512 cached steps with fresh x_t ~ N(0,1).  The native decode's per-head output (before the
+    output projection) of sampled (b, h) is compared at steps 1, 256 and 512 with the oracle's
+    decode_core iterated in fp32 on that head from the oracle's own prefill, and so are the head's
+    lookahead keys in the cache after the last step.  The cache is a bf16 tensor in this
+    configuration, as in the reference, whose step forms `U = U_prev + gate * vu` in the module
+    dtype (lookahead_keys_attention.py:183): the oracle's lookahead keys are therefore rounded to
+    bf16 after every step, like any other bf16 input of the next step.  Against a cache kept in
+    fp32 the 512 roundings show: the last step differs from the parallel pass (fp32 state) by about
+    5e-2 normwise, which is asserted as a bound here and is a property of a bf16 cache."""
     m = make(512, 8, 64, dtype=torch.bfloat16, seed=0).eval()
     g = torch.Generator().manual_seed(0)
-    steps = 4
-    x = torch.randn(32, 2048 + steps, 512, generator=g).bfloat16().to(DEV)
+    steps, t0 = 512, 2048
+    x = torch.randn(32, t0 + steps, 512, generator=g).bfloat16().to(DEV)
+    heads = [(17, 3), (0, 0), (31, 7)]
+    watch = {1, 256, 512}
+    native = {}
     with torch.no_grad():
-        _, cache = m(x[:, :2048], return_next_cache=True)
-        ys = []
-        for t in range(2048, 2048 + steps):
-            y, cache = m(x[:, t:t + 1], cache=cache)
-            ys.append(y)
-        full = m(x)
-    assert cache.U.shape == (32, 8, 2048 + steps, 64)
-    bf16_close(torch.cat(ys, 1), full[:, 2048:], "cached steps vs parallel")
-    # one (b, h) slice of the first step against the oracle's cached step in fp32
-    with torch.no_grad():
-        proj = m.to_all_qkv(x[:, :2049]).view(32, 2049, 6, 8, 64)
-    b, h = 17, 3
-    qu, ku, vu, qc, kc, vc = [proj[b, :, i, h].float().cpu() for i in range(6)]
-    _, U0 = O.parallel_core(*[t[:2048] for t in (qc, kc, vc, qu, ku, vu)], m.scale, want_U=True)
-    step, _ = O.decode_core((U0, qu[:2048], kc[:2048], vc[:2048]), *[t[2048:] for t in (qc, kc, vc, qu, ku, vu)], m.scale)
-    w = m.combine_heads.weight.detach().float().cpu()
-    # compare pre-projection head output: recompute native merged output for that head via the cache-free parallel path
-    from lookahead_keys_attention_amd import ops
-
-    with torch.no_grad():
-        merged = ops.castle_attention_packed(m.to_all_qkv(x[:, :2049]), 8, m.scale)
-    bf16_close(merged.view(32, 2049, 8, 64)[b, 2048, h], step[0], "row 2048 of head vs oracle decode")
-    del w
+        proj_all = m.to_all_qkv(x).view(32, t0 + steps, 6, 8, 64)
+        _, cache = m(x[:, :t0], return_next_cache=True)
+        for n in range(1, steps + 1):
+            t = t0 + n - 1
+            merged, cache = m._step_native(m.to_all_qkv(x[:, t:t + 1]), cache)
+            if n in watch:
+                native[n] = merged.view(32, 8, 64).float().cpu()
+        # the module's own step (projection included) agrees with the parallel pass on the last row
+        full_last = m(x)[:, -1]
+    assert cache.U.shape == (32, 8, t0 + steps, 64)
+    last = m.combine_heads(merged)[:, 0].double().cpu()
+    drift = ((last - full_last.double().cpu()).norm() / full_last.double().norm()).item()
+    assert drift <= 1e-1, f"last cached step vs parallel: {drift:.3e}"
+    for b, h in heads:
+        qu, ku, vu, qc, kc, vc = [proj_all[b, :, i, h].float().cpu() for i in range(6)]
+        _, U0 = O.parallel_core(*[t[:t0] for t in (qc, kc, vc, qu, ku, vu)], m.scale, want_U=True)
+        state = (U0, qu[:t0], kc[:t0], vc[:t0])
+        for n in range(1, steps + 1):
+            t = t0 + n - 1
+            out, state = O.decode_core(state, *[z[t:t + 1] for z in (qc, kc, vc, qu, ku, vu)], m.scale)
+            state = state._replace(U=state.U.bfloat16().float())
+            if n in watch:
+                bf16_close(native[n][b, h], out[0], f"decode step {n} of head ({b},{h}) vs oracle")
+        # 512 independent roundings to bf16 on either side: single elements wander by a few ulps, so the
+        # lookahead keys are held to the normwise half of the bf16 rule
+        gotU = cache.U[b, h].double().cpu()
+        relU = ((gotU - state.U.double()).norm() / state.U.double().norm()).item()
+        assert relU <= 2e-2, f"lookahead keys of head ({b},{h}) after {steps} steps: {relU:.3e}"
+        assert torch.equal(cache.kc_cache[b, h].float().cpu(), kc) and torch.equal(cache.qu_cache[b, h].float().cpu(), qu)

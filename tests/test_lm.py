@@ -55,6 +55,57 @@ def test_oracle_lm_loss_is_log_vocab_for_zero_logits():
     assert abs(loss.item() - math.log(VOCAB)) < 1e-12
 
 
+def test_oracle_lm_wiring_residuals_and_norms():
+    """What a missing residual or a misplaced norm would fail.  (1) Output projections of every
+    attention and feed-forward block zeroed: only the residual stream is left, so the logits are
+    rms_norm(embedding) @ W.  (2) Only the feed-forward projections zeroed: the stream before the
+    final norm is embedding + attention(layer 0) + attention(layer 1), each attention evaluated
+    by module_forward on the running stream (pre-norm inside the layer, LKA:67,95).  (3) Only the
+    attention projections zeroed: the stream is x + ff0(x) + ff1(x + ff0(x)), ff = W2 gelu(W1 rms_norm(.))."""
+    F = torch.nn.functional
+    model = make_lm(depth=2, rotary=True)
+    p = params_of(model)
+    x = tokens(2, 9)
+    emb = p["token_emb.weight"][x]
+    head = lambda h: F.rms_norm(h, (h.shape[-1],), p["final_norm.weight"]) @ p["to_logits.weight"].t()
+    zero = lambda q, keys: {k: (torch.zeros_like(v) if k.endswith(keys) else v) for k, v in q.items()}
+    both = zero(p, ("0.combine_heads.weight", "1.3.weight"))
+    assert torch.allclose(O.lm_forward(x, both, 2, 2), head(emb), atol=1e-12)
+    no_ff = zero(p, ("1.3.weight",))
+    layer = lambda i: {k[len(f"layers.{i}.0."):]: v for k, v in p.items() if k.startswith(f"layers.{i}.0.")}
+    h = emb + O.module_forward(emb, layer(0), 2)
+    h = h + O.module_forward(h, layer(1), 2)
+    assert torch.allclose(O.lm_forward(x, no_ff, 2, 2), head(h), atol=1e-10)
+    no_attn = zero(p, ("0.combine_heads.weight",))
+    ff = lambda i, h: F.gelu(F.rms_norm(h, (h.shape[-1],), p[f"layers.{i}.1.0.weight"]) @ p[f"layers.{i}.1.1.weight"].t()) @ p[f"layers.{i}.1.3.weight"].t()
+    h = emb + ff(0, emb)
+    h = h + ff(1, h)
+    assert torch.allclose(O.lm_forward(x, no_attn, 2, 2), head(h), atol=1e-10)
+
+
+def test_oracle_module_with_rotary_parallel_equals_cached_and_is_causal():
+    """The reference's own properties for rotary_emb=True (tests/test_lookahead.py:10-64,145-182 of
+    the reference), on the oracle: 8 parallel tokens + 8 cached steps == 16 parallel tokens; the
+    first half does not see the second."""
+    torch.manual_seed(3)
+    dim, heads, d = 32, 2, 16
+    p = O.default_init(dim, heads, d, seed=3)
+    p = {k: v.double() for k, v in p.items()}
+    p["rotary_emb.freqs"] = torch.zeros(d // 2)
+    x = torch.randn(2, 16, dim, dtype=torch.float64)
+    full = O.module_forward(x, p, heads)
+    y, cache = O.module_forward(x[:, :8], p, heads, return_next_cache=True)
+    outs = [y]
+    for t in range(8, 16):
+        y, cache = O.module_forward(x[:, t:t + 1], p, heads, cache=cache)
+        outs.append(y)
+    assert torch.allclose(torch.cat(outs, 1), full, atol=1e-9)
+    assert torch.allclose(O.module_forward(x[:, :8], p, heads), full[:, :8], atol=1e-12)
+    q = dict(p)
+    del q["rotary_emb.freqs"]
+    assert not torch.allclose(O.module_forward(x, q, heads), full, atol=1e-3)   # the rotation does something
+
+
 # ---------------------------------------------------------------- host logic
 def test_top_k_keeps_the_largest_fraction():
     logits = torch.randn(3, 50, generator=torch.Generator().manual_seed(0))
@@ -237,14 +288,41 @@ def test_decode_step_with_an_out_of_range_device_count_writes_nothing():
 
 @pytest.mark.gpu
 def test_config5_language_model_step_bf16():
-    """benchmark configuration 5: 12 x [Castle(512, 8 heads, 64) + MLP], tied embedding, (16, 1024) tokens,
-    forward + loss + backward."""
+    """benchmark configuration 5 at full size: 12 x [Castle(512, 8 heads, 64) + MLP], tied embedding,
+    rotary + prenorm, (16, 1024) tokens, bf16, forward + loss + backward on the native path, against
+    the oracle's lm_forward in fp32 on the same bf16-rounded weights (CPU): the full-size loss
+    (forward only on the CPU: the dense autograd graph of 16 x 12 x 8 heads does not fit), then the
+    loss and the gradients of the embedding and of the first and last layers' parameters for two of
+    the sequences, under the bf16 rule."""
     torch.manual_seed(0)
-    model = CastleLM(num_tokens=VOCAB, dim=512, depth=12, heads=8, dim_head=64, use_triton=True,
+    depth = 12
+    model = CastleLM(num_tokens=VOCAB, dim=512, depth=depth, heads=8, dim_head=64, use_triton=True,
                      tie_embedding=True).cuda().bfloat16()
-    x = tokens(16, 1025).cuda()
-    loss = model(x, return_loss=True)
+    x = tokens(16, 1025)
+    loss = model(x.cuda(), return_loss=True)
     loss.backward()
     assert math.isfinite(loss.item())
     for name, param in model.named_parameters():
-        assert param.grad is not None and torch.isfinite(param.grad).all(), name
+        if param.requires_grad:
+            assert param.grad is not None and torch.isfinite(param.grad).all(), name
+    torch.set_num_threads(16)
+    weights = {k: v.detach().float().cpu() for k, v in model.state_dict().items()}
+    with torch.no_grad():
+        ref_loss = sum(O.lm_forward(x[b:b + 4], weights, 8, depth, return_loss=True).item() for b in range(0, 16, 4)) / 4
+    assert abs(loss.item() - ref_loss) <= 2e-2 * abs(ref_loss)
+
+    model.zero_grad()
+    sub = x[:2]
+    loss2 = model(sub.cuda(), return_loss=True)
+    loss2.backward()
+    leaves = {k: v.clone().requires_grad_(not k.endswith("freqs")) for k, v in weights.items()}
+    leaves["to_logits.weight"] = leaves["token_emb.weight"]          # tied
+    ref2 = O.lm_forward(sub, leaves, 8, depth, return_loss=True)
+    ref2.backward()
+    assert abs(loss2.item() - ref2.item()) <= 2e-2 * abs(ref2.item())
+    grads = dict(model.named_parameters())
+    checked = ["token_emb.weight"] + [n for n in grads if n.startswith(("layers.0.", "layers.11.")) and not n.endswith("freqs")]
+    for name in checked:
+        got, want = grads[name].grad.float().cpu(), leaves[name].grad
+        rel = ((got - want).norm() / want.norm()).item()
+        assert rel <= 2e-2, f"{name}: relative norm error {rel:.3e}"
