@@ -48,12 +48,30 @@ class Cache(_CacheFields):
 class _CacheStore:
     """Capacity buffers behind a native cache: four (B, H, capacity, d) tensors and a row count."""
 
-    def __init__(self, B, H, d, capacity, dtype, device):
-        self.buffers = tuple(torch.empty((B, H, capacity, d), dtype=dtype, device=device) for _ in range(4))
+    def __init__(self, B, H, d, capacity, dtype, device, U_buffer=None):
+        # U_buffer: an existing (B, H, capacity, d) tensor to adopt as the lookahead-key buffer
+        first = U_buffer if U_buffer is not None else torch.empty((B, H, capacity, d), dtype=dtype, device=device)
+        self.buffers = (first,) + tuple(torch.empty((B, H, capacity, d), dtype=dtype, device=device) for _ in range(3))
         self.capacity = capacity
         self.length = 0
-        self.workspace = ops.decode_workspace(B, H, d, device)
-        self.views = tuple(_native.view4(buf) for buf in self.buffers)   # reused by every step on these buffers
+        self._geometry = (B, H, d, device)
+        self._workspace = None
+        self._views = None
+
+    @property
+    def workspace(self):
+        """Partial-result workspace of the decode kernels, allocated when the first step needs it."""
+        if self._workspace is None:
+            B, H, d, device = self._geometry
+            self._workspace = ops.decode_workspace(B, H, d, device)
+        return self._workspace
+
+    @property
+    def views(self):
+        """castle_view4 of the four buffers, built once and reused by every step on them."""
+        if self._views is None:
+            self._views = tuple(_native.view4(buf) for buf in self.buffers)
+        return self._views
 
     def as_cache(self) -> Cache:
         n = self.length
@@ -165,15 +183,13 @@ class Castle(nn.Module):
     def _parallel_native(self, proj, want_cache):
         B, n, _ = proj.shape
         H, d = self.heads, self.dim_head
-        store = None
-        if want_cache:
-            store = _CacheStore(B, H, d, _reserve_rows(n), proj.dtype, proj.device)
-        U_view = store.buffers[0][:, :, :n] if want_cache else None
-        res = ops.castle_attention_packed(proj, H, self.scale, want_cache, U_view, rotary=self.use_rotary)
-        merged = res[0] if want_cache else res
-        qu, _, _, _, kc, vc = self._split(proj)
         if not want_cache:
-            return merged, None
+            return ops.castle_attention_packed(proj, H, self.scale, rotary=self.use_rotary), None
+        capacity = _reserve_rows(n)
+        # the kernels write the lookahead keys straight into what becomes the cache's U buffer
+        merged, U = ops.castle_attention_packed(proj, H, self.scale, True, capacity, rotary=self.use_rotary)
+        store = _CacheStore(B, H, d, capacity, proj.dtype, proj.device, U_buffer=U._base.detach())
+        qu, _, _, _, kc, vc = self._split(proj)
         with torch.no_grad():
             if self.use_rotary:   # the cache holds the rotated qu / kc rows
                 ops.castle_rope_hip(qu, store.buffers[1][:, :, :n])

@@ -1642,7 +1642,7 @@ template <typename T, typename TI, int HD> static int launch_bwd_t(const BwdArgs
   {
     ProfScope ps(kSlotDelta, stream);
     if constexpr (sizeof(T) == 2)
-      hipLaunchKernelGGL((amax_kernel<TI, HD>), dim3(kAmaxBlocks), dim3(kThreads), 0, stream, a.dout, a.s.H, a.s.L,
+      hipLaunchKernelGGL((amax_kernel<TI, HD>), dim3(kAmaxBlocks), dim3(kAmaxThreads), 0, stream, a.dout, a.s.H, a.s.L,
                          (int64_t)BH * a.s.L, a.amax_part, (int*)nullptr);
     hipLaunchKernelGGL((delta_kernel<T, TI, HD>), dim3((a.s.Lp + RPB - 1) / RPB, BH), block, 0, stream, a);
   }

@@ -492,7 +492,7 @@ template <typename T, typename TI, int HD> static int launch_fwd_t(const FwdArgs
     ProfScope ps(kSlotTqv, stream);
     constexpr int PIECES_PER_ROW = HD / elem_traits<T>::vec16;
     if constexpr (sizeof(T) == 2)
-      hipLaunchKernelGGL((amax_kernel<TI, HD>), dim3(kAmaxBlocks), dim3(kThreads), 0, stream, a.vu, a.s.H, a.s.L,
+      hipLaunchKernelGGL((amax_kernel<TI, HD>), dim3(kAmaxBlocks), dim3(kAmaxThreads), 0, stream, a.vu, a.s.H, a.s.L,
                          (int64_t)BH * a.s.L, a.ws.amax_part, &a.ws.hdr->status);
     hipLaunchKernelGGL((prep_kernel<T, TI, HD>), dim3((a.s.Lp * PIECES_PER_ROW + kThreads - 1) / kThreads, BH, 6), dim3(kThreads), 0, stream, a);
     hipLaunchKernelGGL((tqv_kernel<T, TI, HD>), dim3(a.s.nblk, BH), dim3(kThreads), 0, stream, a);

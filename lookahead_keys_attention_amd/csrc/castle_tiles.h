@@ -566,30 +566,45 @@ __device__ __forceinline__ vec<float, 2> rope_rot(float x0, float x1, float pos,
 // ---- range control ------------------------------------------------------------------------
 // Partial maxima of |x| over a (B, H, L, HD) view: kAmaxBlocks workgroups, one partial each.  The
 // consumers reduce the partials themselves (amax_from_partials), so no atomics and no clearing.
+constexpr int kAmaxThreads = 1024;
 template <typename TI, int HD>
-__global__ __launch_bounds__(kThreads) void amax_kernel(View4 x, int H, int L, int64_t rows, float* part, int* status) {
+__global__ __launch_bounds__(kAmaxThreads) void amax_kernel(View4 x, int H, int L, int64_t rows, float* part, int* status) {
   constexpr int V = elem_traits<TI>::vec16;
   constexpr int VPR = HD / V;
+  constexpr int UN = 4;   // independent loads in flight per thread
   if (status != nullptr && blockIdx.x == 0 && threadIdx.x == 0) *status = 0;
   float m = 0.f;
   const int64_t pieces = rows * VPR;
-  for (int64_t p = (int64_t)blockIdx.x * kThreads + threadIdx.x; p < pieces; p += (int64_t)gridDim.x * kThreads) {
-    const int64_t row = p / VPR;
-    const int cv = (int)(p % VPR);
-    const int64_t bh = row / L, l = row % L;
-    const TI* src = reinterpret_cast<const TI*>(x.ptr) + (bh / H) * x.sb + (bh % H) * x.sh + l * x.sl + cv * V;
-    const vec<float, V> f = __builtin_convertvector(*reinterpret_cast<const vec<TI, V>*>(src), vec<float, V>);
+  const int64_t stride = (int64_t)gridDim.x * kAmaxThreads;
+  for (int64_t p0 = (int64_t)blockIdx.x * kAmaxThreads + threadIdx.x; p0 < pieces; p0 += UN * stride) {
+    vec<TI, V> v[UN];
 #pragma unroll
-    for (int e = 0; e < V; ++e) m = fmaxf(m, fabsf(f[e]));   // fmaxf drops NaNs
+    for (int u = 0; u < UN; ++u) {
+      const int64_t p = p0 + u * stride;
+#pragma unroll
+      for (int e = 0; e < V; ++e) v[u][e] = (TI)0.f;
+      if (p < pieces) {
+        const int64_t row = p / VPR;
+        const int cv = (int)(p % VPR);
+        const int64_t bh = row / L, l = row % L;
+        v[u] = *reinterpret_cast<const vec<TI, V>*>(reinterpret_cast<const TI*>(x.ptr) + (bh / H) * x.sb + (bh % H) * x.sh + l * x.sl + cv * V);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const vec<float, V> f = __builtin_convertvector(v[u], vec<float, V>);
+#pragma unroll
+      for (int e = 0; e < V; ++e) m = fmaxf(m, fabsf(f[e]));   // fmaxf drops NaNs
+    }
   }
 #pragma unroll
   for (int o = 1; o < 64; o <<= 1) m = fmaxf(m, __shfl_xor(m, o));
-  __shared__ float s_m[kThreads / 64];
+  __shared__ float s_m[kAmaxThreads / 64];
   if ((threadIdx.x & 63) == 0) s_m[threadIdx.x >> 6] = m;
   __syncthreads();
   if (threadIdx.x == 0) {
 #pragma unroll
-    for (int w = 1; w < kThreads / 64; ++w) m = fmaxf(m, s_m[w]);
+    for (int w = 1; w < kAmaxThreads / 64; ++w) m = fmaxf(m, s_m[w]);
     part[blockIdx.x] = fminf(m, 3.0e38f);   // an infinite input counts as the largest finite value
   }
 }

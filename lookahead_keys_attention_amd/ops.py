@@ -12,6 +12,10 @@ the kernels read the six operands through strides, write the output already merg
 
 `castle_decode_step_hip` is the cached single-token step (lookahead_keys_attention.py:166-203)
 over preallocated capacity buffers, updated in place.
+
+The parallel operators are registered with torch.library (torch.ops.castle_hip.attention,
+.attention_packed and their backward passes) with fake implementations and autograd formulas, so
+they trace under FakeTensorMode / torch.compile; the functions above are thin callers of them.
 """
 from __future__ import annotations
 
@@ -86,90 +90,172 @@ def _as_readable(t: torch.Tensor) -> torch.Tensor:
     return t if N.vector_ok(t) else t.contiguous()
 
 
-class _CastleAttention(torch.autograd.Function):
-    """Six separate operands (the reference operator's signature)."""
-
-    @staticmethod
-    def forward(ctx, q, k, v, qu, ku, vu, scale, want_U, rotary=False):
-        _require_gpu(q, "castle_attention_hip")
-        B, H, L, d = q.shape
-        _check_dims(d, q.dtype)
-        ops = [_as_readable(t) for t in (q, k, v, qu, ku, vu)]
-        out = torch.empty((B, L, H, d), dtype=q.dtype, device=q.device).permute(0, 2, 1, 3)
-        U = torch.empty((B, H, L, d), dtype=q.dtype, device=q.device) if want_U else None
-        ctx.flags = DEFAULT_FLAGS | (N.FLAG_ROTARY if rotary else 0)
-        ws = _fwd_raw(*ops, scale, out, U, ctx.flags)
-        ctx.save_for_backward(*ops, out, ws)
-        ctx.scale = scale
-        if want_U:
-            ctx.mark_non_differentiable(U)
-            return out, U
-        return out
-
-    @staticmethod
-    def backward(ctx, dout, dU=None):
-        *ops, out, ws = ctx.saved_tensors
-        B, H, L, d = ops[0].shape
-        dout = _as_readable(dout)
-        packed = torch.empty((6, B, H, L, d), dtype=out.dtype, device=out.device)
-        grads = list(packed.unbind(0))
-        _bwd_raw(*ops, out, dout, ctx.scale, grads, ws, ctx.flags)
-        return (*grads, None, None, None)
+# ---------------------------------------------------------------------------------------------
+# Registered operators (torch.library): the kernels are reachable as torch.ops.castle_hip.*, with
+# fake (meta) implementations for shape propagation / tracing and autograd formulas that call the
+# backward entry point.  The Python functions below them are what callers use.
+#
+#   castle_hip::attention         six (B,H,L,d) operands -> (out, U, workspace)
+#   castle_hip::attention_packed  (B,L,6*H*d) projection -> (merged out, workspace); U written into
+#                                 the optional (B,H,L,d) view `U_out` (a cache buffer)
+#   castle_hip::attention_bwd / attention_packed_bwd   their backward passes
+# `U` is an empty tensor when the lookahead keys are not asked for.  The workspace output is what
+# the backward pass needs back (operand copies, snapshots, log-sum-exp); it carries no gradient.
+def _out_like(q):
+    B, H, L, d = q.shape
+    return torch.empty((B, L, H, d), dtype=q.dtype, device=q.device).permute(0, 2, 1, 3)
 
 
-class _CastleAttentionPacked(torch.autograd.Function):
-    """Fused-projection layout in, merged heads out."""
+def _fwd_ws_bytes(B, H, L, d, dtype):
+    return N.check(N.lib().castle_fwd_workspace_bytes(int(B), int(H), int(L), int(d), N.dtype_code(dtype)),
+                   "castle_fwd_workspace_bytes")
 
-    @staticmethod
-    def forward(ctx, proj, heads, scale, U_out, rotary=False):
-        # U_out: None, or a (B,H,L,d) view without gradient history that receives the lookahead keys
-        _require_gpu(proj, "castle_attention_packed")
-        B, L, width = proj.shape
-        d = width // (6 * heads)
-        _check_dims(d, proj.dtype)
-        proj = proj if (proj.is_contiguous() and proj.data_ptr() % 16 == 0) else proj.contiguous()
-        six = proj.view(B, L, 6, heads, d).permute(2, 0, 3, 1, 4)      # (6, B, H, L, d) views
-        qu, ku, vu, qc, kc, vc = six.unbind(0)
-        merged = torch.empty((B, L, heads * d), dtype=proj.dtype, device=proj.device)
-        out = merged.view(B, L, heads, d).permute(0, 2, 1, 3)
-        ctx.flags = DEFAULT_FLAGS | (N.FLAG_ROTARY if rotary else 0)
-        ws = _fwd_raw(qc, kc, vc, qu, ku, vu, scale, out, U_out, ctx.flags)
-        ctx.save_for_backward(proj, merged, ws)
-        ctx.heads, ctx.scale = heads, scale
-        return merged
 
-    @staticmethod
-    def backward(ctx, dmerged):
-        proj, merged, ws = ctx.saved_tensors
-        heads, scale = ctx.heads, ctx.scale
-        B, L, width = proj.shape
-        d = width // (6 * heads)
-        six = proj.view(B, L, 6, heads, d).permute(2, 0, 3, 1, 4)
-        qu, ku, vu, qc, kc, vc = six.unbind(0)
-        out = merged.view(B, L, heads, d).permute(0, 2, 1, 3)
-        dmerged = dmerged if (dmerged.is_contiguous() and dmerged.data_ptr() % 16 == 0) else dmerged.contiguous()
-        dout = dmerged.view(B, L, heads, d).permute(0, 2, 1, 3)
-        dproj = torch.empty_like(proj)
-        dqu, dku, dvu, dqc, dkc, dvc = dproj.view(B, L, 6, heads, d).permute(2, 0, 3, 1, 4).unbind(0)
-        _bwd_raw(qc, kc, vc, qu, ku, vu, out, dout, scale, (dqc, dkc, dvc, dqu, dku, dvu), ws, ctx.flags)
-        return dproj, None, None, None, None
+@torch.library.custom_op("castle_hip::attention", mutates_args=())
+def _attention_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, qu: torch.Tensor, ku: torch.Tensor,
+                  vu: torch.Tensor, scale: float, want_U: bool, flags: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    _require_gpu(q, "castle_attention_hip")
+    B, H, L, d = q.shape
+    _check_dims(d, q.dtype)
+    ops = [_as_readable(t) for t in (q, k, v, qu, ku, vu)]
+    out = _out_like(q)
+    U = torch.empty((B, H, L, d) if want_U else (0,), dtype=q.dtype, device=q.device)
+    ws = _fwd_raw(*ops, scale, out, U if want_U else None, flags)
+    return out, U, ws
+
+
+@_attention_op.register_fake
+def _(q, k, v, qu, ku, vu, scale, want_U, flags):
+    B, H, L, d = q.shape
+    _check_dims(d, q.dtype)
+    U = torch.empty((B, H, L, d) if want_U else (0,), dtype=q.dtype, device=q.device)
+    ws = torch.empty(_fwd_ws_bytes(B, H, L, d, q.dtype), dtype=torch.uint8, device=q.device)
+    return _out_like(q), U, ws
+
+
+@torch.library.custom_op("castle_hip::attention_bwd", mutates_args=())
+def _attention_bwd_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, qu: torch.Tensor, ku: torch.Tensor,
+                      vu: torch.Tensor, out: torch.Tensor, dout: torch.Tensor, ws: torch.Tensor,
+                      scale: float, flags: int) -> torch.Tensor:
+    B, H, L, d = q.shape
+    ops = [_as_readable(t) for t in (q, k, v, qu, ku, vu)]
+    packed = torch.empty((6, B, H, L, d), dtype=out.dtype, device=out.device)
+    _bwd_raw(*ops, _as_readable(out), _as_readable(dout), scale, list(packed.unbind(0)), ws, flags)
+    return packed
+
+
+@_attention_bwd_op.register_fake
+def _(q, k, v, qu, ku, vu, out, dout, ws, scale, flags):
+    return torch.empty((6, *q.shape), dtype=out.dtype, device=out.device)
+
+
+def _attention_setup(ctx, inputs, output):
+    q, k, v, qu, ku, vu, scale, want_U, flags = inputs
+    out, U, ws = output
+    ctx.save_for_backward(q, k, v, qu, ku, vu, out, ws)
+    ctx.scale, ctx.flags = scale, flags
+    ctx.mark_non_differentiable(U, ws)   # U carries no gradient (lookahead_keys_attention_triton.py:513-515)
+
+
+def _attention_backward(ctx, dout, dU, dws):
+    q, k, v, qu, ku, vu, out, ws = ctx.saved_tensors
+    grads = torch.ops.castle_hip.attention_bwd(q, k, v, qu, ku, vu, out, dout, ws, ctx.scale, ctx.flags)
+    return (*grads.unbind(0), None, None, None)
+
+
+_attention_op.register_autograd(_attention_backward, setup_context=_attention_setup)
+
+
+def _six_views(proj, heads):
+    B, L, width = proj.shape
+    d = width // (6 * heads)
+    six = proj.view(B, L, 6, heads, d).permute(2, 0, 3, 1, 4)      # (6, B, H, L, d) views
+    return six.unbind(0)                                            # qu, ku, vu, qc, kc, vc
+
+
+def _packed_ok(t):
+    return t if (t.is_contiguous() and t.data_ptr() % 16 == 0) else t.contiguous()
+
+
+@torch.library.custom_op("castle_hip::attention_packed", mutates_args=())
+def _attention_packed_op(proj: torch.Tensor, heads: int, scale: float, want_U: bool, row_capacity: int,
+                         flags: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    # The lookahead keys come back as the first L rows of a (B, H, row_capacity, d) buffer, so that a
+    # caller can hand over the U buffer of a decode cache without copying (row_capacity >= L).
+    _require_gpu(proj, "castle_attention_packed")
+    B, L, width = proj.shape
+    d = width // (6 * heads)
+    _check_dims(d, proj.dtype)
+    qu, ku, vu, qc, kc, vc = _six_views(_packed_ok(proj), heads)
+    merged = torch.empty((B, L, heads * d), dtype=proj.dtype, device=proj.device)
+    out = merged.view(B, L, heads, d).permute(0, 2, 1, 3)
+    U = torch.empty((B, heads, max(row_capacity, L), d) if want_U else (0,), dtype=proj.dtype, device=proj.device)
+    ws = _fwd_raw(qc, kc, vc, qu, ku, vu, scale, out, U[:, :, :L] if want_U else None, flags)
+    return merged, U, ws
+
+
+@_attention_packed_op.register_fake
+def _(proj, heads, scale, want_U, row_capacity, flags):
+    B, L, width = proj.shape
+    d = width // (6 * heads)
+    _check_dims(d, proj.dtype)
+    ws = torch.empty(_fwd_ws_bytes(B, heads, L, d, proj.dtype), dtype=torch.uint8, device=proj.device)
+    U = torch.empty((B, heads, max(row_capacity, L), d) if want_U else (0,), dtype=proj.dtype, device=proj.device)
+    return torch.empty((B, L, heads * d), dtype=proj.dtype, device=proj.device), U, ws
+
+
+@torch.library.custom_op("castle_hip::attention_packed_bwd", mutates_args=())
+def _attention_packed_bwd_op(proj: torch.Tensor, merged: torch.Tensor, dmerged: torch.Tensor, ws: torch.Tensor,
+                             heads: int, scale: float, flags: int) -> torch.Tensor:
+    B, L, width = proj.shape
+    d = width // (6 * heads)
+    qu, ku, vu, qc, kc, vc = _six_views(_packed_ok(proj), heads)
+    out = merged.view(B, L, heads, d).permute(0, 2, 1, 3)
+    dout = _packed_ok(dmerged).view(B, L, heads, d).permute(0, 2, 1, 3)
+    dproj = torch.empty((B, L, width), dtype=proj.dtype, device=proj.device)
+    dqu, dku, dvu, dqc, dkc, dvc = _six_views(dproj, heads)
+    _bwd_raw(qc, kc, vc, qu, ku, vu, out, dout, scale, (dqc, dkc, dvc, dqu, dku, dvu), ws, flags)
+    return dproj
+
+
+@_attention_packed_bwd_op.register_fake
+def _(proj, merged, dmerged, ws, heads, scale, flags):
+    return torch.empty(proj.shape, dtype=proj.dtype, device=proj.device)
+
+
+def _packed_setup(ctx, inputs, output):
+    proj, heads, scale, want_U, row_capacity, flags = inputs
+    merged, U, ws = output
+    ctx.save_for_backward(proj, merged, ws)
+    ctx.heads, ctx.scale, ctx.flags = heads, scale, flags
+    ctx.mark_non_differentiable(U, ws)
+
+
+def _packed_backward(ctx, dmerged, dU, dws):
+    proj, merged, ws = ctx.saved_tensors
+    dproj = torch.ops.castle_hip.attention_packed_bwd(proj, merged, dmerged, ws, ctx.heads, ctx.scale, ctx.flags)
+    return dproj, None, None, None, None, None
+
+
+_attention_packed_op.register_autograd(_packed_backward, setup_context=_packed_setup)
 
 
 def castle_attention_hip(q, k, v, qu, ku, vu, scale, return_U_for_cache=False, rotary=False):
     """Drop-in for castle_attention_triton: returns out, or (out, U).  rotary=True applies the
     rotary position embedding (positions 0..L-1) to q, k, qu, ku, vu inside the kernels."""
-    return _CastleAttention.apply(q, k, v, qu, ku, vu, float(scale), bool(return_U_for_cache), bool(rotary))
+    flags = DEFAULT_FLAGS | (N.FLAG_ROTARY if rotary else 0)
+    out, U, _ = torch.ops.castle_hip.attention(q, k, v, qu, ku, vu, float(scale), bool(return_U_for_cache), int(flags))
+    return (out, U) if return_U_for_cache else out
 
 
-def castle_attention_packed(proj, heads, scale, return_U_for_cache=False, U_out=None, rotary=False):
-    """proj (B, L, 6*H*d) -> merged out (B, L, H*d), or (out, U (B,H,L,d)).  `U_out`, if given,
-    is the (B,H,L,d) view (any row stride) the lookahead keys are written into."""
-    if not return_U_for_cache:
-        return _CastleAttentionPacked.apply(proj, int(heads), float(scale), None, bool(rotary))
-    if U_out is None:
-        B, L, width = proj.shape
-        U_out = torch.empty((B, heads, L, width // (6 * heads)), dtype=proj.dtype, device=proj.device)
-    return _CastleAttentionPacked.apply(proj, int(heads), float(scale), U_out, bool(rotary)), U_out
+def castle_attention_packed(proj, heads, scale, return_U_for_cache=False, row_capacity=0, rotary=False):
+    """proj (B, L, 6*H*d) -> merged out (B, L, H*d), or (out, U).  U is (B,H,L,d); with
+    `row_capacity` > L it is the first L rows of a freshly allocated (B,H,row_capacity,d) buffer
+    (reachable as U._base), which a decode cache can adopt as its U buffer without a copy."""
+    flags = DEFAULT_FLAGS | (N.FLAG_ROTARY if rotary else 0)
+    merged, U, _ = torch.ops.castle_hip.attention_packed(proj, int(heads), float(scale), bool(return_U_for_cache),
+                                                         int(row_capacity), int(flags))
+    return (merged, U[:, :, : proj.shape[1]]) if return_U_for_cache else merged
 
 
 def decode_workspace(B, H, d, device):
