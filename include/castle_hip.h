@@ -168,6 +168,15 @@ int castle_decode_step_static(const castle_view4* U, const castle_view4* qu_cach
 int castle_rope(const castle_view4* x, const castle_view4* out, int B, int H, int L, int d, int dtype,
                 int first_position, void* stream);
 
+/* y[M, N] = x[M, K] w[N, K]^T, all three row-major in the 16-bit element type `dtype` (leading
+ * dimensions ldx, ldw, ldy in elements; fp32 accumulation), for the few rows of a decode step: the
+ * fused projection and the output projection around the cached step, which the reference runs as
+ * nn.Linear on a (B, 1, dim) tensor (lookahead_keys_attention.py:99 and :209 with seq_len == 1).
+ * Meant for M up to a few dozen rows (one workgroup per 32 x 32 output tile, K split over its
+ * waves); any M works.  K % 8 == 0, N % 2 == 0, x / w 16-byte aligned with ldx, ldw % 8 == 0. */
+int castle_small_linear(const void* x, const void* w, void* y, int M, int N, int K,
+                        int64_t ldx, int64_t ldw, int64_t ldy, int dtype, void* stream);
+
 /* Per-kernel timing (no counterpart in the reference; for benchmarks).  While enabled, every
  * kernel launched by the entry points above is bracketed by a HIP event pair on its stream.
  * castle_profile_enable(on) also discards pending records.  castle_profile_read waits for the

@@ -162,22 +162,32 @@ class Castle(nn.Module):
         single = n == 1
         if return_next_cache is None:
             return_next_cache = single
-        proj = self.to_all_qkv(self.norm(x))
         native = self.use_triton
         if native and not x.is_cuda:
             if self._explicit_native:
                 raise RuntimeError("Castle(use_triton=True) runs HIP kernels and needs GPU tensors; "
                                    "construct with use_triton=False for the PyTorch formulation")
             native = False   # auto-selected kernels, CPU tensors: the dense formulation (lookahead_keys_attention.py:120)
+        if single and native and torch.is_grad_enabled() and (
+                x.requires_grad or any(p.requires_grad for p in self.parameters())):
+            native = False   # the native step records no autograd graph; the dense step does
+        native_step = single and native
+        proj = self._project(self.to_all_qkv, self.norm(x), native_step)
         if not single:
             assert cache is None, "must be inferencing single tokens if receiving cache"
             merged, next_cache = (self._parallel_native if native else self._parallel_dense)(proj, return_next_cache)
         else:
-            if native and torch.is_grad_enabled() and proj.requires_grad:
-                native = False   # the native step records no autograd graph; the dense step does
             merged, next_cache = (self._step_native if native else self._step_dense)(proj, cache)
-        y = self.combine_heads(merged)
+        y = self._project(self.combine_heads, merged, native_step)
         return (y, next_cache) if return_next_cache else y
+
+    @staticmethod
+    def _project(layer, t, native_step):
+        """The bias-free projections; on the native single-token step the few rows go through the
+        library's own small-M kernel instead of a general GEMM (inference only)."""
+        if native_step and ops.small_linear_ok(t, layer.weight):
+            return ops.small_linear(t, layer.weight)
+        return layer(t)
 
     # -- native HIP paths ---------------------------------------------------
     def _parallel_native(self, proj, want_cache):
@@ -237,11 +247,11 @@ class Castle(nn.Module):
         object is built, `store.length` is left alone: the owner of the graph keeps the count).
         x: (B, 1, dim); store: the `_CacheStore` behind a native cache.  Returns (B, 1, dim)."""
         B = x.shape[0]
-        proj = self.to_all_qkv(self.norm(x))
+        proj = self._project(self.to_all_qkv, self.norm(x), True)
         out = torch.empty((B, 1, self.heads, self.dim_head), dtype=proj.dtype, device=proj.device)
         ops.castle_decode_step_packed(store.views, store.capacity, 0, proj, self.heads, self.scale, out,
                                       store.workspace, rotary=self.use_rotary, t_device=t_device)
-        return self.combine_heads(out.view(B, 1, self.heads * self.dim_head))
+        return self._project(self.combine_heads, out.view(B, 1, self.heads * self.dim_head), True)
 
     # -- dense PyTorch formulation (use_triton=False) -------------------------
     def _parallel_dense(self, proj, want_cache):

@@ -16,6 +16,8 @@ int launch_decode(const DecodeArgs& a, int dtype, hipStream_t stream);
 int launch_rope(const View4& src, const View4& dst, int B, int H, int L, int d, int dtype, int pos0, hipStream_t stream);
 int decode_pick_splits(int BH, int t);
 int decode_static_scratch(float** ptr);
+int launch_small_linear(const void* x, const void* w, void* y, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldy,
+                        int dtype, hipStream_t stream);
 }  // namespace castle
 
 namespace {
@@ -324,6 +326,17 @@ int castle_rope(const castle_view4* x, const castle_view4* out, int B, int H, in
   if (B <= 0 || H <= 0 || L <= 0 || first_position < 0 || !head_dim_ok(d) || (int64_t)B * H > 65535) return CASTLE_ERR_SHAPE;
   if (!view_ok(x, es, true) || !view_ok(out, es, true)) return CASTLE_ERR_ARG;
   return castle::launch_rope(to_view(x), to_view(out), B, H, L, d, dtype, first_position, static_cast<hipStream_t>(stream));
+}
+
+int castle_small_linear(const void* x, const void* w, void* y, int M, int N, int K,
+                        int64_t ldx, int64_t ldw, int64_t ldy, int dtype, void* stream) {
+  if (dtype != CASTLE_BF16 && dtype != CASTLE_F16) return CASTLE_ERR_DTYPE;
+  if (M <= 0 || N <= 0 || K <= 0 || K % 8 != 0 || N % 2 != 0) return CASTLE_ERR_SHAPE;
+  if (x == nullptr || w == nullptr || y == nullptr) return CASTLE_ERR_ARG;
+  if (reinterpret_cast<uintptr_t>(x) % 16 != 0 || reinterpret_cast<uintptr_t>(w) % 16 != 0 ||
+      reinterpret_cast<uintptr_t>(y) % 4 != 0 || ldx % 8 != 0 || ldw % 8 != 0 || ldy % 2 != 0)
+    return CASTLE_ERR_ARG;
+  return castle::launch_small_linear(x, w, y, M, N, K, ldx, ldw, ldy, dtype, static_cast<hipStream_t>(stream));
 }
 
 int castle_profile_enable(int on) { return castle::profile_enable(on); }

@@ -295,6 +295,74 @@ int launch_rope(const View4& src, const View4& dst, int B, int H, int L, int d, 
 }
 
 // ---------------------------------------------------------------------------
+// y[M, N] = x[M, K] w[N, K]^T for the few rows of a decode step (M = batch): the two projections
+// around the cached step (lookahead_keys_attention.py:99, 209 with seq_len == 1).  A library GEMM
+// spends most of its ~8 us here on one 32-row tile per workgroup walking K serially; this kernel
+// gives every 32 x 32 output tile to one workgroup of 8 waves that split K, so each wave issues all
+// its operand loads at once (straight from global memory, rows of x and w are K-contiguous, which is
+// the MFMA operand layout), runs a handful of MFMAs and the partial tiles are summed through LDS.
+constexpr int kLinWaves = 8;
+template <typename T>
+__global__ __launch_bounds__(64 * kLinWaves) void small_linear_kernel(const T* x, const T* w, T* y, int M, int N, int K,
+                                                                       int64_t ldx, int64_t ldw, int64_t ldy) {
+  static_assert(sizeof(T) == 2, "16-bit operands");
+  constexpr int MAXS = 8;   // 16-deep steps a wave handles per pass
+  __shared__ float red[kLinWaves][32][33];
+  const int lane = lane_id(), wave = wave_id(), c = lane & 31, g = lane >> 5;
+  const int n0 = blockIdx.x * 32, m0 = blockIdx.y * 32;
+  const int steps = (K + 15) / 16;
+  const int per = (steps + kLinWaves - 1) / kLinWaves;
+  const bool row_ok = m0 + c < M, col_ok = n0 + c < N;
+  const T* xr = x + (int64_t)(m0 + c) * ldx;
+  const T* wr = w + (int64_t)(n0 + c) * ldw;
+  acc_t acc;
+  zero(acc);
+  for (int s0 = wave * per; s0 < min(steps, (wave + 1) * per); s0 += MAXS) {
+    frag<T> fa[MAXS], fb[MAXS];
+#pragma unroll
+    for (int u = 0; u < MAXS; ++u) {
+      const int kk = 16 * (s0 + u) + 8 * g;
+      const bool in = s0 + u < min(steps, (wave + 1) * per) && kk < K;   // K is a multiple of 8
+      fa[u] = (in && row_ok) ? *reinterpret_cast<const frag_mem<T>*>(xr + kk) : zero_frag<T>();
+      fb[u] = (in && col_ok) ? *reinterpret_cast<const frag_mem<T>*>(wr + kk) : zero_frag<T>();
+    }
+#pragma unroll
+    for (int u = 0; u < MAXS; ++u) mma(acc, fa[u], fb[u]);
+  }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) red[wave][acc_row(r, g)][c] = acc[r];
+  __syncthreads();
+  // 1024 outputs, 512 threads: two neighbouring columns each
+  const int e = 2 * threadIdx.x, row = e / 32, col = e % 32;
+  float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+  for (int v = 0; v < kLinWaves; ++v) { s0 += red[v][row][col]; s1 += red[v][row][col + 1]; }
+  if (m0 + row < M) {
+    T* dst = y + (int64_t)(m0 + row) * ldy + n0 + col;
+    if (n0 + col + 1 < N) {
+      vec<T, 2> o = {(T)s0, (T)s1};
+      *reinterpret_cast<vec<T, 2>*>(dst) = o;
+    } else if (n0 + col < N) {
+      dst[0] = (T)s0;
+    }
+  }
+}
+
+int launch_small_linear(const void* x, const void* w, void* y, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldy,
+                        int dtype, hipStream_t stream) {
+  const dim3 grid((N + 31) / 32, (M + 31) / 32), block(64 * kLinWaves);
+  if (dtype == 1)
+    hipLaunchKernelGGL((small_linear_kernel<bf16_t>), grid, block, 0, stream, static_cast<const bf16_t*>(x),
+                       static_cast<const bf16_t*>(w), static_cast<bf16_t*>(y), M, N, K, ldx, ldw, ldy);
+  else if (dtype == 2)
+    hipLaunchKernelGGL((small_linear_kernel<fp16_t>), grid, block, 0, stream, static_cast<const fp16_t*>(x),
+                       static_cast<const fp16_t*>(w), static_cast<fp16_t*>(y), M, N, K, ldx, ldw, ldy);
+  else
+    return -1;
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+// ---------------------------------------------------------------------------
 // Partial-result buffer of the entry point that allocates nothing: one array per GPU, part of the
 // loaded code object, alive until the process ends.  Host code never uses the array's name as an
 // address (on the host it is only a stand-in for the symbol): the device address is looked up

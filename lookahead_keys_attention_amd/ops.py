@@ -287,6 +287,32 @@ def castle_decode_step_hip(U, qu_cache, kc_cache, vc_cache, t, qc, kc, vc, qu, k
     return out
 
 
+SMALL_LINEAR_MAX_ROWS = 64
+
+
+def small_linear_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    """True if `small_linear` can replace F.linear(x, weight) for this call: a few rows, 16-bit GPU
+    tensors, K-contiguous rows that the kernels can read 16 bytes at a time."""
+    return (x.is_cuda and x.dtype in (torch.bfloat16, torch.float16) and weight.dtype == x.dtype
+            and x.dim() == 3 and x.shape[1] == 1 and x.shape[0] <= SMALL_LINEAR_MAX_ROWS
+            and x.stride(2) == 1 and weight.stride(1) == 1 and x.shape[2] % 8 == 0 and weight.shape[0] % 2 == 0
+            and x.stride(0) % 8 == 0 and weight.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
+
+
+@torch.no_grad()
+def small_linear(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """(B, 1, K) x (N, K) -> (B, 1, N): the projections around the cached single-token step
+    (lookahead_keys_attention.py:99, 209 with seq_len == 1), without bias, for inference."""
+    B, _, K = x.shape
+    n = weight.shape[0]
+    y = torch.empty((B, 1, n), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = N.lib().castle_small_linear(x.data_ptr(), weight.data_ptr(), y.data_ptr(), B, n, K, x.stride(0),
+                                         weight.stride(0), n, N.dtype_code(x.dtype), N.stream_ptr(x.device))
+    N.check(rc, "castle_small_linear")
+    return y
+
+
 @torch.no_grad()
 def castle_rope_hip(x, out, first_position=0):
     """out[b,h,l,:] = R(first_position + l) x[b,h,l,:]: the rotary position embedding the kernels

@@ -343,3 +343,20 @@ def test_decode_steps(B, Hh, t0, steps, d, dtype):
         assert_close(bufs[0][:, :, :L], ref_U, dtype, "U", 1e-3)
     assert torch.equal(bufs[1][:, :, :L].cpu(), ops[3]) and torch.equal(bufs[2][:, :, :L].cpu(), ops[1])
     assert torch.equal(bufs[3][:, :, :L].cpu(), ops[2])
+
+
+@pytest.mark.parametrize("M,N,K,dtype", [(32, 3072, 512, torch.bfloat16), (32, 512, 512, torch.bfloat16), (1, 96, 32, torch.float16),
+                                         (5, 6 * 2 * 16, 40, torch.bfloat16), (64, 130, 264, torch.float16), (33, 64, 2048, torch.bfloat16)])
+def test_small_linear_matches_fp64_matmul(M, N, K, dtype):
+    """The projections around the cached step (lookahead_keys_attention.py:99, 209 with seq_len == 1):
+    y = x w^T with fp32 accumulation, against the product of the same 16-bit values in fp64; ragged
+    tiles, K not a multiple of the per-wave slices."""
+    g = torch.Generator().manual_seed(M + N + K)
+    x = torch.randn(M, 1, K, generator=g).to(dtype)
+    w = (torch.randn(N, K, generator=g) * K ** -0.5).to(dtype)
+    assert H().small_linear_ok(x.to(DEV), w.to(DEV))
+    y = H().small_linear(x.to(DEV), w.to(DEV))
+    ref = x[:, 0].double() @ w.double().t()
+    assert y.shape == (M, 1, N) and y.dtype == dtype
+    err = (y[:, 0].cpu().double() - ref).abs().max().item()
+    assert err <= 2.0 ** (-8 if dtype == torch.bfloat16 else -11) * ref.abs().max().item() * 1.01 + 1e-6   # one rounding of the result
