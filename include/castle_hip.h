@@ -46,6 +46,10 @@ extern "C" {
  * kernel to the second (2 * B * H * Lp * Lp elements of workspace); the second kernel recomputes
  * the score chain instead.  Slower, for callers short of memory. */
 #define CASTLE_FLAG_RECOMPUTE_SCORES 4
+/* castle_bwd / castle_bwd_workspace_bytes only: the forward state buffer was not kept; castle_bwd
+ * runs the forward scan again (from the operand copies in the forward workspace) into its own
+ * workspace before anything else.  What a forward call must keep for its backward is then O(L d). */
+#define CASTLE_FLAG_RECOMPUTE_STATE 8
 
 /* error codes */
 #define CASTLE_OK 0
@@ -68,11 +72,18 @@ typedef struct castle_view4 {
 int castle_abi_version(void);
 const char* castle_error_string(int code);
 
-/* Bytes of device workspace castle_fwd needs.  The forward pass leaves there what the
- * backward pass reads again (operand copies in the compute type, per-block T tiles, forward state
- * snapshots, log-sum-exp);
- * keep the buffer alive and unmodified until castle_bwd has run.  < 0 on error. */
+/* Bytes of the two device buffers castle_fwd needs.  `workspace` (castle_fwd_workspace_bytes,
+ * grows like L d): the forward pass leaves there what the backward pass reads again (a header with
+ * the range-control scalars and a status word, operand copies in the compute type, per-block T
+ * tiles, log-sum-exp); keep it alive and unmodified until castle_bwd has run.  `state`
+ * (castle_fwd_state_bytes, grows like L^2 d / 128): the snapshots of the lookahead state, scratch
+ * for a forward pass alone; castle_bwd reads them too, unless it is told to recompute them
+ * (CASTLE_FLAG_RECOMPUTE_STATE), in which case the buffer can be dropped right after castle_fwd.
+ * < 0 on error.  After the stream has finished castle_fwd, the int32 at workspace + 0 is a status
+ * word: bit 0 = an input element beyond the fp16 range was clamped (bf16 tensors, fp16 operands),
+ * bit 1 = an entry of T' = s qc.vu was. */
 int64_t castle_fwd_workspace_bytes(int B, int H, int L, int d, int dtype);
+int64_t castle_fwd_state_bytes(int B, int H, int L, int d, int dtype);
 
 /* Parallel forward.  qc,kc,vc,qu,ku,vu: (B,H,L,d), unscaled, as handed to
  * castle_attention_triton (lookahead_keys_attention.py:122).  out: (B,H,L,d) view that is
@@ -84,7 +95,7 @@ int castle_fwd(const castle_view4* qc, const castle_view4* kc, const castle_view
                const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
                int B, int H, int L, int d, int dtype, float scale, int flags,
                const castle_view4* out, const castle_view4* U,
-               void* workspace, int64_t workspace_bytes, void* stream);
+               void* workspace, int64_t workspace_bytes, void* state, int64_t state_bytes, void* stream);
 
 /* Bytes of extra device workspace castle_bwd needs: reverse state snapshots, delta, a copy of dout in
  * the compute type and, for the 16-bit element types, the dS / dSu score-gradient tiles its first
@@ -95,7 +106,8 @@ int castle_fwd(const castle_view4* qc, const castle_view4* kc, const castle_view
 int64_t castle_bwd_workspace_bytes(int B, int H, int L, int d, int dtype, int flags);
 
 /* Parallel backward.  Same operands as castle_fwd plus the forward output `out`, the
- * upstream gradient `dout` and the forward workspace as castle_fwd left it.  Writes the six
+ * upstream gradient `dout`, the forward workspace as castle_fwd left it and its state buffer
+ * (NULL with CASTLE_FLAG_RECOMPUTE_STATE).  Writes the six
  * gradients (all (B,H,L,d) views; every element is written, nothing is accumulated).
  * U carries no gradient (lookahead_keys_attention_triton.py:513-515).  d in {16,32,64}, and 128 for
  * the 16-bit element types (there every kernel runs twice, each pass keeping half of the outputs). */
@@ -106,6 +118,7 @@ int castle_bwd(const castle_view4* qc, const castle_view4* kc, const castle_view
                const castle_view4* dqc, const castle_view4* dkc, const castle_view4* dvc,
                const castle_view4* dqu, const castle_view4* dku, const castle_view4* dvu,
                const void* fwd_workspace, int64_t fwd_workspace_bytes,
+               const void* fwd_state, int64_t fwd_state_bytes,
                void* bwd_workspace, int64_t bwd_workspace_bytes, void* stream);
 
 /* Bytes of device workspace castle_decode_step needs for a cache of up to t_max rows. */

@@ -20,11 +20,13 @@ SUPPORTED_HEAD_DIMS = (16, 32, 64, 128)
 FLAG_BF16_OPERANDS = 1   # keep bf16 MFMA operands for bf16 tensors (default: fp16 operands)
 FLAG_ROTARY = 2          # rotary position embedding of qc, kc, qu, ku, vu inside the kernels
 FLAG_RECOMPUTE_SCORES = 4   # backward without the dS / dSu tile hand-over (less workspace, slower)
+FLAG_RECOMPUTE_STATE = 8    # backward re-runs the forward scan: the forward state buffer need not be kept
 
 EXPORTED_SYMBOLS = (
     "castle_abi_version",
     "castle_error_string",
     "castle_fwd_workspace_bytes",
+    "castle_fwd_state_bytes",
     "castle_fwd",
     "castle_bwd_workspace_bytes",
     "castle_bwd",
@@ -63,14 +65,16 @@ def _declare(lib):
     lib.castle_error_string.argtypes = [i]
     lib.castle_fwd_workspace_bytes.restype = i64
     lib.castle_fwd_workspace_bytes.argtypes = [i, i, i, i, i]
+    lib.castle_fwd_state_bytes.restype = i64
+    lib.castle_fwd_state_bytes.argtypes = [i, i, i, i, i]
     lib.castle_bwd_workspace_bytes.restype = i64
     lib.castle_bwd_workspace_bytes.argtypes = [i, i, i, i, i, i]
     lib.castle_decode_workspace_bytes.restype = i64
     lib.castle_decode_workspace_bytes.argtypes = [i, i, i, i]
     lib.castle_fwd.restype = i
-    lib.castle_fwd.argtypes = [_VP] * 6 + [i, i, i, i, i, f, i, _VP, _VP, vp, i64, vp]
+    lib.castle_fwd.argtypes = [_VP] * 6 + [i, i, i, i, i, f, i, _VP, _VP, vp, i64, vp, i64, vp]
     lib.castle_bwd.restype = i
-    lib.castle_bwd.argtypes = [_VP] * 8 + [i, i, i, i, i, f, i] + [_VP] * 6 + [vp, i64, vp, i64, vp]
+    lib.castle_bwd.argtypes = [_VP] * 8 + [i, i, i, i, i, f, i] + [_VP] * 6 + [vp, i64, vp, i64, vp, i64, vp]
     lib.castle_profile_enable.restype = i
     lib.castle_profile_enable.argtypes = [i]
     lib.castle_profile_read.restype = i

@@ -11,6 +11,7 @@
 
 namespace castle {
 int launch_fwd(const FwdArgs& a, int dtype, bool bf16_operands, hipStream_t stream);
+int launch_scan(const FwdArgs& a, int dtype, bool bf16_operands, hipStream_t stream);
 int launch_bwd(const BwdArgs& a, int dtype, bool bf16_operands, hipStream_t stream);
 int launch_decode(const DecodeArgs& a, int dtype, hipStream_t stream);
 int launch_rope(const View4& src, const View4& dst, int B, int H, int L, int d, int dtype, int pos0, hipStream_t stream);
@@ -54,7 +55,7 @@ int64_t max_score_tile_bytes() {
 struct Geometry {
   int Lp, nblk;
   int64_t lse_bytes, tblk_bytes, snap_bytes, mat_bytes, op_bytes;
-  int64_t off_lse, off_t, off_tt, off_ttx, off_snap, off_ops, total;
+  int64_t off_lse, off_t, off_tt, off_ttx, off_ops, total;
   int64_t bwd_total;
 };
 constexpr int64_t kHeaderBytes = 256 + 4 * castle::kAmaxBlocks;   // header + partial maxima, forward and backward alike
@@ -75,12 +76,12 @@ Geometry geometry(int B, int H, int L, int d, int es, int flags = 0) {
   g.off_t = g.off_lse + g.lse_bytes;
   g.off_tt = g.off_t + g.tblk_bytes;
   g.off_ttx = g.off_tt + g.tblk_bytes;
-  g.off_snap = g.off_ttx + g.tblk_bytes;
   g.op_bytes = align_up(BH * g.Lp * d * es, 256);   // one operand in the compute type, padded to Lp rows
-  g.off_ops = g.off_snap + g.snap_bytes;
-  g.total = g.off_ops + 6 * g.op_bytes;
-  // header, reverse-state snapshots, delta, dO copy, dS / dSu tiles
-  g.bwd_total = kHeaderBytes + g.snap_bytes + g.lse_bytes + g.op_bytes + 2 * g.mat_bytes;
+  g.off_ops = g.off_ttx + g.tblk_bytes;
+  g.total = g.off_ops + 6 * g.op_bytes;            // the snapshots live in their own buffer (g.snap_bytes)
+  // header, reverse-state snapshots, delta, dO copy, dS / dSu tiles, and the forward snapshots when they are recomputed
+  g.bwd_total = kHeaderBytes + g.snap_bytes + g.lse_bytes + g.op_bytes + 2 * g.mat_bytes +
+                ((flags & CASTLE_FLAG_RECOMPUTE_STATE) ? g.snap_bytes : 0);
   return g;
 }
 
@@ -113,7 +114,7 @@ int check_core(int B, int H, int L, int d, int dtype) {
   return CASTLE_OK;
 }
 
-castle::FwdWorkspace carve(void* base, const Geometry& g) {
+castle::FwdWorkspace carve(void* base, void* state, const Geometry& g) {
   char* p = static_cast<char*>(base);
   castle::FwdWorkspace w;
   w.hdr = reinterpret_cast<castle::WsHeader*>(p);
@@ -122,7 +123,7 @@ castle::FwdWorkspace carve(void* base, const Geometry& g) {
   w.t_blk = p + g.off_t;
   w.tt_blk = p + g.off_tt;
   w.ttx_blk = p + g.off_ttx;
-  w.usnap = p + g.off_snap;
+  w.usnap = state;
   w.qc_p = p + g.off_ops;
   w.kc_p = p + g.off_ops + g.op_bytes;
   w.vc_p = p + g.off_ops + 2 * g.op_bytes;
@@ -157,11 +158,18 @@ int64_t castle_fwd_workspace_bytes(int B, int H, int L, int d, int dtype) {
   return geometry(B, H, L, d, elem_size(dtype)).total;
 }
 
+int64_t castle_fwd_state_bytes(int B, int H, int L, int d, int dtype) {
+  const int rc = check_core(B, H, L, d, dtype);
+  if (rc != CASTLE_OK) return rc;
+  const int64_t n = geometry(B, H, L, d, elem_size(dtype)).snap_bytes;
+  return n > 0 ? n : 256;   // a single block has no snapshots; keep the buffer non-empty
+}
+
 int castle_fwd(const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
                const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
                int B, int H, int L, int d, int dtype, float scale, int flags,
                const castle_view4* out, const castle_view4* U,
-               void* workspace, int64_t workspace_bytes, void* stream) {
+               void* workspace, int64_t workspace_bytes, void* state, int64_t state_bytes, void* stream) {
   int rc = check_core(B, H, L, d, dtype);
   if (rc != CASTLE_OK) return rc;
   const int es = elem_size(dtype);
@@ -173,6 +181,8 @@ int castle_fwd(const castle_view4* qc, const castle_view4* kc, const castle_view
   const Geometry g = geometry(B, H, L, d, es);
   if (workspace == nullptr || reinterpret_cast<uintptr_t>(workspace) % 256 != 0 || workspace_bytes < g.total)
     return CASTLE_ERR_WORKSPACE;
+  if (state == nullptr || reinterpret_cast<uintptr_t>(state) % 256 != 0 || state_bytes < g.snap_bytes)
+    return CASTLE_ERR_WORKSPACE;
 
   castle::FwdArgs a;
   a.s.B = B; a.s.H = H; a.s.L = L; a.s.d = d; a.s.Lp = g.Lp; a.s.nblk = g.nblk; a.s.scale = scale;
@@ -181,7 +191,7 @@ int castle_fwd(const castle_view4* qc, const castle_view4* kc, const castle_view
   a.qu = to_view(qu); a.ku = to_view(ku); a.vu = to_view(vu);
   a.out = to_view(out);
   a.U = to_view(want_U ? U : nullptr);
-  a.ws = carve(workspace, g);
+  a.ws = carve(workspace, state, g);
   return castle::launch_fwd(a, dtype, (flags & CASTLE_FLAG_BF16_OPERANDS) != 0, static_cast<hipStream_t>(stream));
 }
 
@@ -199,6 +209,7 @@ int castle_bwd(const castle_view4* qc, const castle_view4* kc, const castle_view
                const castle_view4* dqc, const castle_view4* dkc, const castle_view4* dvc,
                const castle_view4* dqu, const castle_view4* dku, const castle_view4* dvu,
                const void* fwd_workspace, int64_t fwd_workspace_bytes,
+               const void* fwd_state, int64_t fwd_state_bytes,
                void* bwd_workspace, int64_t bwd_workspace_bytes, void* stream) {
   int rc = check_core(B, H, L, d, dtype);
   if (rc != CASTLE_OK) return rc;
@@ -212,6 +223,10 @@ int castle_bwd(const castle_view4* qc, const castle_view4* kc, const castle_view
   if (bwd_workspace == nullptr || reinterpret_cast<uintptr_t>(bwd_workspace) % 256 != 0 ||
       bwd_workspace_bytes < g.bwd_total)
     return CASTLE_ERR_WORKSPACE;
+  const bool recompute_state = (flags & CASTLE_FLAG_RECOMPUTE_STATE) != 0;
+  if (!recompute_state &&
+      (fwd_state == nullptr || reinterpret_cast<uintptr_t>(fwd_state) % 256 != 0 || fwd_state_bytes < g.snap_bytes))
+    return CASTLE_ERR_WORKSPACE;
 
   castle::BwdArgs a;
   a.s.B = B; a.s.H = H; a.s.L = L; a.s.d = d; a.s.Lp = g.Lp; a.s.nblk = g.nblk; a.s.scale = scale;
@@ -221,8 +236,10 @@ int castle_bwd(const castle_view4* qc, const castle_view4* kc, const castle_view
   a.out = to_view(out); a.dout = to_view(dout);
   a.dqc = to_view(dqc); a.dkc = to_view(dkc); a.dvc = to_view(dvc);
   a.dqu = to_view(dqu); a.dku = to_view(dku); a.dvu = to_view(dvu);
-  a.ws = carve(const_cast<void*>(fwd_workspace), g);
   char* bw = static_cast<char*>(bwd_workspace);
+  // forward snapshots: the caller's, or recomputed into the tail of this call's own workspace
+  void* state = recompute_state ? bw + (g.bwd_total - g.snap_bytes) : const_cast<void*>(fwd_state);
+  a.ws = carve(const_cast<void*>(fwd_workspace), state, g);
   a.bhdr = reinterpret_cast<castle::BwdHeader*>(bw);
   a.amax_part = reinterpret_cast<float*>(bw + 256);
   bw += kHeaderBytes;
@@ -231,6 +248,16 @@ int castle_bwd(const castle_view4* qc, const castle_view4* kc, const castle_view
   a.dout_p = bw + g.snap_bytes + g.lse_bytes;
   a.ds_mat = g.mat_bytes ? bw + g.snap_bytes + g.lse_bytes + g.op_bytes : nullptr;
   a.dsu_mat = g.mat_bytes ? bw + g.snap_bytes + g.lse_bytes + g.op_bytes + g.mat_bytes : nullptr;
+  if (recompute_state) {   // the scan again, from the operand copies the forward pass left
+    castle::FwdArgs f;
+    f.s = a.s;
+    f.qc = a.qc; f.kc = a.kc; f.vc = a.vc; f.qu = a.qu; f.ku = a.ku; f.vu = a.vu;
+    f.out = a.out;
+    f.U = to_view(nullptr);
+    f.ws = a.ws;
+    rc = castle::launch_scan(f, dtype, (flags & CASTLE_FLAG_BF16_OPERANDS) != 0, static_cast<hipStream_t>(stream));
+    if (rc != 0) return rc;
+  }
   return castle::launch_bwd(a, dtype, (flags & CASTLE_FLAG_BF16_OPERANDS) != 0, static_cast<hipStream_t>(stream));
 }
 

@@ -518,6 +518,38 @@ template <typename T, typename TI> static int launch_fwd_d(const FwdArgs& a, hip
   }
 }
 
+// The scan alone (snapshots of the lookahead state into a.ws.usnap from the operand copies the
+// forward pass left): what the backward pass runs first when the forward snapshots were not kept.
+template <typename T, typename TI, int HD> static int launch_scan_t(const FwdArgs& a, hipStream_t stream) {
+  constexpr int scan_lds = scan_lds_bytes<T, HD>();
+  static PerDeviceOnce once;
+  bool& configured = once.flag();
+  if (!configured) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&scan_kernel<T, TI, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, scan_lds) != hipSuccess) return -3;
+    configured = true;
+  }
+  ProfScope ps(kSlotScan, stream);
+  hipLaunchKernelGGL((scan_kernel<T, TI, HD>), dim3(a.s.Lp / 128 * a.s.B * a.s.H), dim3(kThreads), scan_lds, stream, a);
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+template <typename T, typename TI> static int launch_scan_d(const FwdArgs& a, hipStream_t stream) {
+  switch (a.s.d) {
+    case 16: return launch_scan_t<T, TI, 16>(a, stream);
+    case 32: return launch_scan_t<T, TI, 32>(a, stream);
+    case 64: return launch_scan_t<T, TI, 64>(a, stream);
+    case 128: return launch_scan_t<T, TI, 128>(a, stream);
+    default: return -2;
+  }
+}
+int launch_scan(const FwdArgs& a, int dtype, bool bf16_operands, hipStream_t stream) {
+  switch (dtype) {
+    case 0: return launch_scan_d<float, float>(a, stream);
+    case 1: return bf16_operands ? launch_scan_d<bf16_t, bf16_t>(a, stream) : launch_scan_d<fp16_t, bf16_t>(a, stream);
+    case 2: return launch_scan_d<fp16_t, fp16_t>(a, stream);
+    default: return -1;
+  }
+}
+
 // bf16 tensors: operands are converted to fp16 on load (exact inside the fp16 range) and every
 // operand produced inside the kernels is fp16, unless bf16_operands asks for bf16 MFMA operands.
 int launch_fwd(const FwdArgs& a, int dtype, bool bf16_operands, hipStream_t stream) {

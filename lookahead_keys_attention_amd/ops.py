@@ -27,6 +27,10 @@ from . import _native as N
 # flags handed to castle_fwd / castle_bwd (0, or _native.FLAG_BF16_OPERANDS); read when the
 # forward runs and remembered for its backward.  The `rotary` arguments below add FLAG_ROTARY.
 DEFAULT_FLAGS = 0
+# A forward call keeps its state snapshots (B*H*L^2*d/128 elements) for its backward pass when they
+# take at most this many bytes; beyond it they are dropped after the forward pass and the backward
+# pass runs the scan again first (what a call keeps is then O(L d)).  0 = never keep.
+KEEP_STATE_LIMIT_BYTES = 8 << 30
 # Debugging aid: when True every parallel forward waits for its kernels and raises if they had to
 # clamp a value to the fp16 range (an input element of a bf16 tensor beyond +-65504, or a T' entry):
 # the result is then that of the clamped operands.  Off by default because it synchronises.
@@ -46,24 +50,30 @@ def _check_dims(d: int, dtype: torch.dtype):
 
 
 def _fwd_raw(qc, kc, vc, qu, ku, vu, scale, out, U, flags=0):
-    """Launch castle_fwd; returns the forward workspace tensor."""
+    """Launch castle_fwd; returns (workspace, state): the tensors the backward pass needs back.
+    `state` is an empty tensor when the snapshots are too large to keep (KEEP_STATE_LIMIT_BYTES)."""
     B, H, L, d = qc.shape
     code = N.dtype_code(qc.dtype)
     lib = N.lib()
     nbytes = N.check(lib.castle_fwd_workspace_bytes(B, H, L, d, code), "castle_fwd_workspace_bytes")
+    sbytes = N.check(lib.castle_fwd_state_bytes(B, H, L, d, code), "castle_fwd_state_bytes")
     ws = torch.empty(nbytes, dtype=torch.uint8, device=qc.device)
+    state = torch.empty(sbytes, dtype=torch.uint8, device=qc.device)
     views = [N.view4(t) for t in (qc, kc, vc, qu, ku, vu)]
     vo = N.view4(out)
     vU = N.view4(U) if U is not None else N.View4(None, 0, 0, 0)
     with torch.cuda.device(qc.device):
-        rc = lib.castle_fwd(*views, B, H, L, d, code, float(scale), int(flags), vo, vU, ws.data_ptr(), nbytes, N.stream_ptr(qc.device))
+        rc = lib.castle_fwd(*views, B, H, L, d, code, float(scale), int(flags), vo, vU, ws.data_ptr(), nbytes,
+                            state.data_ptr(), sbytes, N.stream_ptr(qc.device))
     N.check(rc, "castle_fwd")
+    if sbytes > KEEP_STATE_LIMIT_BYTES:
+        state = torch.empty(0, dtype=torch.uint8, device=qc.device)   # the caching allocator keeps the block until the stream is done with it
     if CHECK_RANGE:
         status = range_status(ws)
         if status:
             raise RuntimeError(f"castle_fwd clamped values to the fp16 range (status bits {status:#x}: "
                                "1 = input element, 2 = T' = s qc.vu entry)")
-    return ws
+    return ws, state
 
 
 def range_status(ws: torch.Tensor) -> int:
@@ -72,17 +82,20 @@ def range_status(ws: torch.Tensor) -> int:
     return int(ws[:4].view(torch.int32).item())
 
 
-def _bwd_raw(qc, kc, vc, qu, ku, vu, out, dout, scale, grads, ws, flags=0):
+def _bwd_raw(qc, kc, vc, qu, ku, vu, out, dout, scale, grads, ws, state, flags=0):
     B, H, L, d = qc.shape
     code = N.dtype_code(qc.dtype)
     lib = N.lib()
+    if state.numel() == 0:
+        flags |= N.FLAG_RECOMPUTE_STATE
     nbytes = N.check(lib.castle_bwd_workspace_bytes(B, H, L, d, code, int(flags)), "castle_bwd_workspace_bytes")
     bws = torch.empty(nbytes, dtype=torch.uint8, device=qc.device)
     views = [N.view4(t) for t in (qc, kc, vc, qu, ku, vu, out, dout)]
     gviews = [N.view4(t) for t in grads]
     with torch.cuda.device(qc.device):
         rc = lib.castle_bwd(*views, B, H, L, d, code, float(scale), int(flags), *gviews,
-                            ws.data_ptr(), ws.numel(), bws.data_ptr(), nbytes, N.stream_ptr(qc.device))
+                            ws.data_ptr(), ws.numel(), state.data_ptr() if state.numel() else None, state.numel(),
+                            bws.data_ptr(), nbytes, N.stream_ptr(qc.device))
     N.check(rc, "castle_bwd")
 
 
@@ -106,6 +119,11 @@ def _out_like(q):
     return torch.empty((B, L, H, d), dtype=q.dtype, device=q.device).permute(0, 2, 1, 3)
 
 
+def _fake_state(B, H, L, d, like):
+    n = N.check(N.lib().castle_fwd_state_bytes(int(B), int(H), int(L), int(d), N.dtype_code(like.dtype)), "castle_fwd_state_bytes")
+    return torch.empty(n if n <= KEEP_STATE_LIMIT_BYTES else 0, dtype=torch.uint8, device=like.device)
+
+
 def _fwd_ws_bytes(B, H, L, d, dtype):
     return N.check(N.lib().castle_fwd_workspace_bytes(int(B), int(H), int(L), int(d), N.dtype_code(dtype)),
                    "castle_fwd_workspace_bytes")
@@ -113,15 +131,15 @@ def _fwd_ws_bytes(B, H, L, d, dtype):
 
 @torch.library.custom_op("castle_hip::attention", mutates_args=())
 def _attention_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, qu: torch.Tensor, ku: torch.Tensor,
-                  vu: torch.Tensor, scale: float, want_U: bool, flags: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+                  vu: torch.Tensor, scale: float, want_U: bool, flags: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     _require_gpu(q, "castle_attention_hip")
     B, H, L, d = q.shape
     _check_dims(d, q.dtype)
     ops = [_as_readable(t) for t in (q, k, v, qu, ku, vu)]
     out = _out_like(q)
     U = torch.empty((B, H, L, d) if want_U else (0,), dtype=q.dtype, device=q.device)
-    ws = _fwd_raw(*ops, scale, out, U if want_U else None, flags)
-    return out, U, ws
+    ws, state = _fwd_raw(*ops, scale, out, U if want_U else None, flags)
+    return out, U, ws, state
 
 
 @_attention_op.register_fake
@@ -130,36 +148,36 @@ def _(q, k, v, qu, ku, vu, scale, want_U, flags):
     _check_dims(d, q.dtype)
     U = torch.empty((B, H, L, d) if want_U else (0,), dtype=q.dtype, device=q.device)
     ws = torch.empty(_fwd_ws_bytes(B, H, L, d, q.dtype), dtype=torch.uint8, device=q.device)
-    return _out_like(q), U, ws
+    return _out_like(q), U, ws, _fake_state(B, H, L, d, q)
 
 
 @torch.library.custom_op("castle_hip::attention_bwd", mutates_args=())
 def _attention_bwd_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, qu: torch.Tensor, ku: torch.Tensor,
-                      vu: torch.Tensor, out: torch.Tensor, dout: torch.Tensor, ws: torch.Tensor,
+                      vu: torch.Tensor, out: torch.Tensor, dout: torch.Tensor, ws: torch.Tensor, state: torch.Tensor,
                       scale: float, flags: int) -> torch.Tensor:
     B, H, L, d = q.shape
     ops = [_as_readable(t) for t in (q, k, v, qu, ku, vu)]
     packed = torch.empty((6, B, H, L, d), dtype=out.dtype, device=out.device)
-    _bwd_raw(*ops, _as_readable(out), _as_readable(dout), scale, list(packed.unbind(0)), ws, flags)
+    _bwd_raw(*ops, _as_readable(out), _as_readable(dout), scale, list(packed.unbind(0)), ws, state, flags)
     return packed
 
 
 @_attention_bwd_op.register_fake
-def _(q, k, v, qu, ku, vu, out, dout, ws, scale, flags):
+def _(q, k, v, qu, ku, vu, out, dout, ws, state, scale, flags):
     return torch.empty((6, *q.shape), dtype=out.dtype, device=out.device)
 
 
 def _attention_setup(ctx, inputs, output):
     q, k, v, qu, ku, vu, scale, want_U, flags = inputs
-    out, U, ws = output
-    ctx.save_for_backward(q, k, v, qu, ku, vu, out, ws)
+    out, U, ws, state = output
+    ctx.save_for_backward(q, k, v, qu, ku, vu, out, ws, state)
     ctx.scale, ctx.flags = scale, flags
-    ctx.mark_non_differentiable(U, ws)   # U carries no gradient (lookahead_keys_attention_triton.py:513-515)
+    ctx.mark_non_differentiable(U, ws, state)   # U carries no gradient (lookahead_keys_attention_triton.py:513-515)
 
 
-def _attention_backward(ctx, dout, dU, dws):
-    q, k, v, qu, ku, vu, out, ws = ctx.saved_tensors
-    grads = torch.ops.castle_hip.attention_bwd(q, k, v, qu, ku, vu, out, dout, ws, ctx.scale, ctx.flags)
+def _attention_backward(ctx, dout, dU, dws, dstate):
+    q, k, v, qu, ku, vu, out, ws, state = ctx.saved_tensors
+    grads = torch.ops.castle_hip.attention_bwd(q, k, v, qu, ku, vu, out, dout, ws, state, ctx.scale, ctx.flags)
     return (*grads.unbind(0), None, None, None)
 
 
@@ -179,7 +197,7 @@ def _packed_ok(t):
 
 @torch.library.custom_op("castle_hip::attention_packed", mutates_args=())
 def _attention_packed_op(proj: torch.Tensor, heads: int, scale: float, want_U: bool, row_capacity: int,
-                         flags: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+                         flags: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     # The lookahead keys come back as the first L rows of a (B, H, row_capacity, d) buffer, so that a
     # caller can hand over the U buffer of a decode cache without copying (row_capacity >= L).
     _require_gpu(proj, "castle_attention_packed")
@@ -190,8 +208,8 @@ def _attention_packed_op(proj: torch.Tensor, heads: int, scale: float, want_U: b
     merged = torch.empty((B, L, heads * d), dtype=proj.dtype, device=proj.device)
     out = merged.view(B, L, heads, d).permute(0, 2, 1, 3)
     U = torch.empty((B, heads, max(row_capacity, L), d) if want_U else (0,), dtype=proj.dtype, device=proj.device)
-    ws = _fwd_raw(qc, kc, vc, qu, ku, vu, scale, out, U[:, :, :L] if want_U else None, flags)
-    return merged, U, ws
+    ws, state = _fwd_raw(qc, kc, vc, qu, ku, vu, scale, out, U[:, :, :L] if want_U else None, flags)
+    return merged, U, ws, state
 
 
 @_attention_packed_op.register_fake
@@ -201,12 +219,12 @@ def _(proj, heads, scale, want_U, row_capacity, flags):
     _check_dims(d, proj.dtype)
     ws = torch.empty(_fwd_ws_bytes(B, heads, L, d, proj.dtype), dtype=torch.uint8, device=proj.device)
     U = torch.empty((B, heads, max(row_capacity, L), d) if want_U else (0,), dtype=proj.dtype, device=proj.device)
-    return torch.empty((B, L, heads * d), dtype=proj.dtype, device=proj.device), U, ws
+    return torch.empty((B, L, heads * d), dtype=proj.dtype, device=proj.device), U, ws, _fake_state(B, heads, L, d, proj)
 
 
 @torch.library.custom_op("castle_hip::attention_packed_bwd", mutates_args=())
 def _attention_packed_bwd_op(proj: torch.Tensor, merged: torch.Tensor, dmerged: torch.Tensor, ws: torch.Tensor,
-                             heads: int, scale: float, flags: int) -> torch.Tensor:
+                             state: torch.Tensor, heads: int, scale: float, flags: int) -> torch.Tensor:
     B, L, width = proj.shape
     d = width // (6 * heads)
     qu, ku, vu, qc, kc, vc = _six_views(_packed_ok(proj), heads)
@@ -214,26 +232,26 @@ def _attention_packed_bwd_op(proj: torch.Tensor, merged: torch.Tensor, dmerged: 
     dout = _packed_ok(dmerged).view(B, L, heads, d).permute(0, 2, 1, 3)
     dproj = torch.empty((B, L, width), dtype=proj.dtype, device=proj.device)
     dqu, dku, dvu, dqc, dkc, dvc = _six_views(dproj, heads)
-    _bwd_raw(qc, kc, vc, qu, ku, vu, out, dout, scale, (dqc, dkc, dvc, dqu, dku, dvu), ws, flags)
+    _bwd_raw(qc, kc, vc, qu, ku, vu, out, dout, scale, (dqc, dkc, dvc, dqu, dku, dvu), ws, state, flags)
     return dproj
 
 
 @_attention_packed_bwd_op.register_fake
-def _(proj, merged, dmerged, ws, heads, scale, flags):
+def _(proj, merged, dmerged, ws, state, heads, scale, flags):
     return torch.empty(proj.shape, dtype=proj.dtype, device=proj.device)
 
 
 def _packed_setup(ctx, inputs, output):
     proj, heads, scale, want_U, row_capacity, flags = inputs
-    merged, U, ws = output
-    ctx.save_for_backward(proj, merged, ws)
+    merged, U, ws, state = output
+    ctx.save_for_backward(proj, merged, ws, state)
     ctx.heads, ctx.scale, ctx.flags = heads, scale, flags
-    ctx.mark_non_differentiable(U, ws)
+    ctx.mark_non_differentiable(U, ws, state)
 
 
-def _packed_backward(ctx, dmerged, dU, dws):
-    proj, merged, ws = ctx.saved_tensors
-    dproj = torch.ops.castle_hip.attention_packed_bwd(proj, merged, dmerged, ws, ctx.heads, ctx.scale, ctx.flags)
+def _packed_backward(ctx, dmerged, dU, dws, dstate):
+    proj, merged, ws, state = ctx.saved_tensors
+    dproj = torch.ops.castle_hip.attention_packed_bwd(proj, merged, dmerged, ws, state, ctx.heads, ctx.scale, ctx.flags)
     return dproj, None, None, None, None, None
 
 
@@ -244,7 +262,7 @@ def castle_attention_hip(q, k, v, qu, ku, vu, scale, return_U_for_cache=False, r
     """Drop-in for castle_attention_triton: returns out, or (out, U).  rotary=True applies the
     rotary position embedding (positions 0..L-1) to q, k, qu, ku, vu inside the kernels."""
     flags = DEFAULT_FLAGS | (N.FLAG_ROTARY if rotary else 0)
-    out, U, _ = torch.ops.castle_hip.attention(q, k, v, qu, ku, vu, float(scale), bool(return_U_for_cache), int(flags))
+    out, U, _, _ = torch.ops.castle_hip.attention(q, k, v, qu, ku, vu, float(scale), bool(return_U_for_cache), int(flags))
     return (out, U) if return_U_for_cache else out
 
 
@@ -253,7 +271,7 @@ def castle_attention_packed(proj, heads, scale, return_U_for_cache=False, row_ca
     `row_capacity` > L it is the first L rows of a freshly allocated (B,H,row_capacity,d) buffer
     (reachable as U._base), which a decode cache can adopt as its U buffer without a copy."""
     flags = DEFAULT_FLAGS | (N.FLAG_ROTARY if rotary else 0)
-    merged, U, _ = torch.ops.castle_hip.attention_packed(proj, int(heads), float(scale), bool(return_U_for_cache),
+    merged, U, _, _ = torch.ops.castle_hip.attention_packed(proj, int(heads), float(scale), bool(return_U_for_cache),
                                                          int(row_capacity), int(flags))
     return (merged, U[:, :, : proj.shape[1]]) if return_U_for_cache else merged
 

@@ -43,13 +43,18 @@ def test_version_and_error_strings(lib):
 
 
 def test_workspace_sizes(lib):
-    # B4 H8 L4096 d64 bf16: lse + three T arrays (T', T'^T, cross quarter) + snapshots (64 * nblk*(nblk-1)/2 rows per head) + six operand copies
+    # B4 H8 L4096 d64 bf16.  Kept for backward (O(L d)): header + lse + three T arrays (T', T'^T, cross quarter) +
+    # six operand copies; state buffer (O(L^2 d / 128)): snapshots, 64 * nblk*(nblk-1)/2 rows per head
     n = lib.castle_fwd_workspace_bytes(4, 8, 4096, 64, 1)
     BH, Lp, nblk = 32, 4096, 64
     header = 256 + 4 * 256   # status / scale header + partial maxima
-    expect = header + BH * Lp * 4 + 3 * BH * Lp * 64 * 2 + BH * 64 * nblk * (nblk - 1) // 2 * 64 * 2 + 6 * BH * Lp * 64 * 2
-    assert n == expect
-    assert lib.castle_bwd_workspace_bytes(4, 8, 4096, 64, 1, 0) == header + BH * 64 * nblk * (nblk - 1) // 2 * 64 * 2 + BH * Lp * 4 + BH * Lp * 64 * 2 + 2 * BH * Lp * Lp * 2
+    snaps = BH * 64 * nblk * (nblk - 1) // 2 * 64 * 2
+    assert n == header + BH * Lp * 4 + 3 * BH * Lp * 64 * 2 + 6 * BH * Lp * 64 * 2
+    assert lib.castle_fwd_state_bytes(4, 8, 4096, 64, 1) == snaps
+    bwd = header + snaps + BH * Lp * 4 + BH * Lp * 64 * 2 + 2 * BH * Lp * Lp * 2
+    assert lib.castle_bwd_workspace_bytes(4, 8, 4096, 64, 1, 0) == bwd
+    assert lib.castle_bwd_workspace_bytes(4, 8, 4096, 64, 1, N.FLAG_RECOMPUTE_STATE) == bwd + snaps
+    assert lib.castle_bwd_workspace_bytes(4, 8, 4096, 64, 1, N.FLAG_RECOMPUTE_SCORES) == bwd - 2 * BH * Lp * Lp * 2
     # ragged L rounds up to 128 rows
     assert lib.castle_fwd_workspace_bytes(1, 1, 129, 64, 0) == lib.castle_fwd_workspace_bytes(1, 1, 256, 64, 0)
     assert lib.castle_decode_workspace_bytes(32, 8, 64, 4096) > 0
@@ -68,7 +73,7 @@ def test_null_and_misaligned_views_are_rejected_on_the_host(lib):
     null = N.View4(None, 0, 0, 0)
     odd = N.View4(4098, 64, 64, 64)          # not 16-byte aligned
     bad_stride = N.View4(4096, 64, 64, 3)    # rows not 16-byte aligned
-    args = lambda v: ([ok] * 5 + [v], [1, 1, 16, 64, 1, 0.125, 0, ok, null, 4096, 1 << 30, None])
+    args = lambda v: ([ok] * 5 + [v], [1, 1, 16, 64, 1, 0.125, 0, ok, null, 4096, 1 << 30, 8192, 1 << 30, None])
     for bad in (null, odd, bad_stride):
         a, b = args(bad)
         assert lib.castle_fwd(*a, *b) == -5
@@ -76,6 +81,8 @@ def test_null_and_misaligned_views_are_rejected_on_the_host(lib):
     b[9] = None                                # no workspace
     assert lib.castle_fwd(*a, *b) == -4
     b[9], b[10] = 4096, 16                     # too small
+    assert lib.castle_fwd(*a, *b) == -4
+    b[10], b[11] = 1 << 30, None               # no state buffer
     assert lib.castle_fwd(*a, *b) == -4
 
 

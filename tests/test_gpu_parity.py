@@ -232,6 +232,29 @@ def test_bf16_inputs_beyond_the_fp16_range_are_clamped_and_reported(monkeypatch)
     H().castle_attention_hip(*[t.to(DEV) for t in ops2], s)     # in range: no complaint
 
 
+@pytest.mark.parametrize("L,d,dtype", [(640, 64, torch.bfloat16), (300, 32, torch.float32), (260, 128, torch.bfloat16)])
+def test_backward_that_recomputes_the_forward_state(L, d, dtype, monkeypatch):
+    """KEEP_STATE_LIMIT_BYTES = 0: the snapshot buffer is dropped after the forward pass (what the call
+    keeps is O(L d)) and castle_bwd runs the scan again first (FLAG_RECOMPUTE_STATE).  Same kernels,
+    same inputs: the gradients are bit for bit those of the run that kept the snapshots."""
+    ops, dout = rand_ops(1, 2, L, d, dtype, seed=L + 1)
+    s = d ** -0.5
+
+    def grads():
+        leaves = [t.to(DEV).requires_grad_() for t in ops]
+        H().castle_attention_hip(*leaves, s).backward(dout.to(DEV))
+        return [leaf.grad.cpu() for leaf in leaves]
+
+    kept = grads()
+    monkeypatch.setattr(H(), "KEEP_STATE_LIMIT_BYTES", 0)
+    again = grads()
+    for name, a, b in zip(NAMES, kept, again):
+        assert torch.equal(a, b), name
+    ref = O.closed_form_grads(*[t.double() for t in ops], s, dout.double())
+    for name, got, r in zip(NAMES, again, ref):
+        assert_close(got, r, dtype, name, 2e-2)
+
+
 def test_two_streams_run_the_operator_side_by_side():
     """Every launch goes to the caller's stream and every call owns its workspace: two forward +
     backward passes enqueued on two streams without synchronising in between give, bit for bit,
