@@ -69,6 +69,26 @@ typedef struct castle_view4 {
   int64_t stride_l;
 } castle_view4;
 
+/* Deferred write-back of the lookahead keys in the cached step (optional argument of the three
+ * castle_decode_step* entry points; NULL = U is written by every step, as the reference's step does,
+ * lookahead_keys_attention.py:183).  With it the U rows are written on every 4th step only (the steps
+ * whose row count t has (t + 1) % 4 == 0).  In between, the vu rows of the up to 3 tokens not yet
+ * folded into the stored U ("pending") sit in `vu_ring`, a (B, H, 4, d) buffer in the element type
+ * (token j in row j % 4, written by the step that appends j), and the gate each cached row k got from
+ * pending token j in `gates`, a (B, H, capacity, 4) fp32 array ([k][j % 4]; stride_l is not used, the
+ * rows are 4 floats apart).  Every step adds gate * vu of the pending tokens in fp32: a tenth less
+ * HBM traffic per step and a quarter of the roundings of a 16-bit U.  `base`: every U row already
+ * holds all sources below `base` (the prefill length, or the row count at the last castle_decode_flush);
+ * the sources pending at row count t are max(base, t - t % 4) .. t - 1.  `base_device`, if not NULL,
+ * is read by the kernels instead (graph replay).  The stored U is complete whenever nothing is
+ * pending; castle_decode_flush makes it so at any other time. */
+typedef struct castle_deferred {
+  castle_view4 vu_ring;
+  castle_view4 gates;
+  int32_t base;
+  const int32_t* base_device;
+} castle_deferred;
+
 int castle_abi_version(void);
 const char* castle_error_string(int code);
 
@@ -136,8 +156,13 @@ int castle_decode_step(const castle_view4* U, const castle_view4* qu_cache,
                        const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
                        const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
                        int B, int H, int d, int dtype, float scale, int flags,
-                       const castle_view4* out,
+                       const castle_view4* out, const castle_deferred* deferred,
                        void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Folds the pending sources into the stored lookahead keys (see castle_deferred): afterwards the U
+ * rows 0 .. t-1 are what a step-by-step update would have left, and `base` = t describes the cache. */
+int castle_decode_flush(const castle_view4* U, const castle_view4* qu_cache, int t, const castle_deferred* deferred,
+                        int B, int H, int d, int dtype, float scale, void* stream);
 
 /* The same step with the row count t read by the kernels from device memory (*t_device, an int32
  * the caller keeps and advances), so that the enqueued work does not depend on t: one captured HIP
@@ -152,7 +177,7 @@ int castle_decode_step_device_count(const castle_view4* U, const castle_view4* q
                                     const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
                                     const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
                                     int B, int H, int d, int dtype, float scale, int flags,
-                                    const castle_view4* out,
+                                    const castle_view4* out, const castle_deferred* deferred,
                                     void* workspace, int64_t workspace_bytes, void* stream);
 
 /* The cached step for callers that cannot allocate or bring a workspace (code under HIP graph
@@ -173,7 +198,7 @@ int castle_decode_step_static(const castle_view4* U, const castle_view4* qu_cach
                               const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
                               const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
                               int B, int H, int d, int dtype, float scale, int flags,
-                              const castle_view4* out, void* stream);
+                              const castle_view4* out, const castle_deferred* deferred, void* stream);
 
 /* Rotary position embedding of one tensor, out of place: out[b,h,l,:] = R(first_position + l) x[b,h,l,:]
  * (the rotation CASTLE_FLAG_ROTARY applies inside the kernels; lookahead_keys_attention.py:112).  Used to

@@ -34,6 +34,7 @@ EXPORTED_SYMBOLS = (
     "castle_decode_step",
     "castle_decode_step_device_count",
     "castle_decode_step_static",
+    "castle_decode_flush",
     "castle_rope",
     "castle_small_linear",
     "castle_profile_enable",
@@ -52,7 +53,20 @@ class View4(ctypes.Structure):
     ]
 
 
+class Deferred(ctypes.Structure):
+    """struct castle_deferred"""
+
+    _fields_ = [
+        ("vu_ring", View4),
+        ("gates", View4),
+        ("base", ctypes.c_int32),
+        ("base_device", ctypes.c_void_p),
+    ]
+
+
+DECODE_DEFER = 4   # U is written on every 4th step when a castle_deferred is handed over
 _VP = ctypes.POINTER(View4)
+_DP = ctypes.POINTER(Deferred)
 _lib = None
 _lock = threading.Lock()
 
@@ -80,11 +94,13 @@ def _declare(lib):
     lib.castle_profile_read.restype = i
     lib.castle_profile_read.argtypes = [ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_float), i]
     lib.castle_decode_step.restype = i
-    lib.castle_decode_step.argtypes = [_VP] * 4 + [i, i] + [_VP] * 6 + [i, i, i, i, f, i, _VP, vp, i64, vp]
+    lib.castle_decode_step.argtypes = [_VP] * 4 + [i, i] + [_VP] * 6 + [i, i, i, i, f, i, _VP, _DP, vp, i64, vp]
     lib.castle_decode_step_static.restype = i
-    lib.castle_decode_step_static.argtypes = [_VP] * 4 + [i, vp, i] + [_VP] * 6 + [i, i, i, i, f, i, _VP, vp]
+    lib.castle_decode_step_static.argtypes = [_VP] * 4 + [i, vp, i] + [_VP] * 6 + [i, i, i, i, f, i, _VP, _DP, vp]
+    lib.castle_decode_flush.restype = i
+    lib.castle_decode_flush.argtypes = [_VP, _VP, i, _DP, i, i, i, i, f, vp]
     lib.castle_decode_step_device_count.restype = i
-    lib.castle_decode_step_device_count.argtypes = [_VP] * 4 + [vp, i] + [_VP] * 6 + [i, i, i, i, f, i, _VP, vp, i64, vp]
+    lib.castle_decode_step_device_count.argtypes = [_VP] * 4 + [vp, i] + [_VP] * 6 + [i, i, i, i, f, i, _VP, _DP, vp, i64, vp]
     lib.castle_small_linear.restype = i
     lib.castle_small_linear.argtypes = [vp, vp, vp, i, i, i, i64, i64, i64, i, vp]
     lib.castle_rope.restype = i

@@ -40,9 +40,31 @@ _CacheFields = namedtuple("Cache", ("U", "qu_cache", "kc_cache", "vc_cache"))
 
 
 class Cache(_CacheFields):
-    """Four (B, H, n, d) tensors; field names as in the reference (lookahead_keys_attention.py:26)."""
+    """Four (B, H, n, d) tensors; field names as in the reference (lookahead_keys_attention.py:26).
+
+    A cache made by the native path is a set of views into its capacity buffers.  The native step
+    writes the lookahead keys back on every 4th step only (the tokens in between are kept as pending
+    (ku, vu) rows and applied on the fly), so whoever READS `U` (the attribute, index 0, unpacking)
+    first gets the pending sources folded in: the tensor seen is always the true U."""
 
     _store = None   # set on caches that live in a native capacity buffer
+
+    def _complete(self):
+        if self._store is not None:
+            self._store.flush()
+
+    @property
+    def U(self):
+        self._complete()
+        return tuple.__getitem__(self, 0)
+
+    def __getitem__(self, index):
+        self._complete()
+        return tuple.__getitem__(self, index)
+
+    def __iter__(self):
+        self._complete()
+        return tuple.__iter__(self)
 
 
 class _CacheStore:
@@ -54,6 +76,12 @@ class _CacheStore:
         self.buffers = (first,) + tuple(torch.empty((B, H, capacity, d), dtype=dtype, device=device) for _ in range(3))
         self.capacity = capacity
         self.length = 0
+        # deferred write-back of the lookahead keys: pending (ku, vu) rows, and the row count up to
+        # which every U row is known to be complete
+        self.rings = (torch.empty((B, H, _native.DECODE_DEFER, d), dtype=dtype, device=device),                 # pending vu rows
+                      torch.empty((B, H, capacity, _native.DECODE_DEFER), dtype=torch.float32, device=device))   # their gates per cached row
+        self.base0 = 0
+        self.scale = d ** -0.5
         self._geometry = (B, H, d, device)
         self._workspace = None
         self._views = None
@@ -73,6 +101,24 @@ class _CacheStore:
             self._views = tuple(_native.view4(buf) for buf in self.buffers)
         return self._views
 
+    def deferred(self, base_device=None):
+        """struct castle_deferred of this store, for a step at row count `self.length` (None when the
+        deferred write-back is switched off and nothing is pending: such steps write U themselves)."""
+        if not ops.DEFER_LOOKAHEAD_WRITES and self.pending() == 0:
+            return None
+        return ops.make_deferred(self.rings[0], self.rings[1], self.base0, base_device)
+
+    def pending(self) -> int:
+        """Sources not yet folded into the stored lookahead keys."""
+        t = self.length
+        return t - max(self.base0, t - t % _native.DECODE_DEFER)
+
+    def flush(self):
+        """Completes the stored lookahead keys (no-op when nothing is pending)."""
+        if self.pending() > 0:
+            ops.castle_decode_flush(self.buffers[0], self.buffers[1], self.length, self.deferred(), self.scale)
+        self.base0 = self.length
+
     def as_cache(self) -> Cache:
         n = self.length
         cache = Cache(*(buf[:, :, :n] for buf in self.buffers))
@@ -81,10 +127,12 @@ class _CacheStore:
 
     def grown(self, min_capacity):
         B, H, _, d = self.buffers[0].shape
+        self.flush()
         new = _CacheStore(B, H, d, max(min_capacity, 2 * self.capacity), self.buffers[0].dtype, self.buffers[0].device)
         for dst, src in zip(new.buffers, self.buffers):
             dst[:, :, : self.length].copy_(src[:, :, : self.length])
-        new.length = self.length
+        new.length = new.base0 = self.length
+        new.scale = self.scale
         return new
 
 
@@ -208,7 +256,8 @@ class Castle(nn.Module):
                 store.buffers[1][:, :, :n].copy_(qu)
                 store.buffers[2][:, :, :n].copy_(kc)
             store.buffers[3][:, :, :n].copy_(vc)
-        store.length = n
+        store.length = store.base0 = n
+        store.scale = self.scale
         return merged, store.as_cache()
 
     def _step_native(self, proj, cache):
@@ -223,34 +272,42 @@ class Castle(nn.Module):
             store = _CacheStore(B, H, d, _reserve_rows(t + 1), proj.dtype, proj.device)
             for buf, src in zip(store.buffers, cache):
                 buf[:, :, :t].copy_(src)
-            store.length = t
-        elif store.length != cache[0].shape[-2]:
+            store.length = store.base0 = t
+        elif store.length != cache.kc_cache.shape[-2]:   # (not cache.U: reading it would write the pending keys back)
             raise RuntimeError("this cache was already advanced by a later decode step; the native "
                                "decode updates its cache in place, so a cache can be used once")
+        store.scale = self.scale
         t = store.length
         if t + 1 > store.capacity:
             store = store.grown(_reserve_rows(t + 1))
         out = torch.empty((B, 1, H, d), dtype=proj.dtype, device=proj.device)
+        deferred = store.deferred()
         if proj.is_contiguous() and proj.data_ptr() % 16 == 0:
             ops.castle_decode_step_packed(store.views, store.capacity, t, proj, H, self.scale, out, store.workspace,
-                                          rotary=self.use_rotary)
+                                          rotary=self.use_rotary, deferred=deferred)
         else:
             ops.castle_decode_step_hip(*store.buffers, t, qc, kc, vc, qu, ku, vu, self.scale,
-                                       out.permute(0, 2, 1, 3), store.workspace, rotary=self.use_rotary)
+                                       out.permute(0, 2, 1, 3), store.workspace, rotary=self.use_rotary,
+                                       deferred=deferred)
+        if deferred is None:
+            store.base0 = t + 1   # this step wrote the lookahead keys itself: nothing is pending
         store.length = t + 1
         return out.view(B, 1, H * d), store.as_cache()
 
-    def graph_step(self, x, store, t_device):
+    def graph_step(self, x, store, t_device, base_device=None):
         """The cached single-token step in the form a captured HIP graph needs: the same GPU work
         as forward(x, cache) on the native path, but the row count is read by the kernels from the
         one-element int32 GPU tensor `t_device`, and nothing on the host depends on it (no cache
         object is built, `store.length` is left alone: the owner of the graph keeps the count).
+        `base_device` (one-element int32 GPU tensor: the row count up to which the stored lookahead
+        keys are complete, e.g. the prefill length) switches the deferred write-back on.
         x: (B, 1, dim); store: the `_CacheStore` behind a native cache.  Returns (B, 1, dim)."""
         B = x.shape[0]
         proj = self._project(self.to_all_qkv, self.norm(x), True)
         out = torch.empty((B, 1, self.heads, self.dim_head), dtype=proj.dtype, device=proj.device)
         ops.castle_decode_step_packed(store.views, store.capacity, 0, proj, self.heads, self.scale, out,
-                                      store.workspace, rotary=self.use_rotary, t_device=t_device)
+                                      store.workspace, rotary=self.use_rotary, t_device=t_device,
+                                      deferred=store.deferred(base_device) if base_device is not None else None)
         return self._project(self.combine_heads, out.view(B, 1, self.heads * self.dim_head), True)
 
     # -- dense PyTorch formulation (use_triton=False) -------------------------

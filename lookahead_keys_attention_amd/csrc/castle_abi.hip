@@ -14,6 +14,7 @@ int launch_fwd(const FwdArgs& a, int dtype, bool bf16_operands, hipStream_t stre
 int launch_scan(const FwdArgs& a, int dtype, bool bf16_operands, hipStream_t stream);
 int launch_bwd(const BwdArgs& a, int dtype, bool bf16_operands, hipStream_t stream);
 int launch_decode(const DecodeArgs& a, int dtype, hipStream_t stream);
+int launch_decode_flush(const DecodeArgs& a, int dtype, hipStream_t stream);
 int launch_rope(const View4& src, const View4& dst, int B, int H, int L, int d, int dtype, int pos0, hipStream_t stream);
 int decode_pick_splits(int BH, int t);
 int decode_static_scratch(float** ptr);
@@ -272,7 +273,7 @@ static int decode_step_common(const castle_view4* U, const castle_view4* qu_cach
                               const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
                               const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
                               int B, int H, int d, int dtype, float scale, int flags,
-                              const castle_view4* out,
+                              const castle_view4* out, const castle_deferred* deferred,
                               void* workspace, int64_t workspace_bytes, bool static_scratch, void* stream) {
   const int es = elem_size(dtype);
   if (es == 0) return CASTLE_ERR_DTYPE;
@@ -284,6 +285,13 @@ static int decode_step_common(const castle_view4* U, const castle_view4* qu_cach
   const castle_view4* tok[] = {qc, kc, vc, qu, ku, vu, out};
   for (const castle_view4* v : tok)
     if (!view_ok(v, es, false)) return CASTLE_ERR_ARG;
+  if (deferred != nullptr) {
+    if (!view_ok(&deferred->vu_ring, es, true) || !view_ok(&deferred->gates, 4, false)) return CASTLE_ERR_ARG;
+    if (deferred->base < 0 || (deferred->base_device != nullptr && reinterpret_cast<uintptr_t>(deferred->base_device) % 4 != 0))
+      return CASTLE_ERR_ARG;
+    // host-side counts: the pending sources must all fit the ring
+    if (t_device == nullptr && deferred->base_device == nullptr && deferred->base > t) return CASTLE_ERR_SHAPE;
+  }
   // with a device-side count the split must not depend on it: sized for a full cache
   const int splits = castle::decode_pick_splits(B * H, t_device != nullptr ? capacity : t);
   if (static_scratch) {
@@ -307,6 +315,10 @@ static int decode_step_common(const castle_view4* U, const castle_view4* qu_cach
   a.qu = to_view(qu); a.ku = to_view(ku); a.vu = to_view(vu);
   a.out = to_view(out);
   a.part = static_cast<float*>(workspace);
+  a.pend_vu = to_view(deferred != nullptr ? &deferred->vu_ring : nullptr);
+  a.pend_gate = to_view(deferred != nullptr ? &deferred->gates : nullptr);
+  a.base0 = deferred != nullptr ? deferred->base : 0;
+  a.base0_dev = deferred != nullptr ? deferred->base_device : nullptr;
   return castle::launch_decode(a, dtype, static_cast<hipStream_t>(stream));
 }
 
@@ -315,10 +327,10 @@ int castle_decode_step(const castle_view4* U, const castle_view4* qu_cache,
                        const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
                        const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
                        int B, int H, int d, int dtype, float scale, int flags,
-                       const castle_view4* out,
+                       const castle_view4* out, const castle_deferred* deferred,
                        void* workspace, int64_t workspace_bytes, void* stream) {
   return decode_step_common(U, qu_cache, kc_cache, vc_cache, t, nullptr, capacity, qc, kc, vc, qu, ku, vu,
-                            B, H, d, dtype, scale, flags, out, workspace, workspace_bytes, false, stream);
+                            B, H, d, dtype, scale, flags, out, deferred, workspace, workspace_bytes, false, stream);
 }
 
 int castle_decode_step_static(const castle_view4* U, const castle_view4* qu_cache,
@@ -327,10 +339,10 @@ int castle_decode_step_static(const castle_view4* U, const castle_view4* qu_cach
                               const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
                               const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
                               int B, int H, int d, int dtype, float scale, int flags,
-                              const castle_view4* out, void* stream) {
+                              const castle_view4* out, const castle_deferred* deferred, void* stream) {
   if (t_device != nullptr && reinterpret_cast<uintptr_t>(t_device) % 4 != 0) return CASTLE_ERR_ARG;
   return decode_step_common(U, qu_cache, kc_cache, vc_cache, t_device != nullptr ? 0 : t, t_device, capacity,
-                            qc, kc, vc, qu, ku, vu, B, H, d, dtype, scale, flags, out, nullptr, 0, true, stream);
+                            qc, kc, vc, qu, ku, vu, B, H, d, dtype, scale, flags, out, deferred, nullptr, 0, true, stream);
 }
 
 int castle_decode_step_device_count(const castle_view4* U, const castle_view4* qu_cache,
@@ -339,11 +351,28 @@ int castle_decode_step_device_count(const castle_view4* U, const castle_view4* q
                                     const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
                                     const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
                                     int B, int H, int d, int dtype, float scale, int flags,
-                                    const castle_view4* out,
+                                    const castle_view4* out, const castle_deferred* deferred,
                                     void* workspace, int64_t workspace_bytes, void* stream) {
   if (t_device == nullptr || reinterpret_cast<uintptr_t>(t_device) % 4 != 0) return CASTLE_ERR_ARG;
   return decode_step_common(U, qu_cache, kc_cache, vc_cache, 0, t_device, capacity, qc, kc, vc, qu, ku, vu,
-                            B, H, d, dtype, scale, flags, out, workspace, workspace_bytes, false, stream);
+                            B, H, d, dtype, scale, flags, out, deferred, workspace, workspace_bytes, false, stream);
+}
+
+int castle_decode_flush(const castle_view4* U, const castle_view4* qu_cache, int t, const castle_deferred* deferred,
+                        int B, int H, int d, int dtype, float scale, void* stream) {
+  const int es = elem_size(dtype);
+  if (es == 0) return CASTLE_ERR_DTYPE;
+  if (B <= 0 || H <= 0 || t < 0 || !head_dim_ok(d) || (int64_t)B * H > 65535) return CASTLE_ERR_SHAPE;
+  if (!view_ok(U, es, true) || !view_ok(qu_cache, es, true) || deferred == nullptr) return CASTLE_ERR_ARG;
+  if (!view_ok(&deferred->vu_ring, es, true) || !view_ok(&deferred->gates, 4, false)) return CASTLE_ERR_ARG;
+  if (deferred->base < 0 || deferred->base > t) return CASTLE_ERR_SHAPE;
+  if (t == 0 || castle::decode_base(deferred->base, t) == t) return CASTLE_OK;   // nothing pending
+  castle::DecodeArgs a = {};
+  a.B = B; a.H = H; a.d = d; a.t = t; a.scale = scale;
+  a.U = to_view(U); a.qu_cache = to_view(qu_cache);
+  a.pend_vu = to_view(&deferred->vu_ring); a.pend_gate = to_view(&deferred->gates);
+  a.base0 = deferred->base;
+  return castle::launch_decode_flush(a, dtype, static_cast<hipStream_t>(stream));
 }
 
 int castle_rope(const castle_view4* x, const castle_view4* out, int B, int H, int L, int d, int dtype,

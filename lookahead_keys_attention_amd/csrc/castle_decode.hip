@@ -67,20 +67,64 @@ __global__ __launch_bounds__(kThreads) void decode_stream_kernel(DecodeArgs a) {
     }
   }
 
+  // deferred write-back: the pending tokens' vu pieces of this lane, and whether this step writes U
+  const bool deferred = a.pend_vu.ptr != nullptr;
+  const int base0 = a.base0_dev != nullptr ? *a.base0_dev : a.base0;
+  const int pbase = deferred ? decode_base(base0, t) : t;
+  const int np = t - pbase;                                        // 0 .. kDecodeDefer - 1
+  const bool write_u = !deferred || (t + 1) % kDecodeDefer == 0;
+  float pv[kDecodeDefer][V];   // indexed by ring slot; zero where no pending token sits
+#pragma unroll
+  for (int sl = 0; sl < kDecodeDefer; ++sl) {
+#pragma unroll
+    for (int e = 0; e < V; ++e) pv[sl][e] = 0.f;
+    const int j = pbase + ((sl - pbase % kDecodeDefer + kDecodeDefer) % kDecodeDefer);   // the token that would sit in this slot
+    if (deferred && j < t) load_f32<T, V>(view_row<T>(a.pend_vu, b, h, sl) + sub * V, pv[sl]);
+  }
+  const int slot_t = t % kDecodeDefer;
+
   float acc[V];
 #pragma unroll
   for (int e = 0; e < V; ++e) acc[e] = 0.f;
   float m = -INFINITY, l = 0.f;
 
+  // The row pieces of the NEXT iteration are requested before the current one is processed: twice
+  // the bytes in flight per wave, which is what a latency-bound streaming loop is short of.
+  vt nq, nu, nk, nv;
+  vec<float, 4> ng = {0.f, 0.f, 0.f, 0.f};
+  float* const gbase = deferred ? reinterpret_cast<float*>(a.pend_gate.ptr) + (int64_t)b * a.pend_gate.sb + (int64_t)h * a.pend_gate.sh : nullptr;
+  auto request = [&](int k) __attribute__((always_inline)) {
+    if (k < r1) {
+      nq = *reinterpret_cast<const vt*>(view_row<T>(a.qu_cache, b, h, k) + sub * V);
+      nu = *reinterpret_cast<const vt*>(view_row<T>(a.U, b, h, k) + sub * V);
+      nk = *reinterpret_cast<const vt*>(view_row<T>(a.kc_cache, b, h, k) + sub * V);
+      nv = *reinterpret_cast<const vt*>(view_row<T>(a.vc_cache, b, h, k) + sub * V);
+      if (np > 0) ng = *reinterpret_cast<const vec<float, 4>*>(gbase + (int64_t)k * kDecodeDefer);
+    }
+  };
+  request(r0 + grp);
   for (int base = r0; base < r1; base += RPI) {
     const int k = base + grp;
+    const vt cq = nq, cu = nu, ck = nk, cv = nv;
+    const vec<float, 4> g4 = ng;
+    request(k + RPI);
     if (k < r1) {
       float quk[V], uk[V], kck[V], vck[V];
       T* urow = view_row<T>(a.U, b, h, k) + sub * V;
-      load_f32<T, V>(view_row<T>(a.qu_cache, b, h, k) + sub * V, quk);
-      load_f32<T, V>(urow, uk);
-      load_f32<T, V>(view_row<T>(a.kc_cache, b, h, k) + sub * V, kck);
-      load_f32<T, V>(view_row<T>(a.vc_cache, b, h, k) + sub * V, vck);
+#pragma unroll
+      for (int e = 0; e < V; ++e) { quk[e] = (float)cq[e]; uk[e] = (float)cu[e]; kck[e] = (float)ck[e]; vck[e] = (float)cv[e]; }
+      // pending sources j > k first (none unless the write-back is deferred): their gates were
+      // formed by the steps that appended them and wait in the row's side array
+      float* grow = deferred ? gbase + (int64_t)k * kDecodeDefer : nullptr;
+      if (np > 0) {
+#pragma unroll
+        for (int sl = 0; sl < kDecodeDefer; ++sl) {
+          const int j = pbase + ((sl - pbase % kDecodeDefer + kDecodeDefer) % kDecodeDefer);
+          const float gj = (j < t && j > k) ? g4[sl] : 0.f;   // rows appended inside the window have no gate for earlier tokens
+#pragma unroll
+          for (int e = 0; e < V; ++e) uk[e] = __builtin_fmaf(gj, pv[sl][e], uk[e]);
+        }
+      }
       float dg = 0.f;
 #pragma unroll
       for (int e = 0; e < V; ++e) dg = __builtin_fmaf(quk[e], ku[e], dg);
@@ -88,12 +132,17 @@ __global__ __launch_bounds__(kThreads) void decode_stream_kernel(DecodeArgs a) {
       const float gate = sigmoid_l2(dg * c1);
       vt unew;
 #pragma unroll
-      for (int e = 0; e < V; ++e) unew[e] = (T)__builtin_fmaf(gate, vu[e], uk[e]);
-      *reinterpret_cast<vt*>(urow) = unew;
+      for (int e = 0; e < V; ++e) {
+        uk[e] = __builtin_fmaf(gate, vu[e], uk[e]);
+        unew[e] = (T)uk[e];
+      }
+      if (write_u) *reinterpret_cast<vt*>(urow) = unew;
+      else if (sub == 0) grow[slot_t] = gate;   // the new token stays pending: its gate for this row
       float dsu = 0.f, dsc = 0.f;
 #pragma unroll
       for (int e = 0; e < V; ++e) {
-        dsu = __builtin_fmaf(qc[e], (float)unew[e], dsu);   // the stored (rounded) lookahead key
+        // the lookahead key as later steps will see it: the stored (rounded) one when it is written now
+        dsu = __builtin_fmaf(qc[e], write_u ? (float)unew[e] : uk[e], dsu);
         dsc = __builtin_fmaf(qc[e], kck[e], dsc);
       }
       dsu = group_sum<LPR>(dsu);
@@ -195,6 +244,9 @@ __global__ __launch_bounds__(64) void decode_finish_kernel(DecodeArgs a) {
     }
   }
   const float inv = 1.f / lsum;
+  const bool deferred = a.pend_vu.ptr != nullptr;
+  const T* vu = view_row<T>(a.vu, b, h, 0);
+  T* pvt = deferred ? view_row<T>(a.pend_vu, b, h, t % kDecodeDefer) : nullptr;
   T* out = view_row<T>(a.out, b, h, 0);
   T* Ut = view_row<T>(a.U, b, h, t);
   T* qut = view_row<T>(a.qu_cache, b, h, t);
@@ -220,6 +272,59 @@ __global__ __launch_bounds__(64) void decode_finish_kernel(DecodeArgs a) {
       kct[n] = (T)kcv;
       vct[n] = vc[n];
     }
+    if (deferred) {   // the new token joins the pending sources (rotated like the stream kernel uses it)
+      float vuv = n < HD ? (float)vu[n] : 0.f;
+      if (a.rotary) {
+        const float vup = __shfl_xor(vuv, 1);
+        const bool even = (n & 1) == 0;
+        float v0 = even ? vuv : vup, v1 = even ? vup : vuv;
+        CASTLE_ROPE_PAIR(v0, v1, (float)t, n / 2, HD, false);
+        vuv = even ? v0 : v1;
+      }
+      if (n < HD) pvt[n] = (T)vuv;
+    }
+  }
+}
+
+// Folds the pending sources into the stored lookahead keys (rows 0 .. t-1), for a reader that wants
+// the cache tensor U itself: U_k += sum over pending j > k of sigmoid(s qu_k . ku_j) vu_j.
+template <typename T, int HD>
+__global__ __launch_bounds__(kThreads) void decode_flush_kernel(DecodeArgs a) {
+  constexpr int V = elem_traits<T>::vec16;
+  constexpr int LPR = HD / V;
+  constexpr int RPI = kThreads / LPR;
+  typedef vec<T, V> vt;
+  const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
+  const int t = a.t;
+  const int grp = threadIdx.x / LPR, sub = threadIdx.x % LPR;
+  const float c1 = a.scale * kLog2e;
+  const int pbase = decode_base(a.base0, t);
+  float pv[kDecodeDefer][V];
+#pragma unroll
+  for (int sl = 0; sl < kDecodeDefer; ++sl) {
+#pragma unroll
+    for (int e = 0; e < V; ++e) pv[sl][e] = 0.f;
+    const int j = pbase + ((sl - pbase % kDecodeDefer + kDecodeDefer) % kDecodeDefer);
+    if (j < t) load_f32<T, V>(view_row<T>(a.pend_vu, b, h, sl) + sub * V, pv[sl]);
+  }
+  (void)c1;
+  for (int k = blockIdx.x * RPI + grp; k < t; k += gridDim.x * RPI) {
+    float uk[V];
+    T* urow = view_row<T>(a.U, b, h, k) + sub * V;
+    load_f32<T, V>(urow, uk);
+    const vec<float, 4> g4 = *reinterpret_cast<const vec<float, 4>*>(
+        reinterpret_cast<const float*>(a.pend_gate.ptr) + (int64_t)b * a.pend_gate.sb + (int64_t)h * a.pend_gate.sh + (int64_t)k * kDecodeDefer);
+#pragma unroll
+    for (int sl = 0; sl < kDecodeDefer; ++sl) {
+      const int j = pbase + ((sl - pbase % kDecodeDefer + kDecodeDefer) % kDecodeDefer);
+      const float gj = (j < t && j > k) ? g4[sl] : 0.f;
+#pragma unroll
+      for (int e = 0; e < V; ++e) uk[e] = __builtin_fmaf(gj, pv[sl][e], uk[e]);
+    }
+    vt unew;
+#pragma unroll
+    for (int e = 0; e < V; ++e) unew[e] = (T)uk[e];
+    *reinterpret_cast<vt*>(urow) = unew;
   }
 }
 
@@ -234,6 +339,30 @@ template <typename T, int HD> static int launch_decode_t(const DecodeArgs& a, hi
     hipLaunchKernelGGL((decode_finish_kernel<T, HD>), dim3(BH), dim3(64), 0, stream, a);
   }
   return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+template <typename T> static int launch_flush_d(const DecodeArgs& a, hipStream_t stream) {
+  const int BH = a.B * a.H;
+  int gx = (640 + BH - 1) / BH;
+  if (gx > 64) gx = 64;
+  const dim3 grid(gx, BH), block(kThreads);
+  switch (a.d) {
+    case 16: hipLaunchKernelGGL((decode_flush_kernel<T, 16>), grid, block, 0, stream, a); break;
+    case 32: hipLaunchKernelGGL((decode_flush_kernel<T, 32>), grid, block, 0, stream, a); break;
+    case 64: hipLaunchKernelGGL((decode_flush_kernel<T, 64>), grid, block, 0, stream, a); break;
+    case 128: hipLaunchKernelGGL((decode_flush_kernel<T, 128>), grid, block, 0, stream, a); break;
+    default: return -2;
+  }
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+int launch_decode_flush(const DecodeArgs& a, int dtype, hipStream_t stream) {
+  switch (dtype) {
+    case 0: return launch_flush_d<float>(a, stream);
+    case 1: return launch_flush_d<bf16_t>(a, stream);
+    case 2: return launch_flush_d<fp16_t>(a, stream);
+    default: return -1;
+  }
 }
 
 template <typename T> static int launch_decode_d(const DecodeArgs& a, hipStream_t stream) {

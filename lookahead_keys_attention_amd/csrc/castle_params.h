@@ -79,6 +79,12 @@ struct BwdArgs {
 // size of the per-GPU partial-result array behind castle_decode_step_static
 constexpr int64_t kDecodeStaticScratchBytes = (int64_t)4 << 20;
 
+// Deferred write-back of the lookahead keys: U is written every kDecodeDefer-th step only; in
+// between, the vu rows of the tokens not yet folded into the stored U ("pending") sit in a small
+// ring buffer, the gates they got from every cached row in a per-row fp32 side array, and every step
+// adds gate * vu of the pending tokens on the fly in fp32.
+constexpr int kDecodeDefer = 4;
+
 struct DecodeArgs {
   int B, H, d;
   int t;            // rows already in the cache (used when t_dev is NULL)
@@ -91,6 +97,16 @@ struct DecodeArgs {
   View4 qc, kc, vc, qu, ku, vu;            // new token, L == 1
   View4 out;                               // (B, H, 1, d)
   float* part;      // [B*H][splits][d + 2]  partial (acc, m, l)
+  // deferred write-back (pend_ku.ptr == nullptr: U is written every step)
+  View4 pend_vu;            // (B, H, kDecodeDefer, d): row j % kDecodeDefer holds vu of token j (rotated when rotary)
+  View4 pend_gate;          // (B, H, capacity, kDecodeDefer) fp32: [k][j % kDecodeDefer] = gate of row k for pending token j
+  int base0;                // rows of U are complete up to source base0 - 1 at least (e.g. the prefill length)
+  const int* base0_dev;     // the same from device memory (graph replay): base0_dev[0]
 };
+// first source not yet folded into the stored lookahead keys when the cache holds t rows
+__host__ __device__ inline int decode_base(int base0, int t) {
+  const int b = t - t % kDecodeDefer;
+  return b > base0 ? b : base0;
+}
 
 }  // namespace castle

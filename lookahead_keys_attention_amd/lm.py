@@ -64,13 +64,18 @@ class GraphedDecoder:
         if len(lengths) != 1:
             raise RuntimeError("the layer caches disagree about their length")
         self.length = lengths.pop()
+        for st in stores:
+            st.flush()   # the graph starts from complete lookahead keys
         self.stores = [st if st.capacity >= max_len else st.grown(max_len) for st in stores]
+        self.base0 = self.length
         self.model = model
         device = self.stores[0].buffers[0].device
         batch = self.stores[0].buffers[0].shape[0]
         self.capacity = min(st.capacity for st in self.stores)
         # while warming up and capturing, the count is out of range for every layer: such a step writes nothing
-        self.t_device = torch.full((1,), max(st.capacity for st in self.stores), dtype=torch.int32, device=device)
+        # [row count, row count up to which the stored lookahead keys are complete]
+        self.counters = torch.full((2,), max(st.capacity for st in self.stores), dtype=torch.int32, device=device)
+        self.t_device, self.base_device = self.counters[:1], self.counters[1:]
         self.token = torch.zeros((batch, 1), dtype=torch.long, device=device)
         side = torch.cuda.Stream(device=device)
         side.wait_stream(torch.cuda.current_stream(device))
@@ -82,8 +87,11 @@ class GraphedDecoder:
         with torch.cuda.graph(self.graph), torch.no_grad():
             self.logits = self._step()
             self.t_device += 1
-        self.t_device.fill_(self.length)
+        self._set_counters()
         self.signature = self._signature()
+
+    def _set_counters(self):
+        self.counters.copy_(torch.tensor([self.length, self.base0], dtype=torch.int32), non_blocking=False)
 
     def _signature(self):
         """What the captured graph has baked in: the addresses of the weights it reads."""
@@ -107,16 +115,17 @@ class GraphedDecoder:
         if any(st.length != length for st in stores) or length > self.capacity:
             raise RuntimeError("these caches do not fit the buffers the graph was captured on")
         for mine, theirs in zip(self.stores, stores):
+            theirs.flush()
             for dst, src in zip(mine.buffers, theirs.buffers):
                 dst[:, :, :length].copy_(src[:, :, :length])
-        self.length = length
-        self.t_device.fill_(length)
+        self.length = self.base0 = length
+        self._set_counters()
 
     def _step(self):
         model = self.model
         h = model.token_emb(self.token)
         for (attention, feed_forward), store in zip(model.layers, self.stores):
-            h = h + attention.graph_step(h, store, self.t_device)
+            h = h + attention.graph_step(h, store, self.t_device, self.base_device)
             h = h + feed_forward(h)
         return model.to_logits(model.final_norm(h))
 
@@ -133,7 +142,10 @@ class GraphedDecoder:
     def caches(self):
         """The per-layer caches as they stand after the steps replayed so far."""
         for st in self.stores:
-            st.length = self.length
+            st.length, st.base0 = self.length, self.base0
+            st.flush()   # the lookahead keys complete; the graph's counters must know, or a later replay would add the pending sources twice
+        self.base0 = self.length
+        self._set_counters()
         return [st.as_cache() for st in self.stores]
 
 

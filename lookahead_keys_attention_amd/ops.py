@@ -31,6 +31,9 @@ DEFAULT_FLAGS = 0
 # take at most this many bytes; beyond it they are dropped after the forward pass and the backward
 # pass runs the scan again first (what a call keeps is then O(L d)).  0 = never keep.
 KEEP_STATE_LIMIT_BYTES = 8 << 30
+# The native cached step writes the lookahead keys back on every 4th step only (pending tokens are
+# applied on the fly; see castle_deferred in include/castle_hip.h).  False: every step writes U.
+DEFER_LOOKAHEAD_WRITES = True
 # Debugging aid: when True every parallel forward waits for its kernels and raises if they had to
 # clamp a value to the fp16 range (an input element of a bf16 tensor beyond +-65504, or a T' entry):
 # the result is then that of the clamped operands.  Off by default because it synchronises.
@@ -283,10 +286,12 @@ def decode_workspace(B, H, d, device):
 
 @torch.no_grad()
 def castle_decode_step_hip(U, qu_cache, kc_cache, vc_cache, t, qc, kc, vc, qu, ku, vu, scale, out, workspace,
-                           rotary=False):
+                           rotary=False, deferred=None):
     """In-place cached step.  The four cache tensors are (B,H,capacity,d) buffers with t valid
     rows (capacity > t); the new-token operands and `out` are (B,H,1,d).  rotary=True rotates the
-    new token by position t inside the kernels (the cache rows are stored rotated)."""
+    new token by position t inside the kernels (the cache rows are stored rotated).  `deferred`: a
+    `_native.Deferred` (pending-token buffers and a base row count, `make_deferred`) makes the kernels write the
+    lookahead keys on every 4th step only; `castle_decode_flush` completes them in between."""
     _require_gpu(U, "castle_decode_step_hip")
     B, H, cap, d = U.shape
     if not (0 <= t < cap):
@@ -299,10 +304,28 @@ def castle_decode_step_hip(U, qu_cache, kc_cache, vc_cache, t, qc, kc, vc, qu, k
     tviews = [N.view4(x) for x in toks]
     with torch.cuda.device(U.device):
         rc = N.lib().castle_decode_step(*views, int(t), int(cap), *tviews, B, H, d, code, float(scale),
-                                        N.FLAG_ROTARY if rotary else 0, N.view4(out),
+                                        N.FLAG_ROTARY if rotary else 0, N.view4(out), deferred,
                                         workspace.data_ptr(), workspace.numel(), N.stream_ptr(U.device))
     N.check(rc, "castle_decode_step")
     return out
+
+
+def make_deferred(vu_ring, gates, base, base_device=None):
+    """struct castle_deferred: `vu_ring` (B, H, 4, d) in the cache's element type, `gates`
+    (B, H, capacity, 4) fp32 contiguous; `base_device`: optional int32 GPU tensor whose first
+    element the kernels read instead of `base` (graph replay)."""
+    assert gates.dtype == torch.float32 and gates.is_contiguous() and gates.shape[-1] == N.DECODE_DEFER
+    return N.Deferred(N.view4(vu_ring), N.view4(gates), int(base), base_device.data_ptr() if base_device is not None else None)
+
+
+@torch.no_grad()
+def castle_decode_flush(U, qu_cache, t, deferred, scale):
+    """Folds the pending sources into the stored lookahead keys U[:, :, :t] (see castle_deferred)."""
+    B, H, _, d = U.shape
+    with torch.cuda.device(U.device):
+        rc = N.lib().castle_decode_flush(N.view4(U), N.view4(qu_cache), int(t), deferred, B, H, d, N.dtype_code(U.dtype),
+                                         float(scale), N.stream_ptr(U.device))
+    N.check(rc, "castle_decode_flush")
 
 
 SMALL_LINEAR_MAX_ROWS = 64
@@ -347,7 +370,7 @@ def castle_rope_hip(x, out, first_position=0):
 
 @torch.no_grad()
 def castle_decode_step_packed(cache_views, capacity, t, proj, heads, scale, out, workspace, rotary=False,
-                              t_device=None):
+                              t_device=None, deferred=None):
     """The cached step for a fused projection: `proj` is the contiguous (B, 1, 6*H*d) output of the
     layer's projection for the new token (order qu, ku, vu, qc, kc, vc), `cache_views` the four
     castle_view4 of the (B, H, capacity, d) cache buffers (built once per buffer set), `out` a
@@ -369,14 +392,14 @@ def castle_decode_step_packed(cache_views, capacity, t, proj, heads, scale, out,
             if not (0 <= t < capacity):
                 raise ValueError(f"cache capacity {capacity} cannot take row {t}")
             rc = N.lib().castle_decode_step(*cache_views, int(t), int(capacity), qc, kc, vc, qu, ku, vu, B, heads, d,
-                                            N.dtype_code(proj.dtype), float(scale), flags, vout,
+                                            N.dtype_code(proj.dtype), float(scale), flags, vout, deferred,
                                             workspace.data_ptr(), workspace.numel(), N.stream_ptr(proj.device))
         else:
             if t_device.dtype != torch.int32 or t_device.numel() != 1 or t_device.device != proj.device:
                 raise ValueError("t_device must be a one-element int32 tensor on the GPU of the step")
             rc = N.lib().castle_decode_step_device_count(
                 *cache_views, t_device.data_ptr(), int(capacity), qc, kc, vc, qu, ku, vu, B, heads, d,
-                N.dtype_code(proj.dtype), float(scale), flags, vout,
+                N.dtype_code(proj.dtype), float(scale), flags, vout, deferred,
                 workspace.data_ptr(), workspace.numel(), N.stream_ptr(proj.device))
     N.check(rc, "castle_decode_step")
     return out

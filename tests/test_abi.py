@@ -93,10 +93,10 @@ def test_small_linear_and_static_step_validate_on_the_host(lib):
     assert lib.castle_small_linear(4100, 4096, 4096, 4, 64, 32, 64, 64, 64, 1, None) == -5     # misaligned x
     # castle_decode_step_static: partials beyond the 4 MiB array, and a row beyond the capacity
     v = N.View4(4096, 128, 128, 128)
-    rc = lib.castle_decode_step_static(v, v, v, v, 5, None, 8, v, v, v, v, v, v, 9000, 1, 128, 1, 0.1, 0, v, None)
+    rc = lib.castle_decode_step_static(v, v, v, v, 5, None, 8, v, v, v, v, v, v, 9000, 1, 128, 1, 0.1, 0, v, None, None)
     assert rc == -6 and b"static scratch" in lib.castle_error_string(rc)
-    assert lib.castle_decode_step_static(v, v, v, v, 8, None, 8, v, v, v, v, v, v, 1, 1, 128, 1, 0.1, 0, v, None) == -2
-    assert lib.castle_decode_step(v, v, v, v, 8, 8, v, v, v, v, v, v, 1, 1, 128, 1, 0.1, 0, v, 4096, 1 << 30, None) == -2
+    assert lib.castle_decode_step_static(v, v, v, v, 8, None, 8, v, v, v, v, v, v, 1, 1, 128, 1, 0.1, 0, v, None, None) == -2
+    assert lib.castle_decode_step(v, v, v, v, 8, 8, v, v, v, v, v, v, 1, 1, 128, 1, 0.1, 0, v, None, 4096, 1 << 30, None) == -2
 
 
 def test_check_raises_with_message(lib):

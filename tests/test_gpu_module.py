@@ -101,6 +101,31 @@ def test_decode_from_scratch_and_from_plain_tuple():
             m(x[:, 3:4].to(DEV), cache=c_old)
 
 
+def test_reading_the_lookahead_keys_mid_window_completes_them():
+    """The native step writes U back on every 4th step only.  Whoever reads `cache.U` in between gets
+    the pending tokens folded in first (so the tensor seen is always the true U), and the steps that
+    follow carry on from there: outputs and keys equal the oracle's, whether U was read or not."""
+    m = make(64, 2, 32).eval()
+    p = cpu_params(m)
+    x = torch.randn(2, 14, 64, generator=torch.Generator().manual_seed(6))
+    ref = O.module_forward(x, p, 2)
+    for read_at in ((), (6, 7, 9), (5,)):
+        with torch.no_grad():
+            _, cache = m(x[:, :3].to(DEV), return_next_cache=True)
+            ys = []
+            for t in range(3, 14):
+                y, cache = m(x[:, t:t + 1].to(DEV), cache=cache)
+                ys.append(y)
+                if t in read_at:
+                    _, oc = O.module_forward(x[:, :t + 1], p, 2, return_next_cache=True)
+                    assert (cache.U.cpu() - oc.U).abs().max() <= 1e-3, f"U read after step {t}"
+                    assert cache._store.pending() == 0
+            assert (torch.cat(ys, 1).cpu() - ref[:, 3:]).abs().max() <= 1e-3
+            _, oc = O.module_forward(x, p, 2, return_next_cache=True)
+            U, qu_c, kc_c, vc_c = cache            # unpacking reads U too
+            assert (U.cpu() - oc.U).abs().max() <= 1e-3 and (kc_c.cpu() - oc.kc_cache).abs().max() <= 1e-5
+
+
 def test_multi_token_with_cache_is_rejected():
     m = make(32, 2, 16)
     x = torch.randn(1, 4, 32).to(DEV)
@@ -211,10 +236,12 @@ def test_config4_bf16_decode_after_prefill():
     decode_core iterated in fp32 on that head from the oracle's own prefill, and so are the head's
     lookahead keys in the cache after the last step.  The cache is a bf16 tensor in this
     configuration, as in the reference, whose step forms `U = U_prev + gate * vu` in the module
-    dtype (lookahead_keys_attention.py:183): the oracle's lookahead keys are therefore rounded to
-    bf16 after every step, like any other bf16 input of the next step.  Against a cache kept in
-    fp32 the 512 roundings show: the last step differs from the parallel pass (fp32 state) by about
-    5e-2 normwise, which is asserted as a bound here and is a property of a bf16 cache."""
+    dtype (lookahead_keys_attention.py:183).  The native step writes the lookahead keys back on every
+    4th step (row counts with (t + 1) % 4 == 0) and carries them in fp32 in between, so the oracle's
+    keys are rounded to bf16 at exactly those steps, like any other bf16 input of the next step.
+    Against a cache kept in fp32 the 128 roundings show: the last step differs from the parallel
+    pass (fp32 state) by about 2.4e-2 normwise (4.9e-2 when every step writes), asserted as a
+    bound here; it is a property of a bf16 cache."""
     m = make(512, 8, 64, dtype=torch.bfloat16, seed=0).eval()
     g = torch.Generator().manual_seed(0)
     steps, t0 = 512, 2048
@@ -235,7 +262,7 @@ def test_config4_bf16_decode_after_prefill():
     assert cache.U.shape == (32, 8, t0 + steps, 64)
     last = m.combine_heads(merged)[:, 0].double().cpu()
     drift = ((last - full_last.double().cpu()).norm() / full_last.double().norm()).item()
-    assert drift <= 1e-1, f"last cached step vs parallel: {drift:.3e}"
+    assert drift <= 5e-2, f"last cached step vs parallel: {drift:.3e}"
     for b, h in heads:
         qu, ku, vu, qc, kc, vc = [proj_all[b, :, i, h].float().cpu() for i in range(6)]
         _, U0 = O.parallel_core(*[t[:t0] for t in (qc, kc, vc, qu, ku, vu)], m.scale, want_U=True)
@@ -243,7 +270,8 @@ def test_config4_bf16_decode_after_prefill():
         for n in range(1, steps + 1):
             t = t0 + n - 1
             out, state = O.decode_core(state, *[z[t:t + 1] for z in (qc, kc, vc, qu, ku, vu)], m.scale)
-            state = state._replace(U=state.U.bfloat16().float())
+            if (t + 1) % 4 == 0:
+                state = state._replace(U=state.U.bfloat16().float())
             if n in watch:
                 bf16_close(native[n][b, h], out[0], f"decode step {n} of head ({b},{h}) vs oracle")
         # 512 independent roundings to bf16 on either side: single elements wander by a few ulps, so the

@@ -383,3 +383,59 @@ def test_small_linear_matches_fp64_matmul(M, N, K, dtype):
     assert y.shape == (M, 1, N) and y.dtype == dtype
     err = (y[:, 0].cpu().double() - ref).abs().max().item()
     assert err <= 2.0 ** (-8 if dtype == torch.bfloat16 else -11) * ref.abs().max().item() * 1.01 + 1e-6   # one rounding of the result
+
+
+@pytest.mark.parametrize("B,Hh,t0,steps,d,dtype,rotary", [(2, 2, 0, 23, 64, torch.float32, False), (1, 2, 101, 18, 32, torch.float32, True),
+                                                        (2, 2, 203, 21, 64, torch.bfloat16, False), (1, 2, 130, 9, 128, torch.bfloat16, True)])
+def test_decode_with_deferred_write_back(B, Hh, t0, steps, d, dtype, rotary):
+    """castle_deferred: the lookahead keys are written on every 4th step only, the tokens in between
+    are kept as pending vu rows plus their per-row gates and applied on the fly.  Every step's output equals the
+    oracle's; after castle_decode_flush the stored U is the oracle's; the steps in between leave U
+    untouched (that is where the traffic is saved); and at a step that does write, the U rows equal
+    what the step-by-step mode holds."""
+    from lookahead_keys_attention_amd import _native as N
+
+    L = t0 + steps
+    ops, _ = rand_ops(B, Hh, L, d, dtype, seed=7 * L + d)
+    s = d ** -0.5
+    pos = torch.arange(L)
+    ref = [t.double() if (idx == 2 or not rotary) else O.rope(t.double(), pos) for idx, t in enumerate(ops)]
+    ref_out, ref_U = O.parallel_core(*ref, s, want_U=True)
+
+    def fresh():
+        bufs = [torch.zeros(B, Hh, L + 3, d, dtype=dtype, device=DEV) for _ in range(4)]
+        if t0:
+            _, U0 = O.parallel_core(*[t[:, :, :t0] for t in ref], s, want_U=True)
+            for buf, src in zip(bufs, (U0, ref[3][:, :, :t0], ref[1][:, :, :t0], ref[2][:, :, :t0])):
+                buf[:, :, :t0] = src.to(dtype).to(DEV)
+        return bufs
+
+    bufs, plain = fresh(), fresh()
+    rings = [torch.zeros(B, Hh, N.DECODE_DEFER, d, dtype=dtype, device=DEV),
+             torch.zeros(B, Hh, L + 3, N.DECODE_DEFER, dtype=torch.float32, device=DEV)]
+    ws = H().decode_workspace(B, Hh, d, DEV)
+    dev_ops = [t.to(DEV) for t in ops]
+    outs, wrote = [], 0
+    for t in range(t0, L):
+        tok = [x[:, :, t:t + 1] for x in dev_ops]
+        before = bufs[0][:, :, :t].clone()
+        o = torch.empty(B, Hh, 1, d, dtype=dtype, device=DEV)
+        H().castle_decode_step_hip(*bufs, t, *tok, s, o, ws, rotary=rotary, deferred=H().make_deferred(*rings, t0))
+        H().castle_decode_step_hip(*plain, t, *tok, s, torch.empty_like(o), ws, rotary=rotary)
+        outs.append(o)
+        if (t + 1) % N.DECODE_DEFER == 0:
+            wrote += 1
+            if dtype == torch.float32:
+                assert_close(bufs[0][:, :, :t + 1], plain[0][:, :, :t + 1].cpu(), dtype, f"U at writing step {t}", 1e-5)
+        elif t > 0:
+            assert torch.equal(bufs[0][:, :, :t], before), f"step {t} wrote lookahead keys"
+    assert wrote >= 2
+    got = torch.cat(outs, 2)
+    assert_close(got, ref_out[:, :, t0:], dtype, "decode out", 1e-3)
+    H().castle_decode_flush(bufs[0], bufs[1], L, H().make_deferred(*rings, t0), s)
+    if dtype == torch.float32:
+        assert_close(bufs[0][:, :, :L], ref_U, dtype, "U after the flush", 1e-3)
+    else:   # fewer roundings than the step-by-step mode: closer to the fp64 keys
+        err_def = (bufs[0][:, :, :L].cpu().double() - ref_U).norm()
+        err_plain = (plain[0][:, :, :L].cpu().double() - ref_U).norm()
+        assert err_def <= 1.05 * err_plain

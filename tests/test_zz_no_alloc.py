@@ -33,11 +33,11 @@ def _step(lib, N, static, caches, toks, t, cap, dtype, t_device=None):
     stream = N.stream_ptr(torch.device(DEV))
     if static:
         td = t_device.data_ptr() if t_device is not None else None
-        rc = lib.castle_decode_step_static(*cviews, int(t), td, int(cap), *tviews, B, H, d, code, scale, 0, N.view4(out), stream)
+        rc = lib.castle_decode_step_static(*cviews, int(t), td, int(cap), *tviews, B, H, d, code, scale, 0, N.view4(out), None, stream)
     else:
         nbytes = lib.castle_decode_workspace_bytes(B, H, d, cap)
         ws = torch.empty(nbytes, dtype=torch.uint8, device=DEV)
-        rc = lib.castle_decode_step(*cviews, int(t), int(cap), *tviews, B, H, d, code, scale, 0, N.view4(out),
+        rc = lib.castle_decode_step(*cviews, int(t), int(cap), *tviews, B, H, d, code, scale, 0, N.view4(out), None,
                                     ws.data_ptr(), nbytes, stream)
     assert rc == 0, lib.castle_error_string(rc)
     torch.cuda.synchronize()
@@ -73,9 +73,9 @@ def test_static_scratch_step_rejects_what_does_not_fit():
     lib = N.lib()
     # B*H = 9000 heads at d = 128: 9000 * 130 * 4 bytes of partials > 4 MiB; nothing is launched
     v = N.View4(4096, 128, 128, 128)
-    rc = lib.castle_decode_step_static(v, v, v, v, 5, None, 8, v, v, v, v, v, v, 9000, 1, 128, 1, 0.1, 0, v, None)
+    rc = lib.castle_decode_step_static(v, v, v, v, 5, None, 8, v, v, v, v, v, v, 9000, 1, 128, 1, 0.1, 0, v, None, None)
     assert rc == -6
     assert b"static scratch" in lib.castle_error_string(rc)
     # row t must fit the buffers, as in castle_decode_step
-    rc = lib.castle_decode_step_static(v, v, v, v, 8, None, 8, v, v, v, v, v, v, 1, 1, 128, 1, 0.1, 0, v, None)
+    rc = lib.castle_decode_step_static(v, v, v, v, 8, None, 8, v, v, v, v, v, v, 1, 1, 128, 1, 0.1, 0, v, None, None)
     assert rc == -2
