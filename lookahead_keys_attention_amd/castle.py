@@ -29,6 +29,8 @@ from __future__ import annotations
 
 from collections import namedtuple
 
+import warnings
+
 import torch
 import torch.nn.functional as F
 from torch import nn
@@ -178,6 +180,12 @@ class Castle(nn.Module):
         self._explicit_native = use_triton is True
         if use_triton is None:
             use_triton = torch.cuda.is_available() and _native.is_built()
+            if torch.cuda.is_available() and not use_triton:
+                # the reference falls back silently when Triton is missing (lookahead_keys_attention.py:58);
+                # here a GPU without the kernel library is almost certainly a build problem, so say so
+                warnings.warn("libcastle_hip.so is not built: Castle(use_triton=None) uses the dense PyTorch "
+                              "formulation (python -m lookahead_keys_attention_amd.build builds the kernels)",
+                              RuntimeWarning, stacklevel=2)
         if use_triton and not _native.is_built():
             raise AssertionError(
                 "native kernels requested but libcastle_hip.so is not built "
