@@ -45,6 +45,14 @@ def top_k(logits: torch.Tensor, thres: float = 0.9) -> torch.Tensor:
     return torch.full_like(logits, float("-inf")).scatter_(-1, index, values)
 
 
+def token_feed_forward(feed_forward: nn.Sequential, h: torch.Tensor) -> torch.Tensor:
+    """The feed-forward block [norm, linear, GELU, linear] for a single-token step (inference): the
+    two bias-free projections have `batch` rows, so they go through `ops.small_linear` when it can
+    take them (16-bit GPU tensors) and through the layers themselves otherwise."""
+    norm, up, act, down = feed_forward
+    return Castle._project(down, act(Castle._project(up, norm(h), True)), True)
+
+
 class GraphedDecoder:
     """One captured HIP graph of a whole single-token step of a `CastleLM` on the native path.
 
@@ -126,8 +134,8 @@ class GraphedDecoder:
         h = model.token_emb(self.token)
         for (attention, feed_forward), store in zip(model.layers, self.stores):
             h = h + attention.graph_step(h, store, self.t_device, self.base_device)
-            h = h + feed_forward(h)
-        return model.to_logits(model.final_norm(h))
+            h = h + token_feed_forward(feed_forward, h)
+        return Castle._project(model.to_logits, model.final_norm(h), True)
 
     def step(self, token):
         """Feeds `token` (batch, 1) and returns the logits (batch, 1, num_tokens) of the next
@@ -178,6 +186,8 @@ class CastleLM(nn.Module):
         if return_loss:
             x, target = x[:, :-1], x[:, 1:]
         h = self.token_emb(x)
+        # one token per sequence, no graph to record: the few rows of every projection go through the small-M kernel
+        token_step = h.shape[1] == 1 and h.is_cuda and not torch.is_grad_enabled()
         next_cache = []
         for index, (attention, feed_forward) in enumerate(self.layers):
             layer_cache = cache[index] if cache is not None and index < len(cache) else None
@@ -187,8 +197,8 @@ class CastleLM(nn.Module):
             else:
                 attended = attention(h, cache=layer_cache, return_next_cache=False)
             h = h + attended
-            h = h + feed_forward(h)
-        logits = self.to_logits(self.final_norm(h))
+            h = h + (token_feed_forward(feed_forward, h) if token_step else feed_forward(h))
+        logits = Castle._project(self.to_logits, self.final_norm(h), token_step)
         if return_loss:
             return F.cross_entropy(logits.transpose(1, 2), target)
         return (logits, next_cache) if return_next_cache else logits
