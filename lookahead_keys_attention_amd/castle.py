@@ -224,6 +224,8 @@ class Castle(nn.Module):
                 raise RuntimeError("Castle(use_triton=True) runs HIP kernels and needs GPU tensors; "
                                    "construct with use_triton=False for the PyTorch formulation")
             native = False   # auto-selected kernels, CPU tensors: the dense formulation (lookahead_keys_attention.py:120)
+        if native and not self._explicit_native and not ops.kernels_support(self.dim_head, x.dtype):
+            native = False   # auto-selected kernels that do not cover this head dimension / type: dense as well
         if single and native and torch.is_grad_enabled() and (
                 x.requires_grad or any(p.requires_grad for p in self.parameters())):
             native = False   # the native step records no autograd graph; the dense step does

@@ -45,6 +45,13 @@ def _require_gpu(t: torch.Tensor, what: str):
         raise RuntimeError(f"{what}: the HIP kernels need tensors on the GPU (got {t.device})")
 
 
+def kernels_support(d: int, dtype: torch.dtype) -> bool:
+    """True if the HIP kernels cover this head dimension and tensor type."""
+    if d not in N.SUPPORTED_HEAD_DIMS or dtype not in (torch.float32, torch.bfloat16, torch.float16):
+        return False
+    return not (dtype == torch.float32 and d > 64)
+
+
 def _check_dims(d: int, dtype: torch.dtype):
     if d not in N.SUPPORTED_HEAD_DIMS:
         raise ValueError(f"dim_head must be one of {N.SUPPORTED_HEAD_DIMS} for the HIP kernels, got {d}")

@@ -134,6 +134,30 @@ def test_multi_token_with_cache_is_rejected():
         m(x, cache=cache)
 
 
+def test_auto_selected_kernels_leave_uncovered_shapes_to_the_dense_path():
+    """use_triton=None (the reference's default, lookahead_keys_attention.py:58) picks the kernels where
+    they apply and the PyTorch formulation elsewhere: a head dimension or tensor type the kernels do
+    not cover still runs (forward, backward, cached steps == parallel), while an explicit
+    use_triton=True on the same module raises."""
+    from lookahead_keys_attention_amd import Castle
+
+    torch.manual_seed(3)
+    for d, dtype in ((48, torch.float32), (128, torch.float32), (32, torch.float64)):
+        m = Castle(64, heads=2, dim_head=d, use_triton=None).to(DEV).to(dtype)
+        assert m.use_triton   # the kernels are built and a GPU is there; this shape is simply not theirs
+        x = torch.randn(2, 9, 64, device=DEV, dtype=dtype, requires_grad=True)
+        y, cache = m(x, return_next_cache=True)
+        y.sum().backward()
+        assert torch.isfinite(x.grad).all()
+        with torch.no_grad():
+            full = m(torch.cat([x.detach(), x.detach()[:, :1]], dim=1))
+            step, _ = m(x.detach()[:, :1], cache=cache)
+        assert torch.allclose(step[:, 0], full[:, -1], atol=1e-4)
+        explicit = Castle(64, heads=2, dim_head=d, use_triton=True).to(DEV).to(dtype)
+        with pytest.raises((ValueError, TypeError, RuntimeError)):
+            explicit(x.detach())
+
+
 def test_config1_readme_fp32_parallel_vs_sequential():
     # benchmark configuration 1: Castle(512, 8, 64), x (2,128,512) fp32, parallel vs 128 cached steps, atol 1e-3
     m = make(512, 8, 64, seed=0).eval()
