@@ -1347,8 +1347,9 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
       const bool live = k0 <= i0w;   // the chunk's keys do not lie beyond this wave's rows
       // gate tile A[k rows, j lanes] for this wave's 32 source rows, shared as A^T[j][k]
       acc_t aK;
-      zero(aK);
+      zero(aK);   // a constant operand of the first product where the chunk is live, registers of zeros where it is not
       if (live) {
+        zero(aK);
 #pragma unroll
         for (int s0 = 0; s0 < KS; s0 += 4) {   // operand fragments in batches of four
           frag<T> oqu[4];
@@ -1384,11 +1385,14 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
         for (int half = 0; half < 2; ++half) {   // two batches keep the operand fragments in registers
           frag<T> ods[PS / 2];
 #pragma unroll
-          for (int u = 0; u < PS / 2; ++u) ods[u] = ld_nat<T>(s_dsu, LDD, c, 16 * (half * (PS / 2) + u) + 8 * g);
+          for (int u = 0; u < PS / 2; ++u) ods[u] = ld_nat<T>(s_dsu, LDD, c, 16 * (PS - 1 - (half * (PS / 2) + u)) + 8 * g);
           __builtin_amdgcn_sched_barrier(0);
+          // steps from the last one down: the last two run for every wave, so the product that starts
+          // dA is unconditional and takes the zero as a constant operand
 #pragma unroll
           for (int u = 0; u < PS / 2; ++u) {
-            if (half * (PS / 2) + u >= sfirst) mma(dA, ods[u], ftt[NREG == 1 ? 0 : half * (PS / 2) + u]);
+            const int step = PS - 1 - (half * (PS / 2) + u);
+            if (step >= PS - 2 || step >= sfirst) mma(dA, ods[u], ftt[NREG == 1 ? 0 : step]);
             if (half == 0 && u < KS) mma(dA2, og[u], fvu[NVU == 1 ? 0 : u]);   // og is zero where no reverse state exists
           }
         }

@@ -407,14 +407,16 @@ __global__ __launch_bounds__(kThreads, (sizeof(T) == 2 && HD <= 64) ? 2 : 1) voi
         zero(su);
 #pragma unroll
         for (int s = 0; s < KS; ++s) mma(sc, ld_nat<T>(s_kc, LDK, 32 * kt + c, 16 * s + 8 * g), fqc[s]);
+        // the in-block term first: its first two steps run for every wave, so the product that
+        // starts the accumulator is unconditional and takes the zero as a constant operand
+#pragma unroll
+        for (int s = 0; s < kNB / 16; ++s)
+          if (s < 2 || s < nintra) mma(su, ld_nat<T>(s_a, LDA, 32 * kt + c, cb + 16 * s + 8 * g), ft[s]);
         if (Kb < Iw) {
           const T* ub = s_ub0 + (Iw - Ifirst) * kNB * LDK;
 #pragma unroll
           for (int s = 0; s < KS; ++s) mma(su, ld_nat<T>(ub, LDK, 32 * kt + c, 16 * s + 8 * g), fqc[s]);
         }
-#pragma unroll
-        for (int s = 0; s < kNB / 16; ++s)
-          if (s < nintra) mma(su, ld_nat<T>(s_a, LDA, 32 * kt + c, cb + 16 * s + 8 * g), ft[s]);
 
         // scores in log2 units: x = Sc' - Su' * sigmoid(Su)
         float mx = -INFINITY;
