@@ -183,10 +183,15 @@ def _attention_setup(ctx, inputs, output):
     ctx.save_for_backward(q, k, v, qu, ku, vu, out, ws, state)
     ctx.scale, ctx.flags = scale, flags
     ctx.mark_non_differentiable(U, ws, state)   # U carries no gradient (lookahead_keys_attention_triton.py:513-515)
+    # without this autograd hands the backward formula zero tensors for the unused outputs: a fill of
+    # the whole workspace and state buffers (hundreds of MB) on every backward pass
+    ctx.set_materialize_grads(False)
 
 
 def _attention_backward(ctx, dout, dU, dws, dstate):
     q, k, v, qu, ku, vu, out, ws, state = ctx.saved_tensors
+    if dout is None:
+        dout = torch.zeros_like(out)
     grads = torch.ops.castle_hip.attention_bwd(q, k, v, qu, ku, vu, out, dout, ws, state, ctx.scale, ctx.flags)
     return (*grads.unbind(0), None, None, None)
 
@@ -257,10 +262,13 @@ def _packed_setup(ctx, inputs, output):
     ctx.save_for_backward(proj, merged, ws, state)
     ctx.heads, ctx.scale, ctx.flags = heads, scale, flags
     ctx.mark_non_differentiable(U, ws, state)
+    ctx.set_materialize_grads(False)   # see _attention_setup
 
 
 def _packed_backward(ctx, dmerged, dU, dws, dstate):
     proj, merged, ws, state = ctx.saved_tensors
+    if dmerged is None:
+        dmerged = torch.zeros_like(merged)
     dproj = torch.ops.castle_hip.attention_packed_bwd(proj, merged, dmerged, ws, state, ctx.heads, ctx.scale, ctx.flags)
     return dproj, None, None, None, None, None
 
