@@ -215,6 +215,21 @@ int castle_rope(const castle_view4* x, const castle_view4* out, int B, int H, in
 int castle_small_linear(const void* x, const void* w, void* y, int M, int N, int K,
                         int64_t ldx, int64_t ldw, int64_t ldy, int dtype, void* stream);
 
+/* The same product with the per-row work of a transformer block's token step folded in (each saves a
+ * launch and a pass over the activations; no counterpart in the reference, whose callers run these as
+ * separate modules: train_triton.py:102-107, 161-165 around lookahead_keys_attention.py:95, 99, 209):
+ *   norm_weight != NULL: RMS normalisation of the x rows in front, y = ((x / sqrt(mean(x^2) + eps)) * norm_weight) w^T
+ *                        (nn.RMSNorm; K elements, 16-byte aligned);
+ *   activation:          CASTLE_ACT_GELU applies the erf form of GELU to the product;
+ *   residual != NULL:    a (M, N) tensor with leading dimension ldr added last (may alias y).
+ * Order: normalise, multiply, activate, add. */
+#define CASTLE_ACT_NONE 0
+#define CASTLE_ACT_GELU 1
+int castle_small_linear_fused(const void* x, const void* w, void* y, int M, int N, int K,
+                              int64_t ldx, int64_t ldw, int64_t ldy, int dtype,
+                              const void* norm_weight, float eps, int activation,
+                              const void* residual, int64_t ldr, void* stream);
+
 /* Per-kernel timing (no counterpart in the reference; for benchmarks).  While enabled, every
  * kernel launched by the entry points above is bracketed by a HIP event pair on its stream.
  * castle_profile_enable(on) also discards pending records.  castle_profile_read waits for the

@@ -37,6 +37,7 @@ EXPORTED_SYMBOLS = (
     "castle_decode_flush",
     "castle_rope",
     "castle_small_linear",
+    "castle_small_linear_fused",
     "castle_profile_enable",
     "castle_profile_read",
 )
@@ -103,6 +104,8 @@ def _declare(lib):
     lib.castle_decode_step_device_count.argtypes = [_VP] * 4 + [vp, i] + [_VP] * 6 + [i, i, i, i, f, i, _VP, _DP, vp, i64, vp]
     lib.castle_small_linear.restype = i
     lib.castle_small_linear.argtypes = [vp, vp, vp, i, i, i, i64, i64, i64, i, vp]
+    lib.castle_small_linear_fused.restype = i
+    lib.castle_small_linear_fused.argtypes = [vp, vp, vp, i, i, i, i64, i64, i64, i, vp, ctypes.c_float, i, vp, i64, vp]
     lib.castle_rope.restype = i
     lib.castle_rope.argtypes = [_VP, _VP, i, i, i, i, i, i, vp]
 

@@ -230,7 +230,7 @@ class Castle(nn.Module):
                 x.requires_grad or any(p.requires_grad for p in self.parameters())):
             native = False   # the native step records no autograd graph; the dense step does
         native_step = single and native
-        proj = self._project(self.to_all_qkv, self.norm(x), native_step)
+        proj = self._project(self.to_all_qkv, x, native_step, norm=self.norm)
         if not single:
             assert cache is None, "must be inferencing single tokens if receiving cache"
             merged, next_cache = (self._parallel_native if native else self._parallel_dense)(proj, return_next_cache)
@@ -240,12 +240,19 @@ class Castle(nn.Module):
         return (y, next_cache) if return_next_cache else y
 
     @staticmethod
-    def _project(layer, t, native_step):
-        """The bias-free projections; on the native single-token step the few rows go through the
-        library's own small-M kernel instead of a general GEMM (inference only)."""
-        if native_step and ops.small_linear_ok(t, layer.weight):
-            return ops.small_linear(t, layer.weight)
-        return layer(t)
+    def _project(layer, t, native_step, norm=None, activation=None, residual=None):
+        """A bias-free projection with what surrounds it in a block: `norm` (an nn.RMSNorm or
+        nn.Identity) in front, GELU (`activation="gelu"`) and a residual behind.  On the native
+        single-token step the few rows go through the library's own small-M kernel, which does all
+        of it in one launch (inference only); otherwise the layers themselves run."""
+        if isinstance(norm, nn.Identity):
+            norm = None
+        if native_step and ops.small_linear_ok(t, layer.weight) and (norm is None or isinstance(norm, nn.RMSNorm)):
+            return ops.small_linear(t, layer.weight, norm=norm, activation=activation, residual=residual)
+        y = layer(t if norm is None else norm(t))
+        if activation == "gelu":
+            y = F.gelu(y)
+        return y if residual is None else residual + y
 
     # -- native HIP paths ---------------------------------------------------
     def _parallel_native(self, proj, want_cache):
@@ -304,21 +311,22 @@ class Castle(nn.Module):
         store.length = t + 1
         return out.view(B, 1, H * d), store.as_cache()
 
-    def graph_step(self, x, store, t_device, base_device=None):
+    def graph_step(self, x, store, t_device, base_device=None, residual=None):
         """The cached single-token step in the form a captured HIP graph needs: the same GPU work
         as forward(x, cache) on the native path, but the row count is read by the kernels from the
         one-element int32 GPU tensor `t_device`, and nothing on the host depends on it (no cache
         object is built, `store.length` is left alone: the owner of the graph keeps the count).
         `base_device` (one-element int32 GPU tensor: the row count up to which the stored lookahead
         keys are complete, e.g. the prefill length) switches the deferred write-back on.
-        x: (B, 1, dim); store: the `_CacheStore` behind a native cache.  Returns (B, 1, dim)."""
+        x: (B, 1, dim); store: the `_CacheStore` behind a native cache.  Returns (B, 1, dim), plus
+        `residual` when one is given (added inside the output projection's launch)."""
         B = x.shape[0]
-        proj = self._project(self.to_all_qkv, self.norm(x), True)
+        proj = self._project(self.to_all_qkv, x, True, norm=self.norm)
         out = torch.empty((B, 1, self.heads, self.dim_head), dtype=proj.dtype, device=proj.device)
         ops.castle_decode_step_packed(store.views, store.capacity, 0, proj, self.heads, self.scale, out,
                                       store.workspace, rotary=self.use_rotary, t_device=t_device,
                                       deferred=store.deferred(base_device) if base_device is not None else None)
-        return self._project(self.combine_heads, out.view(B, 1, self.heads * self.dim_head), True)
+        return self._project(self.combine_heads, out.view(B, 1, self.heads * self.dim_head), True, residual=residual)
 
     # -- dense PyTorch formulation (use_triton=False) -------------------------
     def _parallel_dense(self, proj, want_cache):

@@ -19,7 +19,7 @@ int launch_rope(const View4& src, const View4& dst, int B, int H, int L, int d, 
 int decode_pick_splits(int BH, int t);
 int decode_static_scratch(float** ptr);
 int launch_small_linear(const void* x, const void* w, void* y, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldy,
-                        int dtype, hipStream_t stream);
+                        int dtype, const void* norm_w, float eps, int act, const void* res, int64_t ldr, hipStream_t stream);
 }  // namespace castle
 
 namespace {
@@ -384,15 +384,26 @@ int castle_rope(const castle_view4* x, const castle_view4* out, int B, int H, in
   return castle::launch_rope(to_view(x), to_view(out), B, H, L, d, dtype, first_position, static_cast<hipStream_t>(stream));
 }
 
-int castle_small_linear(const void* x, const void* w, void* y, int M, int N, int K,
-                        int64_t ldx, int64_t ldw, int64_t ldy, int dtype, void* stream) {
+int castle_small_linear_fused(const void* x, const void* w, void* y, int M, int N, int K,
+                              int64_t ldx, int64_t ldw, int64_t ldy, int dtype,
+                              const void* norm_weight, float eps, int activation,
+                              const void* residual, int64_t ldr, void* stream) {
   if (dtype != CASTLE_BF16 && dtype != CASTLE_F16) return CASTLE_ERR_DTYPE;
   if (M <= 0 || N <= 0 || K <= 0 || K % 8 != 0 || N % 2 != 0) return CASTLE_ERR_SHAPE;
   if (x == nullptr || w == nullptr || y == nullptr) return CASTLE_ERR_ARG;
   if (reinterpret_cast<uintptr_t>(x) % 16 != 0 || reinterpret_cast<uintptr_t>(w) % 16 != 0 ||
       reinterpret_cast<uintptr_t>(y) % 4 != 0 || ldx % 8 != 0 || ldw % 8 != 0 || ldy % 2 != 0)
     return CASTLE_ERR_ARG;
-  return castle::launch_small_linear(x, w, y, M, N, K, ldx, ldw, ldy, dtype, static_cast<hipStream_t>(stream));
+  if (activation != CASTLE_ACT_NONE && activation != CASTLE_ACT_GELU) return CASTLE_ERR_ARG;
+  if (norm_weight != nullptr && (reinterpret_cast<uintptr_t>(norm_weight) % 16 != 0 || !(eps >= 0.f))) return CASTLE_ERR_ARG;
+  if (residual != nullptr && (reinterpret_cast<uintptr_t>(residual) % 4 != 0 || ldr % 2 != 0)) return CASTLE_ERR_ARG;
+  return castle::launch_small_linear(x, w, y, M, N, K, ldx, ldw, ldy, dtype, norm_weight, eps, activation, residual, ldr,
+                                     static_cast<hipStream_t>(stream));
+}
+
+int castle_small_linear(const void* x, const void* w, void* y, int M, int N, int K,
+                        int64_t ldx, int64_t ldw, int64_t ldy, int dtype, void* stream) {
+  return castle_small_linear_fused(x, w, y, M, N, K, ldx, ldw, ldy, dtype, nullptr, 0.f, CASTLE_ACT_NONE, nullptr, 0, stream);
 }
 
 int castle_profile_enable(int on) { return castle::profile_enable(on); }

@@ -431,12 +431,21 @@ int launch_rope(const View4& src, const View4& dst, int B, int H, int L, int d, 
 // its operand loads at once (straight from global memory, rows of x and w are K-contiguous, which is
 // the MFMA operand layout), runs a handful of MFMAs and the partial tiles are summed through LDS.
 constexpr int kLinWaves = 8;
+// Optional work around the product (all of it per output row, so it costs one pass less each):
+//   norm_w   RMS normalisation of the x rows in front: y = ((x / rms(x)) * norm_w) w^T.  The weight
+//            goes into the operand, the 1 / rms factor (a per-row scalar) onto the accumulated sum;
+//            the sums of squares are collected from the fragments the product loads anyway.
+//   act      1: GELU (erf form) of the sum
+//   res      a tensor of the output's shape added at the end
 template <typename T>
 __global__ __launch_bounds__(64 * kLinWaves) void small_linear_kernel(const T* x, const T* w, T* y, int M, int N, int K,
-                                                                       int64_t ldx, int64_t ldw, int64_t ldy) {
+                                                                       int64_t ldx, int64_t ldw, int64_t ldy,
+                                                                       const T* norm_w, float eps, int act,
+                                                                       const T* res, int64_t ldr) {
   static_assert(sizeof(T) == 2, "16-bit operands");
   constexpr int MAXS = 8;   // 16-deep steps a wave handles per pass
   __shared__ float red[kLinWaves][32][33];
+  __shared__ float ssq[kLinWaves][32];
   const int lane = lane_id(), wave = wave_id(), c = lane & 31, g = lane >> 5;
   const int n0 = blockIdx.x * 32, m0 = blockIdx.y * 32;
   const int steps = (K + 15) / 16;
@@ -446,6 +455,7 @@ __global__ __launch_bounds__(64 * kLinWaves) void small_linear_kernel(const T* x
   const T* wr = w + (int64_t)(n0 + c) * ldw;
   acc_t acc;
   zero(acc);
+  float sq = 0.f;
   for (int s0 = wave * per; s0 < min(steps, (wave + 1) * per); s0 += MAXS) {
     frag<T> fa[MAXS], fb[MAXS];
 #pragma unroll
@@ -454,38 +464,70 @@ __global__ __launch_bounds__(64 * kLinWaves) void small_linear_kernel(const T* x
       const bool in = s0 + u < min(steps, (wave + 1) * per) && kk < K;   // K is a multiple of 8
       fa[u] = (in && row_ok) ? *reinterpret_cast<const frag_mem<T>*>(xr + kk) : zero_frag<T>();
       fb[u] = (in && col_ok) ? *reinterpret_cast<const frag_mem<T>*>(wr + kk) : zero_frag<T>();
+      if (norm_w != nullptr) {
+        const frag<T> fg = in ? *reinterpret_cast<const frag_mem<T>*>(norm_w + kk) : zero_frag<T>();
+        const vec<float, 8> xv = __builtin_convertvector(fa[u], vec<float, 8>);
+        const vec<float, 8> gv = __builtin_convertvector(fg, vec<float, 8>);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sq = __builtin_fmaf(xv[e], xv[e], sq);
+        fa[u] = __builtin_convertvector(xv * gv, frag<T>);
+      }
     }
 #pragma unroll
     for (int u = 0; u < MAXS; ++u) mma(acc, fa[u], fb[u]);
   }
 #pragma unroll
   for (int r = 0; r < 16; ++r) red[wave][acc_row(r, g)][c] = acc[r];
+  if (norm_w != nullptr) {
+    sq += __shfl_xor(sq, 32);   // the two halves of a row's 16-deep steps
+    if (g == 0) ssq[wave][c] = sq;
+  }
   __syncthreads();
   // 1024 outputs, 512 threads: two neighbouring columns each
   const int e = 2 * threadIdx.x, row = e / 32, col = e % 32;
   float s0 = 0.f, s1 = 0.f;
 #pragma unroll
   for (int v = 0; v < kLinWaves; ++v) { s0 += red[v][row][col]; s1 += red[v][row][col + 1]; }
+  if (norm_w != nullptr) {
+    float t = 0.f;
+#pragma unroll
+    for (int v = 0; v < kLinWaves; ++v) t += ssq[v][row];
+    const float rstd = __builtin_amdgcn_rsqf(t / (float)K + eps);
+    s0 *= rstd;
+    s1 *= rstd;
+  }
+  if (act == 1) {
+    s0 = 0.5f * s0 * (1.f + erff(s0 * 0.70710678f));
+    s1 = 0.5f * s1 * (1.f + erff(s1 * 0.70710678f));
+  }
   if (m0 + row < M) {
     T* dst = y + (int64_t)(m0 + row) * ldy + n0 + col;
+    const T* rsrc = res != nullptr ? res + (int64_t)(m0 + row) * ldr + n0 + col : nullptr;
     if (n0 + col + 1 < N) {
+      if (rsrc != nullptr) {
+        const vec<T, 2> rv = *reinterpret_cast<const vec<T, 2>*>(rsrc);
+        s0 += (float)rv[0];
+        s1 += (float)rv[1];
+      }
       vec<T, 2> o = {(T)s0, (T)s1};
       *reinterpret_cast<vec<T, 2>*>(dst) = o;
     } else if (n0 + col < N) {
+      if (rsrc != nullptr) s0 += (float)rsrc[0];
       dst[0] = (T)s0;
     }
   }
 }
-
 int launch_small_linear(const void* x, const void* w, void* y, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldy,
-                        int dtype, hipStream_t stream) {
+                        int dtype, const void* norm_w, float eps, int act, const void* res, int64_t ldr, hipStream_t stream) {
   const dim3 grid((N + 31) / 32, (M + 31) / 32), block(64 * kLinWaves);
   if (dtype == 1)
     hipLaunchKernelGGL((small_linear_kernel<bf16_t>), grid, block, 0, stream, static_cast<const bf16_t*>(x),
-                       static_cast<const bf16_t*>(w), static_cast<bf16_t*>(y), M, N, K, ldx, ldw, ldy);
+                       static_cast<const bf16_t*>(w), static_cast<bf16_t*>(y), M, N, K, ldx, ldw, ldy,
+                       static_cast<const bf16_t*>(norm_w), eps, act, static_cast<const bf16_t*>(res), ldr);
   else if (dtype == 2)
     hipLaunchKernelGGL((small_linear_kernel<fp16_t>), grid, block, 0, stream, static_cast<const fp16_t*>(x),
-                       static_cast<const fp16_t*>(w), static_cast<fp16_t*>(y), M, N, K, ldx, ldw, ldy);
+                       static_cast<const fp16_t*>(w), static_cast<fp16_t*>(y), M, N, K, ldx, ldw, ldy,
+                       static_cast<const fp16_t*>(norm_w), eps, act, static_cast<const fp16_t*>(res), ldr);
   else
     return -1;
   return hipGetLastError() == hipSuccess ? 0 : -3;

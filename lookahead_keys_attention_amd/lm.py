@@ -46,11 +46,12 @@ def top_k(logits: torch.Tensor, thres: float = 0.9) -> torch.Tensor:
 
 
 def token_feed_forward(feed_forward: nn.Sequential, h: torch.Tensor) -> torch.Tensor:
-    """The feed-forward block [norm, linear, GELU, linear] for a single-token step (inference): the
-    two bias-free projections have `batch` rows, so they go through `ops.small_linear` when it can
-    take them (16-bit GPU tensors) and through the layers themselves otherwise."""
+    """h + feed_forward(h) for a single-token step (inference), the block being [norm, linear,
+    GELU, linear]: two launches of the small-M linear kernel (norm and GELU ride on the first, the
+    residual on the second) when it can take them (16-bit GPU tensors), the layers themselves otherwise."""
     norm, up, act, down = feed_forward
-    return Castle._project(down, act(Castle._project(up, norm(h), True)), True)
+    hidden = Castle._project(up, h, True, norm=norm, activation="gelu")
+    return Castle._project(down, hidden, True, residual=h)
 
 
 class GraphedDecoder:
@@ -133,9 +134,9 @@ class GraphedDecoder:
         model = self.model
         h = model.token_emb(self.token)
         for (attention, feed_forward), store in zip(model.layers, self.stores):
-            h = h + attention.graph_step(h, store, self.t_device, self.base_device)
-            h = h + token_feed_forward(feed_forward, h)
-        return Castle._project(model.to_logits, model.final_norm(h), True)
+            h = attention.graph_step(h, store, self.t_device, self.base_device, residual=h)
+            h = token_feed_forward(feed_forward, h)
+        return Castle._project(model.to_logits, h, True, norm=model.final_norm)
 
     def step(self, token):
         """Feeds `token` (batch, 1) and returns the logits (batch, 1, num_tokens) of the next
@@ -197,8 +198,8 @@ class CastleLM(nn.Module):
             else:
                 attended = attention(h, cache=layer_cache, return_next_cache=False)
             h = h + attended
-            h = h + (token_feed_forward(feed_forward, h) if token_step else feed_forward(h))
-        logits = Castle._project(self.to_logits, self.final_norm(h), token_step)
+            h = token_feed_forward(feed_forward, h) if token_step else h + feed_forward(h)
+        logits = Castle._project(self.to_logits, h, token_step, norm=self.final_norm)
         if return_loss:
             return F.cross_entropy(logits.transpose(1, 2), target)
         return (logits, next_cache) if return_next_cache else logits

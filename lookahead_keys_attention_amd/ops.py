@@ -356,16 +356,34 @@ def small_linear_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:
 
 
 @torch.no_grad()
-def small_linear(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+def small_linear(x: torch.Tensor, weight: torch.Tensor, norm=None, activation=None, residual=None) -> torch.Tensor:
     """(B, 1, K) x (N, K) -> (B, 1, N): the projections around the cached single-token step
-    (lookahead_keys_attention.py:99, 209 with seq_len == 1), without bias, for inference."""
+    (lookahead_keys_attention.py:99, 209 with seq_len == 1), without bias, for inference.
+
+    The per-row work next to such a projection in a token step can ride along (one launch instead
+    of up to four): `norm` an nn.RMSNorm applied to x first (lookahead_keys_attention.py:95,
+    train_triton.py:103, 164), `activation="gelu"` the erf GELU of train_triton.py:105 on the
+    product, `residual` a (B, 1, N) tensor added last (train_triton.py:161-162)."""
     B, _, K = x.shape
     n = weight.shape[0]
     y = torch.empty((B, 1, n), dtype=x.dtype, device=x.device)
+    norm_weight, eps = None, 0.0
+    if norm is not None:
+        norm_weight = norm.weight
+        eps = norm.eps if norm.eps is not None else torch.finfo(x.dtype).eps   # what F.rms_norm uses for eps=None
+        if norm_weight.dtype != x.dtype or norm_weight.numel() != K or not norm_weight.is_contiguous():
+            raise ValueError("small_linear: the norm weight must be a contiguous (K,) tensor of the input type")
+    if activation not in (None, "gelu"):
+        raise ValueError(f"small_linear: unknown activation {activation!r}")
+    if residual is not None and (residual.shape != y.shape or residual.dtype != x.dtype or residual.stride(2) != 1):
+        raise ValueError("small_linear: the residual must have the output's shape and type")
     with torch.cuda.device(x.device):
-        rc = N.lib().castle_small_linear(x.data_ptr(), weight.data_ptr(), y.data_ptr(), B, n, K, x.stride(0),
-                                         weight.stride(0), n, N.dtype_code(x.dtype), N.stream_ptr(x.device))
-    N.check(rc, "castle_small_linear")
+        rc = N.lib().castle_small_linear_fused(
+            x.data_ptr(), weight.data_ptr(), y.data_ptr(), B, n, K, x.stride(0), weight.stride(0), n, N.dtype_code(x.dtype),
+            norm_weight.data_ptr() if norm_weight is not None else None, eps, 1 if activation == "gelu" else 0,
+            residual.data_ptr() if residual is not None else None, residual.stride(0) if residual is not None else 0,
+            N.stream_ptr(x.device))
+    N.check(rc, "castle_small_linear_fused")
     return y
 
 

@@ -385,6 +385,45 @@ def test_small_linear_matches_fp64_matmul(M, N, K, dtype):
     assert err <= 2.0 ** (-8 if dtype == torch.bfloat16 else -11) * ref.abs().max().item() * 1.01 + 1e-6   # one rounding of the result
 
 
+@pytest.mark.parametrize("M,N,K,dtype,norm,act,res", [(16, 2048, 512, torch.bfloat16, True, "gelu", False),
+                                                       (16, 512, 2048, torch.bfloat16, False, None, True),
+                                                       (3, 258, 264, torch.float16, True, None, True),
+                                                       (33, 96, 40, torch.bfloat16, True, "gelu", True)])
+def test_small_linear_with_norm_activation_and_residual(M, N, K, dtype, norm, act, res):
+    """castle_small_linear_fused: RMS normalisation in front, erf GELU and a residual behind, in one
+    launch, against the same chain in fp64 on the same 16-bit values (nn.RMSNorm with eps=None takes
+    the type's machine epsilon; the norm weight multiplies the normalised row)."""
+    g = torch.Generator().manual_seed(M + N + K)
+    x = (torch.randn(M, 1, K, generator=g) * 1.7).to(dtype).to(DEV)
+    w = (torch.randn(N, K, generator=g) * K ** -0.5).to(dtype).to(DEV)
+    r = torch.randn(M, 1, N, generator=g).to(dtype).to(DEV) if res else None
+    layer = torch.nn.RMSNorm(K).to(DEV).to(dtype) if norm else None
+    if norm:
+        with torch.no_grad():
+            layer.weight.copy_((1 + 0.3 * torch.randn(K, generator=g)).to(dtype))
+    y = H().small_linear(x, w, norm=layer, activation=act, residual=r)
+    ref = x.double()
+    if norm:
+        eps = torch.finfo(dtype).eps
+        ref = ref * torch.rsqrt(ref.pow(2).mean(-1, keepdim=True) + eps) * layer.weight.double()
+    ref = ref @ w.double().T
+    if act == "gelu":
+        ref = torch.nn.functional.gelu(ref)
+    if res:
+        ref = ref + r.double()
+    assert y.shape == (M, 1, N) and y.dtype == dtype
+    err = (y.double() - ref).abs().max().item()
+    assert err <= 1e-2 * max(ref.abs().max().item(), 1.0), err
+    # the unfused modules give the same within the rounding of their intermediate tensors
+    if norm:
+        mods = torch.nn.functional.linear(layer(x), w)
+        if act == "gelu":
+            mods = torch.nn.functional.gelu(mods)
+        if res:
+            mods = mods + r
+        assert (y.float() - mods.float()).abs().max() <= 3e-2 * max(mods.float().abs().max().item(), 1.0)
+
+
 @pytest.mark.parametrize("B,Hh,t0,steps,d,dtype,rotary", [(2, 2, 0, 23, 64, torch.float32, False), (1, 2, 101, 18, 32, torch.float32, True),
                                                         (2, 2, 203, 21, 64, torch.bfloat16, False), (1, 2, 130, 9, 128, torch.bfloat16, True)])
 def test_decode_with_deferred_write_back(B, Hh, t0, steps, d, dtype, rotary):
