@@ -1193,7 +1193,7 @@ struct TileStage {
   __device__ __forceinline__ void load(const T* src) {
     const int slab = threadIdx.x >> 6, l = threadIdx.x & 63;       // slab = 2 * tile + s2
     const int g = (l >> 4) & 1, k = (l & 15) + 16 * (l >> 5);
-    r = *reinterpret_cast<const frag_mem<T>*>(src + slab * 512 + k * 16 + g * 8);
+    r = __builtin_nontemporal_load(reinterpret_cast<const frag_mem<T>*>(src + slab * 512 + k * 16 + g * 8));   // read once
   }
   __device__ __forceinline__ void store(T* dst) const {
     const int slab = threadIdx.x >> 6, l = threadIdx.x & 63;

@@ -491,7 +491,7 @@ __device__ __forceinline__ void store_snap_tile(T* tile, const acc_t (&st)[NT], 
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int n = 32 * nt + 8 * q + 4 * g;
-      if (n < HD) st4<T>(tile + snap_elem<T>(c, n), pack4<T>(st[nt], q));
+      if (n < HD) __builtin_nontemporal_store(pack4<T>(st[nt], q), reinterpret_cast<vec4_mem<T>*>(tile + snap_elem<T>(c, n)));
     }
 }
 
@@ -499,7 +499,7 @@ __device__ __forceinline__ void store_snap_tile(T* tile, const acc_t (&st)[NT], 
 template <typename T> __device__ __forceinline__ frag<T> ldg_snap_nat(const T* tile, int c, int col) {
   constexpr int V = elem_traits<T>::vec16;
   if constexpr (V == 8) {
-    return *reinterpret_cast<const frag_mem<T>*>(tile + snap_elem<T>(c, col));
+    return __builtin_nontemporal_load(reinterpret_cast<const frag_mem<T>*>(tile + snap_elem<T>(c, col)));   // read once
   } else {
     frag<T> f;
     const vec<T, 4> lo = *reinterpret_cast<const vec<T, 4>*>(tile + snap_elem<T>(c, col));
@@ -525,7 +525,7 @@ struct SnapStage {
 #pragma unroll
     for (int n = 0; n < N; ++n) {
       const int v = tid + n * kThreads;
-      if (v < TOTAL) r[n] = *reinterpret_cast<const vec<T, V>*>(src + (int64_t)v * V);
+      if (v < TOTAL) r[n] = __builtin_nontemporal_load(reinterpret_cast<const vec<T, V>*>(src + (int64_t)v * V));   // read once
     }
   }
   __device__ __forceinline__ void store(T* dst, int ld, int tid = threadIdx.x) const {
