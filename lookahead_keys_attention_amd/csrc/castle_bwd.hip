@@ -241,7 +241,7 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
         const int i0 = I * kNB + 32 * it;
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2)
-          tdsu[it][s2] = (active && i0 + 31 >= kw0) ? *reinterpret_cast<const frag_mem<T>*>(dsu_tiles + (int64_t)(i0 / 32) * 1024 + s2 * 512)
+          tdsu[it][s2] = (active && i0 + 31 >= kw0) ? __builtin_nontemporal_load(reinterpret_cast<const frag_mem<T>*>(dsu_tiles + (int64_t)(i0 / 32) * 1024 + s2 * 512))
                                                    : zero_frag<T>();
       }
     }
@@ -388,8 +388,8 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
           const int64_t tile = ((int64_t)(kw0 / 32) * (a.s.Lp / 32) + i0 / 32) * 1024 + c * 16 + 4 * g;
 #pragma unroll
           for (int q = 0; q < 4; ++q) {   // registers 4q .. 4q+3: queries 8q + 4g .. + 3 of the tile
-            st4<T>(ds_mat + tile + (q / 2) * 512 + 8 * (q % 2), pack4<T>(ds, q));
-            st4<T>(dsu_mat + tile + (q / 2) * 512 + 8 * (q % 2), pack4<T>(dsu, q));
+            st4_stream<T>(ds_mat + tile + (q / 2) * 512 + 8 * (q % 2), pack4<T>(ds, q));
+            st4_stream<T>(dsu_mat + tile + (q / 2) * 512 + 8 * (q % 2), pack4<T>(dsu, q));
           }
         }
       }

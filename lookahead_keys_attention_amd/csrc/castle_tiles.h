@@ -97,6 +97,8 @@ template <typename T> __device__ __forceinline__ frag<T> chain(const acc_t& c, i
 
 // store 4 packed elements (8 bytes for 16-bit types, 16 for fp32)
 template <typename T> __device__ __forceinline__ void st4(T* p, vec<T, 4> v) { *reinterpret_cast<vec4_mem<T>*>(p) = v; }
+// the same for data that is written once and read once by a later kernel: kept out of the way of what the caches hold
+template <typename T> __device__ __forceinline__ void st4_stream(T* p, vec<T, 4> v) { __builtin_nontemporal_store(v, reinterpret_cast<vec4_mem<T>*>(p)); }
 
 // 8 contiguous elements tile[row][col .. col+7]
 template <typename T> __device__ __forceinline__ frag<T> ld_nat(const T* tile, int ld, int row, int col) {
@@ -491,7 +493,7 @@ __device__ __forceinline__ void store_snap_tile(T* tile, const acc_t (&st)[NT], 
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int n = 32 * nt + 8 * q + 4 * g;
-      if (n < HD) __builtin_nontemporal_store(pack4<T>(st[nt], q), reinterpret_cast<vec4_mem<T>*>(tile + snap_elem<T>(c, n)));
+      if (n < HD) st4_stream<T>(tile + snap_elem<T>(c, n), pack4<T>(st[nt], q));
     }
 }
 
