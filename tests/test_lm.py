@@ -326,3 +326,21 @@ def test_config5_language_model_step_bf16():
         got, want = grads[name].grad.float().cpu(), leaves[name].grad
         rel = ((got - want).norm() / want.norm()).item()
         assert rel <= 2e-2, f"{name}: relative norm error {rel:.3e}"
+
+
+def test_token_feed_forward_equals_the_block_on_the_cpu():
+    """Off the GPU the single-token form of the feed-forward block (train_triton.py:102-107, 162)
+    runs the layers themselves: h + W2 gelu(W1 norm(h)), exactly what the block plus the residual give;
+    the same holds for Castle._project with a norm in front and a residual behind."""
+    from lookahead_keys_attention_amd import Castle
+    from lookahead_keys_attention_amd.lm import token_feed_forward
+
+    torch.manual_seed(2)
+    model = make_lm(depth=1, dim=32, heads=2, dim_head=16, rotary=False, native=False)
+    _, feed_forward = model.layers[0]
+    h = torch.randn(3, 1, 32)
+    assert torch.allclose(token_feed_forward(feed_forward, h), h + feed_forward(h), atol=1e-6)
+    got = Castle._project(model.to_logits, h, True, norm=model.final_norm)
+    assert torch.allclose(got, model.to_logits(model.final_norm(h)), atol=1e-6)
+    assert torch.allclose(Castle._project(feed_forward[1], h, False, norm=torch.nn.Identity(), activation="gelu", residual=None),
+                          torch.nn.functional.gelu(feed_forward[1](h)), atol=1e-6)
