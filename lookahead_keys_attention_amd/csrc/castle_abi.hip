@@ -24,6 +24,19 @@ int launch_small_linear(const void* x, const void* w, void* y, int M, int N, int
 
 namespace {
 
+// compute units of the current device, looked up once per device
+int device_cus() {
+  static int cus[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  if (cus[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 0;
+    cus[dev] = n;
+  }
+  return cus[dev];
+}
+
 using castle::kNB;
 
 int elem_size(int dtype) {
@@ -188,6 +201,7 @@ int castle_fwd(const castle_view4* qc, const castle_view4* kc, const castle_view
   castle::FwdArgs a;
   a.s.B = B; a.s.H = H; a.s.L = L; a.s.d = d; a.s.Lp = g.Lp; a.s.nblk = g.nblk; a.s.scale = scale;
   a.s.rotary = (flags & CASTLE_FLAG_ROTARY) != 0;
+  a.s.cus = device_cus();
   a.qc = to_view(qc); a.kc = to_view(kc); a.vc = to_view(vc);
   a.qu = to_view(qu); a.ku = to_view(ku); a.vu = to_view(vu);
   a.out = to_view(out);
@@ -232,6 +246,7 @@ int castle_bwd(const castle_view4* qc, const castle_view4* kc, const castle_view
   castle::BwdArgs a;
   a.s.B = B; a.s.H = H; a.s.L = L; a.s.d = d; a.s.Lp = g.Lp; a.s.nblk = g.nblk; a.s.scale = scale;
   a.s.rotary = (flags & CASTLE_FLAG_ROTARY) != 0;
+  a.s.cus = device_cus();
   a.qc = to_view(qc); a.kc = to_view(kc); a.vc = to_view(vc);
   a.qu = to_view(qu); a.ku = to_view(ku); a.vu = to_view(vu);
   a.out = to_view(out); a.dout = to_view(dout);

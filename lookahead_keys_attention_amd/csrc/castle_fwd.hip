@@ -294,6 +294,7 @@ __global__ __launch_bounds__(kThreads, (sizeof(T) == 2 && HD <= 64) ? 2 : 1) voi
   T* s_a = s_vct + vtile_elems<T, HD>();         // [kNB][LDA]
   constexpr bool TRV = sizeof(T) == 2;
 
+  prio_by_band(blockIdx.x, a.s.cus);
   int rank, bh;
   work_item(a.s.B * a.s.H, rank, bh);
   const int qb = a.s.Lp / 128 - 1 - rank;   // the last query block sees the most keys

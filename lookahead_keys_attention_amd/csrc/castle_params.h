@@ -16,6 +16,7 @@ struct CoreShape {
   int nblk;   // Lp / kNB
   float scale;
   int rotary;   // 1: qc, kc, qu, ku, vu are rotated by their row position (RoPE) inside the kernels
+  int cus;      // compute units of the device (0: unknown), for prio_by_band
 };
 
 // Header of the forward workspace (its first 256 bytes), written on the device by the forward pass.
