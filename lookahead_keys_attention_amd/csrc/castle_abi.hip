@@ -271,6 +271,7 @@ int castle_bwd(const castle_view4* qc, const castle_view4* kc, const castle_view
     f.out = a.out;
     f.U = to_view(nullptr);
     f.ws = a.ws;
+    f.with_t = 0;
     rc = castle::launch_scan(f, dtype, (flags & CASTLE_FLAG_BF16_OPERANDS) != 0, static_cast<hipStream_t>(stream));
     if (rc != 0) return rc;
   }

@@ -3,7 +3,8 @@
 //   prep_kernel  the six operands -> compute type, [B*H][Lp][d] contiguous, rows >= L zero, Qc
 //                pre-multiplied by scale*log2(e); every other kernel reads these copies, so its
 //                tile loads need neither conversions nor bounds nor strides
-//   tqv_kernel   per 64-row block I:  T_II = tril(Qc_I Vu_I^T)  (and its transpose)
+//   tqv_block    per 64-row block I:  T_II = tril(Qc_I Vu_I^T), both orientations, and the cross quarter
+//                of a block pair; run by the trailing workgroups of the scan launch
 //   scan_kernel  key-stationary: for a group of 128 keys sweep the source blocks I,
 //                A_KI = sigmoid(s Qu_K Ku_I^T) (strictly j>k), state += A_KI Vu_I.
 //                The state as of the start of block I is stored as snapshot
@@ -114,12 +115,15 @@ __global__ __launch_bounds__(kThreads) void prep_kernel(FwdArgs a) {
 }
 
 // ---------------------------------------------------------------------------
+// T' of one 64-row block, by the four waves of a workgroup (one 32x32 tile each).  These blocks have
+// no kernel of their own: they are the last workgroups of the scan launch, which reads none of them,
+// so they run in the slots the scan's tail leaves empty (its last fifth runs at under half occupancy:
+// the launch cannot end before the 64-block sweep of key group 0 does).
 template <typename T, typename TI, int HD>
-__global__ __launch_bounds__(kThreads) void tqv_kernel(FwdArgs a) {
+__device__ __forceinline__ void tqv_block(const FwdArgs& a, int I, int bh) {
   constexpr int KS = HD / 16;
   constexpr int TB = kNB / 32;
   static_assert(TB * TB == kThreads / 64, "one 32x32 tile of the block per wave");
-  const int I = blockIdx.x, bh = blockIdx.y;
   const int lane = lane_id(), c = lane & 31, g = lane >> 5;
   const T* qc = prep_ptr<T>(a.ws.qc_p, bh, a.s.Lp, HD);   // pre-scaled by c1
   const T* vu = prep_ptr<T>(a.ws.vu_p, bh, a.s.Lp, HD);
@@ -189,6 +193,14 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(FwdArgs a) {
   T* s_vut = s_ku + kNB * LDK;                   // fp32: [HDP][LDV] (transposed); 16-bit: [kNB][LDK]
   constexpr bool TRV = sizeof(T) == 2;
 
+  {
+    const int BH = a.s.B * a.s.H, n_scan = a.s.Lp / 128 * BH;
+    if ((int)blockIdx.x >= n_scan) {   // behind the key groups: the T' blocks
+      const int id = blockIdx.x - n_scan;
+      tqv_block<T, TI, HD>(a, id / BH, id % BH);
+      return;
+    }
+  }
   int kb, bh;   // key group 0 sweeps every source block: rank order = kb
   work_item(a.s.B * a.s.H, kb, bh);
   const int b = bh / a.s.H, h = bh % a.s.H;
@@ -498,11 +510,10 @@ template <typename T, typename TI, int HD> static int launch_fwd_t(const FwdArgs
       hipLaunchKernelGGL((amax_kernel<TI, HD>), dim3(kAmaxBlocks), dim3(kAmaxThreads), 0, stream, a.vu, a.s.H, a.s.L,
                          (int64_t)BH * a.s.L, a.ws.amax_part, &a.ws.hdr->status);
     hipLaunchKernelGGL((prep_kernel<T, TI, HD>), dim3((a.s.Lp * PIECES_PER_ROW + kThreads - 1) / kThreads, BH, 6), dim3(kThreads), 0, stream, a);
-    hipLaunchKernelGGL((tqv_kernel<T, TI, HD>), dim3(a.s.nblk, BH), dim3(kThreads), 0, stream, a);
   }
   {
     ProfScope ps(kSlotScan, stream);
-    hipLaunchKernelGGL((scan_kernel<T, TI, HD>), dim3(a.s.Lp / 128 * BH), dim3(kThreads), scan_lds, stream, a);
+    hipLaunchKernelGGL((scan_kernel<T, TI, HD>), dim3(a.s.Lp / 128 * BH + (a.with_t ? a.s.nblk * BH : 0)), dim3(kThreads), scan_lds, stream, a);
   }
   {
     ProfScope ps(kSlotAttn, stream);
@@ -532,7 +543,7 @@ template <typename T, typename TI, int HD> static int launch_scan_t(const FwdArg
     configured = true;
   }
   ProfScope ps(kSlotScan, stream);
-  hipLaunchKernelGGL((scan_kernel<T, TI, HD>), dim3(a.s.Lp / 128 * a.s.B * a.s.H), dim3(kThreads), scan_lds, stream, a);
+  hipLaunchKernelGGL((scan_kernel<T, TI, HD>), dim3(a.s.Lp / 128 * a.s.B * a.s.H + (a.with_t ? a.s.nblk * a.s.B * a.s.H : 0)), dim3(kThreads), scan_lds, stream, a);
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 template <typename T, typename TI> static int launch_scan_d(const FwdArgs& a, hipStream_t stream) {

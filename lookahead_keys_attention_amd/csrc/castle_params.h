@@ -57,6 +57,7 @@ struct FwdArgs {
   View4 out;      // written as (B, H, L, d) through arbitrary strides
   View4 U;        // ptr == nullptr when the final lookahead keys are not wanted
   FwdWorkspace ws;
+  int with_t = 1; // the scan launch also fills the T' blocks (0 when only the snapshots are recomputed for a backward pass)
 };
 
 struct BwdArgs {
