@@ -51,7 +51,7 @@ def recorded_traffic():
 # algorithmic contractions (unit: B*H*L^2*d flop = 2*d flop per causal pair) attributed to each kernel.
 # They sum to 18: the 19th contraction of the algorithmic count (the forward state update, which a
 # backward pass that keeps nothing would repeat) is not executed because the snapshots are kept.
-KERNEL_UNITS = {"tqv": 0.0, "scan": 2.0, "attn": 3.0, "delta": 0.0, "bwd_key": 9.0, "bwd_query": 4.0}
+KERNEL_UNITS = {"prep": 0.0, "scan": 2.0, "attn": 3.0, "delta": 0.0, "bwd_key": 9.0, "bwd_query": 4.0}
 
 
 def cfg2_flops(B, H, L, d, dim):

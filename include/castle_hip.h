@@ -234,7 +234,7 @@ int castle_small_linear_fused(const void* x, const void* w, void* y, int M, int 
  * kernel launched by the entry points above is bracketed by a HIP event pair on its stream.
  * castle_profile_enable(on) also discards pending records.  castle_profile_read waits for the
  * recorded kernels, writes up to max_records (slot, milliseconds) pairs in launch order, clears
- * the records and returns their number (< 0 on error).  Slots: 0 T-blocks, 1 forward scan,
+ * the records and returns their number (< 0 on error).  Slots: 0 operand copies (with the pass for max|vu|), 1 forward scan (with the T' blocks),
  * 2 forward attention, 3 delta, 4 backward key-stationary, 5 backward query-stationary,
  * 6 decode stream, 7 decode finish. */
 int castle_profile_enable(int on);

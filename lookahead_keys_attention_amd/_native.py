@@ -168,7 +168,7 @@ def stream_ptr(device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
 
-PROFILE_SLOTS = ("tqv", "scan", "attn", "delta", "bwd_key", "bwd_query", "decode_stream", "decode_finish")
+PROFILE_SLOTS = ("prep", "scan", "attn", "delta", "bwd_key", "bwd_query", "decode_stream", "decode_finish")
 
 
 def profile_enable(on: bool):

@@ -504,7 +504,7 @@ template <typename T, typename TI, int HD> static int launch_fwd_t(const FwdArgs
     configured = true;
   }
   {
-    ProfScope ps(kSlotTqv, stream);
+    ProfScope ps(kSlotPrep, stream);
     constexpr int PIECES_PER_ROW = HD / elem_traits<T>::vec16;
     if constexpr (sizeof(T) == 2)
       hipLaunchKernelGGL((amax_kernel<TI, HD>), dim3(kAmaxBlocks), dim3(kAmaxThreads), 0, stream, a.vu, a.s.H, a.s.L,

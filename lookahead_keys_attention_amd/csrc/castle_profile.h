@@ -6,7 +6,7 @@ namespace castle {
 
 // kernel slots reported by castle_profile_read
 enum ProfSlot {
-  kSlotTqv = 0, kSlotScan = 1, kSlotAttn = 2,
+  kSlotPrep = 0, kSlotScan = 1, kSlotAttn = 2,
   kSlotDelta = 3, kSlotBwdKey = 4, kSlotBwdQuery = 5,
   kSlotDecodeStream = 6, kSlotDecodeFinish = 7,
 };
