@@ -290,43 +290,57 @@ def blockwise_forward(qc, kc, vc, qu, ku, vu, scale, nb):
         snap[I][k] = sum_{k<j<I*nb} A[k,j] vu_j
     is the lookahead key of k as of the start of block I, so that for i in block I
         Su[i,k] = (s qc_i).snap[I][k] + sum_{j in block I, k<j<=i} T[i,j] A[k,j].
+    Row blocks are streamed: the gate columns of a block, its scores and its softmax are formed
+    and dropped per block, so nothing of size L x L exists and L = 16384 fits a host.
     Returns dict(out, lse, U, snaps=[None, snap_1, ...], T=[T_II per block])."""
     L, d = qc.shape
     assert L % nb == 0
     nblk = L // nb
-    q = qc * scale
-    A = lookahead_gate(qu, ku, scale)
+    q, qus = qc * scale, qu * scale
     state = torch.zeros(L, d, dtype=qc.dtype)
     snaps, Tblocks = [], []
-    S = torch.full((L, L), -float("inf"), dtype=qc.dtype)
+    out = torch.empty_like(qc)
+    lse = torch.empty(L, dtype=qc.dtype)
     tri = torch.ones(nb, nb, dtype=torch.bool).tril(0)
     for I in range(nblk):
         r = slice(I * nb, (I + 1) * nb)
+        hi = (I + 1) * nb
         snaps.append(state[: I * nb].clone() if I > 0 else None)
         T_II = (q[r] @ vu[r].t()) * tri
         Tblocks.append(T_II)
-        hi = (I + 1) * nb
-        Su = q[r] @ state[:hi].t() + T_II @ A[:hi, r].t()
+        A_KI = _gate_columns(qus, ku, I, nb)
+        Su = q[r] @ state[:hi].t() + T_II @ A_KI.t()
         Sblk = q[r] @ kc[:hi].t() - F.silu(Su)
         cols = torch.arange(hi)[None, :] <= torch.arange(I * nb, hi)[:, None]
-        S[r, :hi] = torch.where(cols, Sblk, torch.full_like(Sblk, -float("inf")))
-        state[:hi] += A[:hi, r] @ vu[r]
-    lse = torch.logsumexp(S, dim=-1)
-    out = torch.exp(S - lse[:, None]) @ vc
+        Sblk = torch.where(cols, Sblk, torch.full_like(Sblk, -float("inf")))
+        lse[r] = torch.logsumexp(Sblk, dim=-1)
+        out[r] = torch.exp(Sblk - lse[r, None]) @ vc[:hi]
+        state[:hi] += A_KI @ vu[r]
     return {"out": out, "lse": lse, "U": state, "snaps": snaps, "T": Tblocks}
 
 
+def _gate_columns(qus, ku, I, nb):
+    """A[:hi, block I] of lookahead_gate: sigmoid(s qu_k . ku_j) for j in block I and k < j, else 0."""
+    hi = (I + 1) * nb
+    j = torch.arange(I * nb, hi)
+    k = torch.arange(hi)
+    return torch.sigmoid(qus[:hi] @ ku[I * nb:hi].t()) * (j[None, :] > k[:, None])
+
+
 def blockwise_backward(qc, kc, vc, qu, ku, vu, scale, nb, d_out):
-    """Reverse-state form of closed_form_grads for ONE head (L multiple of nb).
+    """Reverse-state form of closed_form_grads for ONE head (L multiple of nb), row blocks streamed.
 
     gsnap[I][k] (k < (I+1)*nb) = sum_{i >= (I+1)*nb} dSu[i,k] (s qc_i) is the reverse
     state of key k as of query block I.  Returns dict(grads=(dqc,dkc,dvc,dqu,dku,dvu),
-    gsnaps=[...], delta)."""
+    gsnaps=[...] (only when keep_gsnaps), delta)."""
+    return _blockwise_backward(qc, kc, vc, qu, ku, vu, scale, nb, d_out, keep_gsnaps=True)
+
+
+def _blockwise_backward(qc, kc, vc, qu, ku, vu, scale, nb, d_out, keep_gsnaps):
     L, d = qc.shape
     nblk = L // nb
     fw = blockwise_forward(qc, kc, vc, qu, ku, vu, scale, nb)
     q, qus = qc * scale, qu * scale
-    A = lookahead_gate(qu, ku, scale)
     delta = (d_out * fw["out"]).sum(-1)
     dq = torch.zeros_like(qc); dKc = torch.zeros_like(qc); dVc = torch.zeros_like(qc)
     dqu = torch.zeros_like(qc); dKu = torch.zeros_like(qc); dVu = torch.zeros_like(qc)
@@ -336,12 +350,14 @@ def blockwise_backward(qc, kc, vc, qu, ku, vu, scale, nb, d_out):
     for I in reversed(range(nblk)):
         r = slice(I * nb, (I + 1) * nb)
         hi = (I + 1) * nb
-        gsnaps[I] = G[:hi].clone()
+        if keep_gsnaps:
+            gsnaps[I] = G[:hi].clone()
         Ub = torch.zeros(hi, d, dtype=qc.dtype)
         if I > 0:
             Ub[: I * nb] = fw["snaps"][I]
+            fw["snaps"][I] = None   # consumed: blocks are visited once, from the last to the first
         T_II = fw["T"][I]
-        A_KI = A[:hi, r]
+        A_KI = _gate_columns(qus, ku, I, nb)
         Su = q[r] @ Ub.t() + T_II @ A_KI.t()
         Sraw = q[r] @ kc[:hi].t() - F.silu(Su)
         cols = torch.arange(hi)[None, :] <= torch.arange(I * nb, hi)[:, None]
@@ -359,4 +375,12 @@ def blockwise_backward(qc, kc, vc, qu, ku, vu, scale, nb, d_out):
         dqu[:hi] += dZ @ ku[r]
         dKu[r] += dZ.t() @ qus[:hi]
         G[:hi] += dSu.t() @ q[r]
-    return {"grads": (dq * scale, dKc, dVc, dqu * scale, dKu, dVu), "gsnaps": gsnaps, "delta": delta}
+    return {"out": fw["out"], "U": fw["U"], "grads": (dq * scale, dKc, dVc, dqu * scale, dKu, dVu), "gsnaps": gsnaps, "delta": delta}
+
+
+def blockwise_head(qc, kc, vc, qu, ku, vu, scale, nb, d_out):
+    """out, U and the six gradients of ONE head through the streamed state forms, keeping no
+    reverse-state snapshots: the checker for full-length heads (L = 16384) that the dense
+    functions cannot reach."""
+    bw = _blockwise_backward(qc, kc, vc, qu, ku, vu, scale, nb, d_out, keep_gsnaps=False)
+    return bw["out"], bw["U"], bw["grads"]

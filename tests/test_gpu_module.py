@@ -174,16 +174,22 @@ def test_config1_readme_fp32_parallel_vs_sequential():
     assert (full.cpu() - ref).abs().max() <= 1e-3 and (seq.cpu() - ref).abs().max() <= 1e-3
 
 
-def _head_oracle_check(proj, dmerged, merged, dproj, heads, d, b, h):
-    """fp32 oracle for one (b, h) slice of a packed bf16 run: out and the six gradients."""
+def _head_oracle_check(proj, dmerged, merged, dproj, heads, d, b, h, nb=None, dtype=torch.float32):
+    """Oracle for one (b, h) slice of a packed bf16 run: out and the six gradients.  nb=None takes the
+    dense formulation (parallel_core, closed_form_grads), else the streamed state forms with row blocks
+    of nb (blockwise_head: pinned against the dense ones in tests/test_oracle_core.py), which reach
+    full-length heads."""
     B, L, _ = proj.shape
     six = proj.view(B, L, 6, heads, d)
-    qu, ku, vu, qc, kc, vc = [six[b, :, i, h].float().cpu() for i in range(6)]
-    do = dmerged.view(B, L, heads, d)[b, :, h].float().cpu()
+    qu, ku, vu, qc, kc, vc = [six[b, :, i, h].to(dtype).cpu() for i in range(6)]
+    do = dmerged.view(B, L, heads, d)[b, :, h].to(dtype).cpu()
     s = d ** -0.5
-    out = O.parallel_core(qc, kc, vc, qu, ku, vu, s)
+    if nb is None:
+        out = O.parallel_core(qc, kc, vc, qu, ku, vu, s)
+        grads = O.closed_form_grads(qc, kc, vc, qu, ku, vu, s, do)
+    else:
+        out, _, grads = O.blockwise_head(qc, kc, vc, qu, ku, vu, s, nb, do)
     bf16_close(merged.view(B, L, heads, d)[b, :, h], out, f"out[{b},{h}]")
-    grads = O.closed_form_grads(qc, kc, vc, qu, ku, vu, s, do)
     g6 = dproj.view(B, L, 6, heads, d)
     for name, idx, r in zip(("dqc", "dkc", "dvc", "dqu", "dku", "dvu"), (3, 4, 5, 0, 1, 2), grads):
         bf16_close(g6[b, :, idx, h], r, f"{name}[{b},{h}]")
@@ -202,6 +208,10 @@ def test_config2_bf16_full_size_sampled_heads():
     dmerged = (gy @ m.combine_heads.weight.detach())
     merged.backward(dmerged)
     assert torch.isfinite(merged).all() and torch.isfinite(proj.grad).all()
+    # eight (b, h) slices, one per value of (b * 8 + h) % 8: the kernels keep head bh on XCD bh % 8,
+    # so every XCD's share is checked; two of them also against the dense formulation
+    for b, h in ((0, 0), (1, 1), (2, 2), (3, 3), (0, 4), (3, 5), (2, 6), (1, 7)):
+        _head_oracle_check(proj.detach(), dmerged, merged.detach(), proj.grad, 8, 64, b, h, nb=256, dtype=torch.float64)
     for b, h in ((0, 0), (3, 5)):
         _head_oracle_check(proj.detach(), dmerged, merged.detach(), proj.grad, 8, 64, b, h)
     # causality at full size: the first 1024 positions do not depend on the rest
@@ -211,11 +221,13 @@ def test_config2_bf16_full_size_sampled_heads():
 
 def test_config3_bf16_long_context_forward_backward():
     # benchmark configuration 3: dim 2048, H16, d128, B1, L16384, bf16, forward + backward at full size.
-    # The dense oracle at L=16384 is out of reach on CPU, so the full-size run is checked through
+    # The dense oracle at L=16384 is out of reach on CPU; the streamed state form of the oracle is not:
+    # (o) two heads of the full-length run, forward and all six gradients, against oracle.blockwise_head
+    # in fp32 (lookahead scores have a standard deviation of about 20 at this length).  Beside it,
     # size-independent properties: (i) prefix invariance of the forward output; (iii) the backward
     # pass is linear in dO, and positions whose dO is zero (and that no later position with a
     # non-zero dO exists for) get exactly zero query/key/value gradients; and (ii) the same operator
-    # on the first 2048 positions is compared with the oracle (forward and all six gradients, one head).
+    # on the first 2048 positions is compared with the dense oracle (one head).
     from lookahead_keys_attention_amd import ops
 
     m = make(2048, 16, 128, dtype=torch.bfloat16, seed=0)
@@ -230,6 +242,9 @@ def test_config3_bf16_long_context_forward_backward():
     merged.backward(dmerged)
     g1 = leaf.grad.clone()
     assert torch.isfinite(merged).all() and torch.isfinite(g1).all()
+    # (o) full-length heads against the streamed oracle
+    for h in (7, 12):
+        _head_oracle_check(proj, dmerged, merged.detach(), g1, 16, 128, 0, h, nb=256)
     # (i) prefix invariance of the forward
     with torch.no_grad():
         short = ops.castle_attention_packed(proj[:, :2048].contiguous(), 16, m.scale)

@@ -129,7 +129,13 @@ def test_blockwise_state_form_equals_dense(L, d, nb):
     fw = O.blockwise_forward(qc, kc, vc, qu, ku, vu, s, nb)
     assert torch.allclose(fw["out"], out, atol=1e-11) and torch.allclose(fw["U"], U, atol=1e-11)
     bw = O.blockwise_backward(qc, kc, vc, qu, ku, vu, s, nb, g)
-    for a, b in zip(bw["grads"], O.closed_form_grads(qc, kc, vc, qu, ku, vu, s, g)):
+    dense = O.closed_form_grads(qc, kc, vc, qu, ku, vu, s, g)
+    for a, b in zip(bw["grads"], dense):
+        assert torch.allclose(a, b, atol=1e-10)
+    # the full-length checker (no reverse-state snapshots kept) is the same computation
+    out_h, U_h, grads_h = O.blockwise_head(qc, kc, vc, qu, ku, vu, s, nb, g)
+    assert torch.allclose(out_h, out, atol=1e-11) and torch.allclose(U_h, U, atol=1e-11)
+    for a, b in zip(grads_h, dense):
         assert torch.allclose(a, b, atol=1e-10)
 
 
