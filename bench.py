@@ -184,6 +184,15 @@ def bench_long_context(steps=3, warmup=2):
             "workspace_bytes": N_lib_code_ints(B, H, L, d)}
 
 
+def decode_step_bytes(B, H, t, d, es, base, defer=4):
+    """HBM bytes one cached step moves at row count t with the deferred write-back: the four cached
+    rows read, the cached gates (16 bytes per row) read while tokens are pending, the lookahead keys
+    written on every `defer`-th step and one gate (4 bytes) per row on the others, the new rows."""
+    pending = t - max(base, t - t % defer)
+    per_row = 4 * d * es + (4 * defer if pending > 0 else 0) + (d * es if (t + 1) % defer == 0 else 4)
+    return B * H * (t * per_row + 8 * d * es)
+
+
 def bench_decode(n_steps=512, prefill=2048):
     import torch
 
@@ -220,22 +229,26 @@ def bench_decode(n_steps=512, prefill=2048):
         _native.profile_enable(False)
     stream_ms = [ms for name, ms in rec if name == "decode_stream"]
     finish_ms = [ms for name, ms in rec if name == "decode_finish"]
-    bytes_total = sum(B * H * (5 * (prefill + i) * d + 8 * d) * 2 for i in range(len(stream_ms)))
+    n_rec = len(stream_ms)
+    # bytes per step: `moved` is what this kernel reads and writes (lookahead keys written back on every 4th
+    # step, 16 bytes of cached gates per row read while tokens are pending, 4 written per row otherwise);
+    # `reference` is what the reference's step moves (every lookahead key rewritten on every step):
+    # B*H*(5*t*d + 8*d)*2.  The roofline figures use the bytes moved.
+    bytes_moved = sum(decode_step_bytes(B, H, prefill + i, d, 2, prefill) for i in range(n_rec))
+    bytes_reference = sum(B * H * (5 * (prefill + i) * d + 8 * d) * 2 for i in range(n_rec))
     kern_s = (sum(stream_ms) + sum(finish_ms)) * 1e-3
-    gbs = bytes_total / (sum(stream_ms) * 1e-3) / 1e9
-    out["kernel_ms_per_step"] = round(kern_s * 1e3 / max(1, len(stream_ms)), 4)
-    out["kernel_tokens_per_s"] = round(B * len(stream_ms) / kern_s, 1)
+    gbs = bytes_moved / (sum(stream_ms) * 1e-3) / 1e9
+    out["kernel_ms_per_step"] = round(kern_s * 1e3 / max(1, n_rec), 4)
+    out["kernel_tokens_per_s"] = round(B * n_rec / kern_s, 1)
     rec = recorded_traffic()
     out["roofline"] = {"bound": "hbm", "kernel": "decode_stream", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
                        "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4),
-                       "traffic": rec.get("bytes", {}).get("decode_stream"), "traffic_source": rec.get("source")}
-    # the algorithmic bytes are the reference's (every lookahead key rewritten on every step); the kernel writes
-    # them back on every 4th step only, so the bytes it really moves (recorded counters) are fewer
-    moved = out["roofline"]["traffic"]
-    if moved:
-        out["roofline"]["moved_GBps"] = round(moved / (sum(stream_ms) / len(stream_ms) * 1e-3) / 1e9, 1)
-    # the whole step (two projections, stream and finish kernels) against the same algorithmic bytes
-    out["end_to_end_GBps"] = round(bytes_total / (t2 - t1) / 1e9 * (len(stream_ms) / n_steps), 1)
+                       "bytes_per_step": round(bytes_moved / max(1, n_rec)),
+                       "traffic": rec.get("bytes", {}).get("decode_stream"), "traffic_source": rec.get("source"),
+                       "reference_bytes_per_step": round(bytes_reference / max(1, n_rec)),
+                       "reference_bytes_GBps": round(bytes_reference / (sum(stream_ms) * 1e-3) / 1e9, 1)}
+    # the whole step (two projections, stream and finish kernels) against the bytes moved
+    out["end_to_end_GBps"] = round(bytes_moved / (t2 - t1) / 1e9 * (n_rec / n_steps), 1)
     out["end_to_end_frac_of_hbm_peak"] = round(out["end_to_end_GBps"] / PEAK_HBM_GBS, 4)
     out["workload"] = f"config 4: B{B} H{H} d{d} bf16, prefill {prefill}, {n_steps} cached steps"
     for k in ("prefill_tokens_per_s", "tokens_per_s", "ms_per_decode_step"):

@@ -23,7 +23,7 @@
 extern "C" {
 #endif
 
-#define CASTLE_ABI_VERSION 4
+#define CASTLE_ABI_VERSION 5
 
 /* element types of the tensors (accumulation is always fp32) */
 #define CASTLE_F32 0
@@ -50,6 +50,16 @@ extern "C" {
  * runs the forward scan again (from the operand copies in the forward workspace) into its own
  * workspace before anything else.  What a forward call must keep for its backward is then O(L d). */
 #define CASTLE_FLAG_RECOMPUTE_STATE 8
+
+/* castle_fwd (its U output), castle_decode_step*, castle_decode_flush; bf16 tensors only (else
+ * CASTLE_ERR_DTYPE); castle_bwd ignores it.  The lookahead-key buffer U is held in a half-precision
+ * cache format instead of bf16: each 2-byte element is the IEEE fp16 value of U * 2^-6, saturated at
+ * +-65504 (so |U| up to 4.2e6 is held, with 11 significant bits down to |U| = 2^-8 and an absolute
+ * step of 4e-6 below).  The reference's step re-rounds the whole of U to the module type at every
+ * token (lookahead_keys_attention.py:183); in bf16 those roundings add up to a few per cent over some
+ * hundred steps, in this format to an eighth of that, for the same bytes.  Every entry point that
+ * touches one U buffer must get the same setting; a reader converts with  U = 64 * (fp16 bits). */
+#define CASTLE_FLAG_U_HALF 16
 
 /* error codes */
 #define CASTLE_OK 0
@@ -109,8 +119,8 @@ int64_t castle_fwd_state_bytes(int B, int H, int L, int d, int dtype);
  * castle_attention_triton (lookahead_keys_attention.py:122).  out: (B,H,L,d) view that is
  * written (any strides, e.g. those of a (B,L,H,d) buffer).  U: optional (NULL, or a view
  * with ptr == NULL, to skip) final lookahead keys for the decode cache
- * (lookahead_keys_attention.py:161-164).  d in {16,32,64,128}; fp32 needs d <= 64. 
- * flags: 0 or CASTLE_FLAG_BF16_OPERANDS. */
+ * (lookahead_keys_attention.py:161-164).  d in {16,32,64,128}; fp32 needs d <= 64.
+ * flags: any of CASTLE_FLAG_BF16_OPERANDS, CASTLE_FLAG_ROTARY, CASTLE_FLAG_U_HALF (format of U). */
 int castle_fwd(const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
                const castle_view4* qu, const castle_view4* ku, const castle_view4* vu,
                int B, int H, int L, int d, int dtype, float scale, int flags,
@@ -150,7 +160,7 @@ int64_t castle_decode_workspace_bytes(int B, int H, int d, int t_max);
  * writes row t of all four (U_t = 0, qu, kc, vc of the new token) and writes
  * out (B,H,1,d) = softmax_k(s qc.kc_k - silu(s qc.U_k)) vc_k over k = 0..t.
  * qc..vu: the new token's (B,H,1,d) operands (stride_l unused).  After the call the cache
- * holds t+1 rows.  d in {16,32,64,128}.  flags: 0 or CASTLE_FLAG_ROTARY. */
+ * holds t+1 rows.  d in {16,32,64,128}.  flags: any of CASTLE_FLAG_ROTARY, CASTLE_FLAG_U_HALF. */
 int castle_decode_step(const castle_view4* U, const castle_view4* qu_cache,
                        const castle_view4* kc_cache, const castle_view4* vc_cache, int t, int capacity,
                        const castle_view4* qc, const castle_view4* kc, const castle_view4* vc,
@@ -160,9 +170,13 @@ int castle_decode_step(const castle_view4* U, const castle_view4* qu_cache,
                        void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Folds the pending sources into the stored lookahead keys (see castle_deferred): afterwards the U
- * rows 0 .. t-1 are what a step-by-step update would have left, and `base` = t describes the cache. */
+ * rows 0 .. t-1 are what a step-by-step update would have left.  POSTCONDITION the caller must
+ * establish before the next step or flush on this cache: `base` (and *base_device, when the steps read
+ * the base from device memory) = t.  The call does not write either; a second flush, or a step, with
+ * the old base adds the same gate * vu terms again.  `gates` must hold `capacity` rows of 4 floats
+ * (not checked).  flags: 0 or CASTLE_FLAG_U_HALF. */
 int castle_decode_flush(const castle_view4* U, const castle_view4* qu_cache, int t, const castle_deferred* deferred,
-                        int B, int H, int d, int dtype, float scale, void* stream);
+                        int B, int H, int d, int dtype, float scale, int flags, void* stream);
 
 /* The same step with the row count t read by the kernels from device memory (*t_device, an int32
  * the caller keeps and advances), so that the enqueued work does not depend on t: one captured HIP

@@ -14,13 +14,15 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libcastle_hip.so")
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 DTYPE_CODES = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
 SUPPORTED_HEAD_DIMS = (16, 32, 64, 128)
 FLAG_BF16_OPERANDS = 1   # keep bf16 MFMA operands for bf16 tensors (default: fp16 operands)
 FLAG_ROTARY = 2          # rotary position embedding of qc, kc, qu, ku, vu inside the kernels
 FLAG_RECOMPUTE_SCORES = 4   # backward without the dS / dSu tile hand-over (less workspace, slower)
 FLAG_RECOMPUTE_STATE = 8    # backward re-runs the forward scan: the forward state buffer need not be kept
+FLAG_U_HALF = 16            # bf16 caches: the lookahead-key buffer holds fp16 bits of U / 64 (see castle_hip.h)
+U_HALF_UNSCALE = 64.0
 
 EXPORTED_SYMBOLS = (
     "castle_abi_version",
@@ -99,7 +101,7 @@ def _declare(lib):
     lib.castle_decode_step_static.restype = i
     lib.castle_decode_step_static.argtypes = [_VP] * 4 + [i, vp, i] + [_VP] * 6 + [i, i, i, i, f, i, _VP, _DP, vp]
     lib.castle_decode_flush.restype = i
-    lib.castle_decode_flush.argtypes = [_VP, _VP, i, _DP, i, i, i, i, f, vp]
+    lib.castle_decode_flush.argtypes = [_VP, _VP, i, _DP, i, i, i, i, f, i, vp]
     lib.castle_decode_step_device_count.restype = i
     lib.castle_decode_step_device_count.argtypes = [_VP] * 4 + [vp, i] + [_VP] * 6 + [i, i, i, i, f, i, _VP, _DP, vp, i64, vp]
     lib.castle_small_linear.restype = i

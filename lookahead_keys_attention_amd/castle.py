@@ -46,27 +46,31 @@ class Cache(_CacheFields):
 
     A cache made by the native path is a set of views into its capacity buffers.  The native step
     writes the lookahead keys back on every 4th step only (the tokens in between are kept as pending
-    (ku, vu) rows and applied on the fly), so whoever READS `U` (the attribute, index 0, unpacking)
-    first gets the pending sources folded in: the tensor seen is always the true U."""
+    (ku, vu) rows and applied on the fly), and a bf16 cache keeps them in a half-precision format of
+    its own (`ops.LOOKAHEAD_KEYS_HALF`).  Whoever READS `U` (the attribute, index 0, unpacking) gets
+    the true U in the cache's type: the pending sources are folded in first, and a buffer in the
+    half-precision format is converted into a new tensor (a copy: a later step does not change it)."""
 
     _store = None   # set on caches that live in a native capacity buffer
 
-    def _complete(self):
-        if self._store is not None:
-            self._store.flush()
+    def _read(self):
+        raw = tuple.__getitem__(self, slice(None))
+        if self._store is None:
+            return raw
+        self._store.flush()
+        if self._store.u_half:
+            return (ops.decode_lookahead_keys(raw[0]),) + raw[1:]
+        return raw
 
     @property
     def U(self):
-        self._complete()
-        return tuple.__getitem__(self, 0)
+        return self._read()[0]
 
     def __getitem__(self, index):
-        self._complete()
-        return tuple.__getitem__(self, index)
+        return self._read()[index]
 
     def __iter__(self):
-        self._complete()
-        return tuple.__iter__(self)
+        return iter(self._read())
 
 
 class _CacheStore:
@@ -84,6 +88,8 @@ class _CacheStore:
                       torch.empty((B, H, capacity, _native.DECODE_DEFER), dtype=torch.float32, device=device))   # their gates per cached row
         self.base0 = 0
         self.scale = d ** -0.5
+        # bf16 buffers hold the lookahead keys in the half-precision cache format (fp16 bits of U / 64)
+        self.u_half = dtype == torch.bfloat16 and ops.LOOKAHEAD_KEYS_HALF
         self._geometry = (B, H, d, device)
         self._workspace = None
         self._views = None
@@ -118,7 +124,8 @@ class _CacheStore:
     def flush(self):
         """Completes the stored lookahead keys (no-op when nothing is pending)."""
         if self.pending() > 0:
-            ops.castle_decode_flush(self.buffers[0], self.buffers[1], self.length, self.deferred(), self.scale)
+            ops.castle_decode_flush(self.buffers[0], self.buffers[1], self.length, self.deferred(), self.scale,
+                                    u_half=self.u_half)
         self.base0 = self.length
 
     def as_cache(self) -> Cache:
@@ -131,11 +138,21 @@ class _CacheStore:
         B, H, _, d = self.buffers[0].shape
         self.flush()
         new = _CacheStore(B, H, d, max(min_capacity, 2 * self.capacity), self.buffers[0].dtype, self.buffers[0].device)
+        new.u_half = self.u_half   # the rows are copied as they are stored
         for dst, src in zip(new.buffers, self.buffers):
             dst[:, :, : self.length].copy_(src[:, :, : self.length])
         new.length = new.base0 = self.length
         new.scale = self.scale
         return new
+
+    def adopt(self, cache):
+        """Fills the buffers from a plain 4-tuple of (B, H, t, d) tensors."""
+        t = cache[0].shape[-2]
+        for buf, src in zip(self.buffers, cache):
+            buf[:, :, :t].copy_(src)
+        if self.u_half:
+            ops.encode_lookahead_keys(cache[0], self.buffers[0][:, :, :t])
+        self.length = self.base0 = t
 
 
 def _reserve_rows(n: int) -> int:
@@ -262,8 +279,10 @@ class Castle(nn.Module):
             return ops.castle_attention_packed(proj, H, self.scale, rotary=self.use_rotary), None
         capacity = _reserve_rows(n)
         # the kernels write the lookahead keys straight into what becomes the cache's U buffer
-        merged, U = ops.castle_attention_packed(proj, H, self.scale, True, capacity, rotary=self.use_rotary)
+        u_half = proj.dtype == torch.bfloat16 and ops.LOOKAHEAD_KEYS_HALF
+        merged, U = ops.castle_attention_packed(proj, H, self.scale, True, capacity, rotary=self.use_rotary, u_half=u_half)
         store = _CacheStore(B, H, d, capacity, proj.dtype, proj.device, U_buffer=U._base.detach())
+        store.u_half = u_half
         qu, _, _, _, kc, vc = self._split(proj)
         with torch.no_grad():
             if self.use_rotary:   # the cache holds the rotated qu / kc rows
@@ -285,11 +304,8 @@ class Castle(nn.Module):
         if cache is None:
             store = _CacheStore(B, H, d, _reserve_rows(1), proj.dtype, proj.device)
         elif store is None:
-            t = cache[0].shape[-2]
-            store = _CacheStore(B, H, d, _reserve_rows(t + 1), proj.dtype, proj.device)
-            for buf, src in zip(store.buffers, cache):
-                buf[:, :, :t].copy_(src)
-            store.length = store.base0 = t
+            store = _CacheStore(B, H, d, _reserve_rows(cache[0].shape[-2] + 1), proj.dtype, proj.device)
+            store.adopt(cache)
         elif store.length != cache.kc_cache.shape[-2]:   # (not cache.U: reading it would write the pending keys back)
             raise RuntimeError("this cache was already advanced by a later decode step; the native "
                                "decode updates its cache in place, so a cache can be used once")
@@ -301,11 +317,11 @@ class Castle(nn.Module):
         deferred = store.deferred()
         if proj.is_contiguous() and proj.data_ptr() % 16 == 0:
             ops.castle_decode_step_packed(store.views, store.capacity, t, proj, H, self.scale, out, store.workspace,
-                                          rotary=self.use_rotary, deferred=deferred)
+                                          rotary=self.use_rotary, deferred=deferred, u_half=store.u_half)
         else:
             ops.castle_decode_step_hip(*store.buffers, t, qc, kc, vc, qu, ku, vu, self.scale,
                                        out.permute(0, 2, 1, 3), store.workspace, rotary=self.use_rotary,
-                                       deferred=deferred)
+                                       deferred=deferred, u_half=store.u_half)
         if deferred is None:
             store.base0 = t + 1   # this step wrote the lookahead keys itself: nothing is pending
         store.length = t + 1
@@ -325,7 +341,8 @@ class Castle(nn.Module):
         out = torch.empty((B, 1, self.heads, self.dim_head), dtype=proj.dtype, device=proj.device)
         ops.castle_decode_step_packed(store.views, store.capacity, 0, proj, self.heads, self.scale, out,
                                       store.workspace, rotary=self.use_rotary, t_device=t_device,
-                                      deferred=store.deferred(base_device) if base_device is not None else None)
+                                      deferred=store.deferred(base_device) if base_device is not None else None,
+                                      u_half=store.u_half)
         return self._project(self.combine_heads, out.view(B, 1, self.heads * self.dim_head), True, residual=residual)
 
     # -- dense PyTorch formulation (use_triton=False) -------------------------

@@ -192,6 +192,7 @@ int castle_fwd(const castle_view4* qc, const castle_view4* kc, const castle_view
     if (!view_ok(v, es, true)) return CASTLE_ERR_ARG;
   const bool want_U = U != nullptr && U->ptr != nullptr;
   if (want_U && !view_ok(U, es, true)) return CASTLE_ERR_ARG;
+  if ((flags & CASTLE_FLAG_U_HALF) && dtype != CASTLE_BF16) return CASTLE_ERR_DTYPE;   // the format replaces bf16 only
   const Geometry g = geometry(B, H, L, d, es);
   if (workspace == nullptr || reinterpret_cast<uintptr_t>(workspace) % 256 != 0 || workspace_bytes < g.total)
     return CASTLE_ERR_WORKSPACE;
@@ -206,6 +207,7 @@ int castle_fwd(const castle_view4* qc, const castle_view4* kc, const castle_view
   a.qu = to_view(qu); a.ku = to_view(ku); a.vu = to_view(vu);
   a.out = to_view(out);
   a.U = to_view(want_U ? U : nullptr);
+  a.u_half = (flags & CASTLE_FLAG_U_HALF) != 0;
   a.ws = carve(workspace, state, g);
   return castle::launch_fwd(a, dtype, (flags & CASTLE_FLAG_BF16_OPERANDS) != 0, static_cast<hipStream_t>(stream));
 }
@@ -293,6 +295,7 @@ static int decode_step_common(const castle_view4* U, const castle_view4* qu_cach
                               void* workspace, int64_t workspace_bytes, bool static_scratch, void* stream) {
   const int es = elem_size(dtype);
   if (es == 0) return CASTLE_ERR_DTYPE;
+  if ((flags & CASTLE_FLAG_U_HALF) && dtype != CASTLE_BF16) return CASTLE_ERR_DTYPE;
   if (B <= 0 || H <= 0 || t < 0 || capacity <= 0 || !head_dim_ok(d) || (int64_t)B * H > 65535) return CASTLE_ERR_SHAPE;
   if (t_device == nullptr && t >= capacity) return CASTLE_ERR_SHAPE;   // row t would be written past the buffers
   const castle_view4* caches[] = {U, qu_cache, kc_cache, vc_cache};
@@ -325,6 +328,7 @@ static int decode_step_common(const castle_view4* U, const castle_view4* qu_cach
   a.B = B; a.H = H; a.d = d; a.t = t; a.scale = scale;
   a.t_dev = t_device; a.capacity = capacity;
   a.rotary = (flags & CASTLE_FLAG_ROTARY) != 0;
+  a.u_half = (flags & CASTLE_FLAG_U_HALF) != 0;
   a.splits = splits;
   a.U = to_view(U); a.qu_cache = to_view(qu_cache); a.kc_cache = to_view(kc_cache); a.vc_cache = to_view(vc_cache);
   a.qc = to_view(qc); a.kc = to_view(kc); a.vc = to_view(vc);
@@ -375,9 +379,10 @@ int castle_decode_step_device_count(const castle_view4* U, const castle_view4* q
 }
 
 int castle_decode_flush(const castle_view4* U, const castle_view4* qu_cache, int t, const castle_deferred* deferred,
-                        int B, int H, int d, int dtype, float scale, void* stream) {
+                        int B, int H, int d, int dtype, float scale, int flags, void* stream) {
   const int es = elem_size(dtype);
   if (es == 0) return CASTLE_ERR_DTYPE;
+  if ((flags & CASTLE_FLAG_U_HALF) && dtype != CASTLE_BF16) return CASTLE_ERR_DTYPE;
   if (B <= 0 || H <= 0 || t < 0 || !head_dim_ok(d) || (int64_t)B * H > 65535) return CASTLE_ERR_SHAPE;
   if (!view_ok(U, es, true) || !view_ok(qu_cache, es, true) || deferred == nullptr) return CASTLE_ERR_ARG;
   if (!view_ok(&deferred->vu_ring, es, true) || !view_ok(&deferred->gates, 4, false)) return CASTLE_ERR_ARG;
@@ -388,6 +393,7 @@ int castle_decode_flush(const castle_view4* U, const castle_view4* qu_cache, int
   a.U = to_view(U); a.qu_cache = to_view(qu_cache);
   a.pend_vu = to_view(&deferred->vu_ring); a.pend_gate = to_view(&deferred->gates);
   a.base0 = deferred->base;
+  a.u_half = (flags & CASTLE_FLAG_U_HALF) != 0;
   return castle::launch_decode_flush(a, dtype, static_cast<hipStream_t>(stream));
 }
 

@@ -26,6 +26,33 @@ template <typename T, int N> __device__ __forceinline__ void load_f32(const T* p
   for (int e = 0; e < N; ++e) dst[e] = (float)x[e];
 }
 
+// One 16-byte piece of a U row to fp32 and back.  UH: the buffer is in the half-precision cache
+// format (fp16 bits of U * kUHalfScale, saturated) whatever the element type T of the cache is.
+template <typename T, int N, bool UH> __device__ __forceinline__ void u_unpack(vec<T, N> raw, float (&dst)[N]) {
+  if constexpr (UH) {
+    static_assert(sizeof(T) == 2, "the half-precision format replaces a 16-bit element type");
+    const vec<fp16_t, N> x = __builtin_bit_cast(vec<fp16_t, N>, raw);
+#pragma unroll
+    for (int e = 0; e < N; ++e) dst[e] = (float)x[e] * kUHalfUnscale;
+  } else {
+#pragma unroll
+    for (int e = 0; e < N; ++e) dst[e] = (float)raw[e];
+  }
+}
+template <typename T, int N, bool UH> __device__ __forceinline__ vec<T, N> u_pack(const float (&src)[N]) {
+  if constexpr (UH) {
+    vec<fp16_t, N> x;
+#pragma unroll
+    for (int e = 0; e < N; ++e) x[e] = (fp16_t)__builtin_amdgcn_fmed3f(src[e] * kUHalfScale, -kHalfMax, kHalfMax);
+    return __builtin_bit_cast(vec<T, N>, x);
+  } else {
+    vec<T, N> x;
+#pragma unroll
+    for (int e = 0; e < N; ++e) x[e] = (T)src[e];
+    return x;
+  }
+}
+
 template <int LPR> __device__ __forceinline__ float group_sum(float v) {
 #pragma unroll
   for (int o = 1; o < LPR; o <<= 1) v += __shfl_xor(v, o);
@@ -33,7 +60,7 @@ template <int LPR> __device__ __forceinline__ float group_sum(float v) {
 }
 
 // One workgroup = 4 waves; a group of LPR = d / V lanes owns one cache row per iteration.
-template <typename T, int HD>
+template <typename T, int HD, bool UH>
 __global__ __launch_bounds__(kThreads) void decode_stream_kernel(DecodeArgs a) {
   constexpr int V = elem_traits<T>::vec16;   // elements per 16-byte lane load
   constexpr int LPR = HD / V;                // lanes per row
@@ -112,7 +139,8 @@ __global__ __launch_bounds__(kThreads) void decode_stream_kernel(DecodeArgs a) {
       float quk[V], uk[V], kck[V], vck[V];
       T* urow = view_row<T>(a.U, b, h, k) + sub * V;
 #pragma unroll
-      for (int e = 0; e < V; ++e) { quk[e] = (float)cq[e]; uk[e] = (float)cu[e]; kck[e] = (float)ck[e]; vck[e] = (float)cv[e]; }
+      for (int e = 0; e < V; ++e) { quk[e] = (float)cq[e]; kck[e] = (float)ck[e]; vck[e] = (float)cv[e]; }
+      u_unpack<T, V, UH>(cu, uk);
       // pending sources j > k first (none unless the write-back is deferred): their gates were
       // formed by the steps that appended them and wait in the row's side array
       float* grow = deferred ? gbase + (int64_t)k * kDecodeDefer : nullptr;
@@ -130,19 +158,20 @@ __global__ __launch_bounds__(kThreads) void decode_stream_kernel(DecodeArgs a) {
       for (int e = 0; e < V; ++e) dg = __builtin_fmaf(quk[e], ku[e], dg);
       dg = group_sum<LPR>(dg);
       const float gate = sigmoid_l2(dg * c1);
-      vt unew;
 #pragma unroll
-      for (int e = 0; e < V; ++e) {
-        uk[e] = __builtin_fmaf(gate, vu[e], uk[e]);
-        unew[e] = (T)uk[e];
+      for (int e = 0; e < V; ++e) uk[e] = __builtin_fmaf(gate, vu[e], uk[e]);
+      if (write_u) {
+        // the lookahead key as later steps will see it: the stored (rounded) one when it is written now
+        const vt unew = u_pack<T, V, UH>(uk);
+        *reinterpret_cast<vt*>(urow) = unew;
+        u_unpack<T, V, UH>(unew, uk);
+      } else if (sub == 0) {
+        grow[slot_t] = gate;   // the new token stays pending: its gate for this row
       }
-      if (write_u) *reinterpret_cast<vt*>(urow) = unew;
-      else if (sub == 0) grow[slot_t] = gate;   // the new token stays pending: its gate for this row
       float dsu = 0.f, dsc = 0.f;
 #pragma unroll
       for (int e = 0; e < V; ++e) {
-        // the lookahead key as later steps will see it: the stored (rounded) one when it is written now
-        dsu = __builtin_fmaf(qc[e], write_u ? (float)unew[e] : uk[e], dsu);
+        dsu = __builtin_fmaf(qc[e], uk[e], dsu);
         dsc = __builtin_fmaf(qc[e], kck[e], dsc);
       }
       dsu = group_sum<LPR>(dsu);
@@ -288,7 +317,7 @@ __global__ __launch_bounds__(64) void decode_finish_kernel(DecodeArgs a) {
 
 // Folds the pending sources into the stored lookahead keys (rows 0 .. t-1), for a reader that wants
 // the cache tensor U itself: U_k += sum over pending j > k of sigmoid(s qu_k . ku_j) vu_j.
-template <typename T, int HD>
+template <typename T, int HD, bool UH>
 __global__ __launch_bounds__(kThreads) void decode_flush_kernel(DecodeArgs a) {
   constexpr int V = elem_traits<T>::vec16;
   constexpr int LPR = HD / V;
@@ -311,7 +340,7 @@ __global__ __launch_bounds__(kThreads) void decode_flush_kernel(DecodeArgs a) {
   for (int k = blockIdx.x * RPI + grp; k < t; k += gridDim.x * RPI) {
     float uk[V];
     T* urow = view_row<T>(a.U, b, h, k) + sub * V;
-    load_f32<T, V>(urow, uk);
+    u_unpack<T, V, UH>(*reinterpret_cast<const vt*>(urow), uk);
     const vec<float, 4> g4 = *reinterpret_cast<const vec<float, 4>*>(
         reinterpret_cast<const float*>(a.pend_gate.ptr) + (int64_t)b * a.pend_gate.sb + (int64_t)h * a.pend_gate.sh + (int64_t)k * kDecodeDefer);
 #pragma unroll
@@ -321,10 +350,7 @@ __global__ __launch_bounds__(kThreads) void decode_flush_kernel(DecodeArgs a) {
 #pragma unroll
       for (int e = 0; e < V; ++e) uk[e] = __builtin_fmaf(gj, pv[sl][e], uk[e]);
     }
-    vt unew;
-#pragma unroll
-    for (int e = 0; e < V; ++e) unew[e] = (T)uk[e];
-    *reinterpret_cast<vt*>(urow) = unew;
+    *reinterpret_cast<vt*>(urow) = u_pack<T, V, UH>(uk);
   }
 }
 
@@ -332,7 +358,12 @@ template <typename T, int HD> static int launch_decode_t(const DecodeArgs& a, hi
   const int BH = a.B * a.H;
   if (a.t_dev != nullptr || a.t > 0) {
     ProfScope ps(kSlotDecodeStream, stream);
-    hipLaunchKernelGGL((decode_stream_kernel<T, HD>), dim3(a.splits, BH), dim3(kThreads), 0, stream, a);
+    if constexpr (__is_same(T, bf16_t)) {
+      if (a.u_half) hipLaunchKernelGGL((decode_stream_kernel<T, HD, true>), dim3(a.splits, BH), dim3(kThreads), 0, stream, a);
+      else hipLaunchKernelGGL((decode_stream_kernel<T, HD, false>), dim3(a.splits, BH), dim3(kThreads), 0, stream, a);
+    } else {
+      hipLaunchKernelGGL((decode_stream_kernel<T, HD, false>), dim3(a.splits, BH), dim3(kThreads), 0, stream, a);
+    }
   }
   {
     ProfScope ps(kSlotDecodeFinish, stream);
@@ -341,16 +372,22 @@ template <typename T, int HD> static int launch_decode_t(const DecodeArgs& a, hi
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
+template <typename T, int HD> static void launch_flush_t(const DecodeArgs& a, dim3 grid, hipStream_t stream) {
+  if constexpr (__is_same(T, bf16_t)) {
+    if (a.u_half) { hipLaunchKernelGGL((decode_flush_kernel<T, HD, true>), grid, dim3(kThreads), 0, stream, a); return; }
+  }
+  hipLaunchKernelGGL((decode_flush_kernel<T, HD, false>), grid, dim3(kThreads), 0, stream, a);
+}
 template <typename T> static int launch_flush_d(const DecodeArgs& a, hipStream_t stream) {
   const int BH = a.B * a.H;
   int gx = (640 + BH - 1) / BH;
   if (gx > 64) gx = 64;
-  const dim3 grid(gx, BH), block(kThreads);
+  const dim3 grid(gx, BH);
   switch (a.d) {
-    case 16: hipLaunchKernelGGL((decode_flush_kernel<T, 16>), grid, block, 0, stream, a); break;
-    case 32: hipLaunchKernelGGL((decode_flush_kernel<T, 32>), grid, block, 0, stream, a); break;
-    case 64: hipLaunchKernelGGL((decode_flush_kernel<T, 64>), grid, block, 0, stream, a); break;
-    case 128: hipLaunchKernelGGL((decode_flush_kernel<T, 128>), grid, block, 0, stream, a); break;
+    case 16: launch_flush_t<T, 16>(a, grid, stream); break;
+    case 32: launch_flush_t<T, 32>(a, grid, stream); break;
+    case 64: launch_flush_t<T, 64>(a, grid, stream); break;
+    case 128: launch_flush_t<T, 128>(a, grid, stream); break;
     default: return -2;
   }
   return hipGetLastError() == hipSuccess ? 0 : -3;

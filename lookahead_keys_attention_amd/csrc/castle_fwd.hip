@@ -274,16 +274,28 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(FwdArgs a) {
   if (a.U.ptr != nullptr && k < L) {
     TI* dst = head_ptr_mut<TI>(a.U, b, h) + (int64_t)k * a.U.sl;
     const float su_mul = a.ws.hdr->su_mul;   // the state was built from vu * vu_scale
+    bool half_format = false;
+    if constexpr (sizeof(TI) == 2) half_format = a.u_half != 0;
+    const float mul = half_format ? su_mul * kUHalfScale : su_mul;
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) st[nt][r] *= su_mul;
+      for (int r = 0; r < 16; ++r) st[nt][r] *= mul;
+    if (half_format) {   // half-precision cache format: fp16 bits of U * kUHalfScale, saturated
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) st[nt][r] = __builtin_amdgcn_fmed3f(st[nt][r], -kHalfMax, kHalfMax);
+    }
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int n = 32 * nt + 8 * q + 4 * g;
-        if (n < HD) st4<TI>(dst + n, pack4<TI>(st[nt], q));
+        if (n < HD) {
+          if (half_format) st4<fp16_t>(reinterpret_cast<fp16_t*>(dst + n), pack4<fp16_t>(st[nt], q));
+          else st4<TI>(dst + n, pack4<TI>(st[nt], q));
+        }
       }
   }
 }

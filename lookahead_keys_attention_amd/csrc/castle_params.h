@@ -58,6 +58,7 @@ struct FwdArgs {
   View4 U;        // ptr == nullptr when the final lookahead keys are not wanted
   FwdWorkspace ws;
   int with_t = 1; // the scan launch also fills the T' blocks (0 when only the snapshots are recomputed for a backward pass)
+  int u_half = 0; // U is written in the half-precision cache format (see kUHalfScale) instead of the tensor type
 };
 
 struct BwdArgs {
@@ -78,6 +79,16 @@ struct BwdArgs {
   void* dsu_mat;  // dSu
 };
 
+// Half-precision cache format of the lookahead keys, for bf16 caches: the U buffer holds IEEE fp16
+// values of U * kUHalfScale, saturated at +-65504, in the same 2 bytes per element.  The cached step
+// rounds every U row once per write-back; bf16 keeps 8 significant bits, fp16 keeps 11, so the
+// rounding noise a long decode accumulates is 8 times smaller.  The power-of-two factor moves the
+// fp16 window to |U| in [2^-18, 4.2e6]: below it the absolute error (4e-6) is far under what a bf16
+// value of any score-relevant size carries; above it the silu term of that key's score has long
+// saturated (the key is masked out either way).
+constexpr float kUHalfScale = 0.015625f;   // 2^-6
+constexpr float kUHalfUnscale = 64.f;
+
 // size of the per-GPU partial-result array behind castle_decode_step_static
 constexpr int64_t kDecodeStaticScratchBytes = (int64_t)4 << 20;
 
@@ -95,6 +106,7 @@ struct DecodeArgs {
   int splits;       // partitions of the t rows per (b, h)
   float scale;
   int rotary;       // 1: the new token's qc, kc, qu, ku, vu are rotated by position t
+  int u_half;       // 1: the U buffer is in the half-precision cache format (kUHalfScale)
   View4 U, qu_cache, kc_cache, vc_cache;   // capacity buffers, row t is appended
   View4 qc, kc, vc, qu, ku, vu;            // new token, L == 1
   View4 out;                               // (B, H, 1, d)

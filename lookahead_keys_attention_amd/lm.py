@@ -112,7 +112,8 @@ class GraphedDecoder:
         mine = self.stores[0].buffers[0]
         return (first is not None and max_len <= self.capacity and self.signature == self._signature()
                 and first.buffers[0].shape[:2] == mine.shape[:2] and first.buffers[0].shape[3] == mine.shape[3]
-                and first.buffers[0].dtype == mine.dtype and first.buffers[0].device == mine.device)
+                and first.buffers[0].dtype == mine.dtype and first.buffers[0].device == mine.device
+                and first.u_half == self.stores[0].u_half)
 
     def load(self, caches):
         """Restarts the decoder from the caches of a new prefill: their rows are copied into the

@@ -34,6 +34,10 @@ KEEP_STATE_LIMIT_BYTES = 8 << 30
 # The native cached step writes the lookahead keys back on every 4th step only (pending tokens are
 # applied on the fly; see castle_deferred in include/castle_hip.h).  False: every step writes U.
 DEFER_LOOKAHEAD_WRITES = True
+# bf16 decode caches made by the module keep their lookahead keys in the half-precision cache format
+# (fp16 bits of U / 64 in the same buffer: CASTLE_FLAG_U_HALF in include/castle_hip.h), which takes the
+# rounding noise of a long decode down by a factor of 8.  False: the buffer holds plain bf16.
+LOOKAHEAD_KEYS_HALF = True
 # Debugging aid: when True every parallel forward waits for its kernels and raises if they had to
 # clamp a value to the fp16 range (an input element of a bf16 tensor beyond +-65504, or a T' entry):
 # the result is then that of the clamped operands.  Off by default because it synchronises.
@@ -96,6 +100,7 @@ def _bwd_raw(qc, kc, vc, qu, ku, vu, out, dout, scale, grads, ws, state, flags=0
     B, H, L, d = qc.shape
     code = N.dtype_code(qc.dtype)
     lib = N.lib()
+    flags &= ~N.FLAG_U_HALF   # describes the forward's U output only
     if state.numel() == 0:
         flags |= N.FLAG_RECOMPUTE_STATE
     nbytes = N.check(lib.castle_bwd_workspace_bytes(B, H, L, d, code, int(flags)), "castle_bwd_workspace_bytes")
@@ -284,14 +289,26 @@ def castle_attention_hip(q, k, v, qu, ku, vu, scale, return_U_for_cache=False, r
     return (out, U) if return_U_for_cache else out
 
 
-def castle_attention_packed(proj, heads, scale, return_U_for_cache=False, row_capacity=0, rotary=False):
+def castle_attention_packed(proj, heads, scale, return_U_for_cache=False, row_capacity=0, rotary=False, u_half=False):
     """proj (B, L, 6*H*d) -> merged out (B, L, H*d), or (out, U).  U is (B,H,L,d); with
     `row_capacity` > L it is the first L rows of a freshly allocated (B,H,row_capacity,d) buffer
-    (reachable as U._base), which a decode cache can adopt as its U buffer without a copy."""
-    flags = DEFAULT_FLAGS | (N.FLAG_ROTARY if rotary else 0)
+    (reachable as U._base), which a decode cache can adopt as its U buffer without a copy.
+    `u_half` (bf16 only): U comes back in the half-precision cache format (`decode_lookahead_keys`
+    reads it), the format the cached step then keeps it in."""
+    flags = DEFAULT_FLAGS | (N.FLAG_ROTARY if rotary else 0) | (N.FLAG_U_HALF if u_half and return_U_for_cache else 0)
     merged, U, _, _ = torch.ops.castle_hip.attention_packed(proj, int(heads), float(scale), bool(return_U_for_cache),
                                                          int(row_capacity), int(flags))
     return (merged, U[:, :, : proj.shape[1]]) if return_U_for_cache else merged
+
+
+def decode_lookahead_keys(raw: torch.Tensor) -> torch.Tensor:
+    """A bf16-typed buffer in the half-precision cache format -> the lookahead keys as a new bf16 tensor."""
+    return (raw.view(torch.float16).to(torch.float32) * N.U_HALF_UNSCALE).to(raw.dtype)
+
+
+def encode_lookahead_keys(U: torch.Tensor, out: torch.Tensor):
+    """Writes lookahead keys into `out` (same shape, bf16-typed) in the half-precision cache format."""
+    out.view(torch.float16).copy_((U.to(torch.float32) / N.U_HALF_UNSCALE).clamp_(-65504.0, 65504.0))
 
 
 def decode_workspace(B, H, d, device):
@@ -301,12 +318,13 @@ def decode_workspace(B, H, d, device):
 
 @torch.no_grad()
 def castle_decode_step_hip(U, qu_cache, kc_cache, vc_cache, t, qc, kc, vc, qu, ku, vu, scale, out, workspace,
-                           rotary=False, deferred=None):
+                           rotary=False, deferred=None, u_half=False):
     """In-place cached step.  The four cache tensors are (B,H,capacity,d) buffers with t valid
     rows (capacity > t); the new-token operands and `out` are (B,H,1,d).  rotary=True rotates the
     new token by position t inside the kernels (the cache rows are stored rotated).  `deferred`: a
     `_native.Deferred` (pending-token buffers and a base row count, `make_deferred`) makes the kernels write the
-    lookahead keys on every 4th step only; `castle_decode_flush` completes them in between."""
+    lookahead keys on every 4th step only; `castle_decode_flush` completes them in between.
+    `u_half` (bf16 only): the U buffer is in the half-precision cache format."""
     _require_gpu(U, "castle_decode_step_hip")
     B, H, cap, d = U.shape
     if not (0 <= t < cap):
@@ -319,7 +337,7 @@ def castle_decode_step_hip(U, qu_cache, kc_cache, vc_cache, t, qc, kc, vc, qu, k
     tviews = [N.view4(x) for x in toks]
     with torch.cuda.device(U.device):
         rc = N.lib().castle_decode_step(*views, int(t), int(cap), *tviews, B, H, d, code, float(scale),
-                                        N.FLAG_ROTARY if rotary else 0, N.view4(out), deferred,
+                                        (N.FLAG_ROTARY if rotary else 0) | (N.FLAG_U_HALF if u_half else 0), N.view4(out), deferred,
                                         workspace.data_ptr(), workspace.numel(), N.stream_ptr(U.device))
     N.check(rc, "castle_decode_step")
     return out
@@ -334,12 +352,13 @@ def make_deferred(vu_ring, gates, base, base_device=None):
 
 
 @torch.no_grad()
-def castle_decode_flush(U, qu_cache, t, deferred, scale):
-    """Folds the pending sources into the stored lookahead keys U[:, :, :t] (see castle_deferred)."""
+def castle_decode_flush(U, qu_cache, t, deferred, scale, u_half=False):
+    """Folds the pending sources into the stored lookahead keys U[:, :, :t] (see castle_deferred).  The
+    caller then sets the base row count of its castle_deferred (host and device copy) to t."""
     B, H, _, d = U.shape
     with torch.cuda.device(U.device):
         rc = N.lib().castle_decode_flush(N.view4(U), N.view4(qu_cache), int(t), deferred, B, H, d, N.dtype_code(U.dtype),
-                                         float(scale), N.stream_ptr(U.device))
+                                         float(scale), N.FLAG_U_HALF if u_half else 0, N.stream_ptr(U.device))
     N.check(rc, "castle_decode_flush")
 
 
@@ -403,7 +422,7 @@ def castle_rope_hip(x, out, first_position=0):
 
 @torch.no_grad()
 def castle_decode_step_packed(cache_views, capacity, t, proj, heads, scale, out, workspace, rotary=False,
-                              t_device=None, deferred=None):
+                              t_device=None, deferred=None, u_half=False):
     """The cached step for a fused projection: `proj` is the contiguous (B, 1, 6*H*d) output of the
     layer's projection for the new token (order qu, ku, vu, qc, kc, vc), `cache_views` the four
     castle_view4 of the (B, H, capacity, d) cache buffers (built once per buffer set), `out` a
@@ -419,7 +438,7 @@ def castle_decode_step_packed(cache_views, capacity, t, proj, heads, scale, out,
     es, base, part = proj.element_size(), proj.data_ptr(), heads * d
     qu, ku, vu, qc, kc, vc = (N.View4(base + i * part * es, width, d, width) for i in range(6))
     vout = N.View4(out.data_ptr(), heads * d, d, heads * d)
-    flags = N.FLAG_ROTARY if rotary else 0
+    flags = (N.FLAG_ROTARY if rotary else 0) | (N.FLAG_U_HALF if u_half else 0)
     with torch.cuda.device(proj.device):
         if t_device is None:
             if not (0 <= t < capacity):

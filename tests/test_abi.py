@@ -36,7 +36,7 @@ def test_header_symbols_are_exported(lib):
 
 
 def test_version_and_error_strings(lib):
-    assert lib.castle_abi_version() == 4
+    assert lib.castle_abi_version() == 5
     assert lib.castle_error_string(0) == b"ok"
     for code in (-1, -2, -3, -4, -5, -6):
         assert len(lib.castle_error_string(code)) > 3

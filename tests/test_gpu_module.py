@@ -272,15 +272,13 @@ def test_config4_bf16_decode_after_prefill():
     """benchmark configuration 4 at full size: B32, prefill 2048 through the parallel path, then all
     512 cached steps with fresh x_t ~ N(0,1).  The native decode's per-head output (before the
     output projection) of sampled (b, h) is compared at steps 1, 256 and 512 with the oracle's
-    decode_core iterated in fp32 on that head from the oracle's own prefill, and so are the head's
-    lookahead keys in the cache after the last step.  The cache is a bf16 tensor in this
-    configuration, as in the reference, whose step forms `U = U_prev + gate * vu` in the module
-    dtype (lookahead_keys_attention.py:183).  The native step writes the lookahead keys back on every
-    4th step (row counts with (t + 1) % 4 == 0) and carries them in fp32 in between, so the oracle's
-    keys are rounded to bf16 at exactly those steps, like any other bf16 input of the next step.
-    Against a cache kept in fp32 the 128 roundings show: the last step differs from the parallel
-    pass (fp32 state) by about 2.4e-2 normwise (4.9e-2 when every step writes), asserted as a
-    bound here; it is a property of a bf16 cache."""
+    decode_core iterated in fp32 on that head from the oracle's own prefill (nothing of the native
+    step's rounding cadence is imitated), and so are the head's lookahead keys in the cache after the
+    last step.  The reference's step forms `U = U_prev + gate * vu` in the module dtype
+    (lookahead_keys_attention.py:183): in bf16 that is 512 roundings of every row to 8 significant
+    bits, and its last step then differs from its own parallel pass by about 5e-2 normwise.  The native
+    cache writes the keys back on every 4th step and holds them with 11 significant bits, so parallel
+    and sequential agree inside the 2e-2 rule."""
     m = make(512, 8, 64, dtype=torch.bfloat16, seed=0).eval()
     g = torch.Generator().manual_seed(0)
     steps, t0 = 512, 2048
@@ -298,10 +296,12 @@ def test_config4_bf16_decode_after_prefill():
                 native[n] = merged.view(32, 8, 64).float().cpu()
         # the module's own step (projection included) agrees with the parallel pass on the last row
         full_last = m(x)[:, -1]
-    assert cache.U.shape == (32, 8, t0 + steps, 64)
+    assert cache.U.shape == (32, 8, t0 + steps, 64) and cache.U.dtype == torch.bfloat16
     last = m.combine_heads(merged)[:, 0].double().cpu()
     drift = ((last - full_last.double().cpu()).norm() / full_last.double().norm()).item()
-    assert drift <= 5e-2, f"last cached step vs parallel: {drift:.3e}"
+    worst = ((last - full_last.double().cpu()).abs().max() / full_last.double().abs().max()).item()
+    assert drift <= 2e-2 and worst <= 2e-2, f"last cached step vs parallel: {drift:.3e} normwise, {worst:.3e} of max"
+    gotU_all = cache.U
     for b, h in heads:
         qu, ku, vu, qc, kc, vc = [proj_all[b, :, i, h].float().cpu() for i in range(6)]
         _, U0 = O.parallel_core(*[t[:t0] for t in (qc, kc, vc, qu, ku, vu)], m.scale, want_U=True)
@@ -309,13 +309,7 @@ def test_config4_bf16_decode_after_prefill():
         for n in range(1, steps + 1):
             t = t0 + n - 1
             out, state = O.decode_core(state, *[z[t:t + 1] for z in (qc, kc, vc, qu, ku, vu)], m.scale)
-            if (t + 1) % 4 == 0:
-                state = state._replace(U=state.U.bfloat16().float())
             if n in watch:
                 bf16_close(native[n][b, h], out[0], f"decode step {n} of head ({b},{h}) vs oracle")
-        # 512 independent roundings to bf16 on either side: single elements wander by a few ulps, so the
-        # lookahead keys are held to the normwise half of the bf16 rule
-        gotU = cache.U[b, h].double().cpu()
-        relU = ((gotU - state.U.double()).norm() / state.U.double().norm()).item()
-        assert relU <= 2e-2, f"lookahead keys of head ({b},{h}) after {steps} steps: {relU:.3e}"
+        bf16_close(gotU_all[b, h], state.U, f"lookahead keys of head ({b},{h}) after {steps} steps")
         assert torch.equal(cache.kc_cache[b, h].float().cpu(), kc) and torch.equal(cache.qu_cache[b, h].float().cpu(), qu)

@@ -478,3 +478,61 @@ def test_decode_with_deferred_write_back(B, Hh, t0, steps, d, dtype, rotary):
         err_def = (bufs[0][:, :, :L].cpu().double() - ref_U).norm()
         err_plain = (plain[0][:, :, :L].cpu().double() - ref_U).norm()
         assert err_def <= 1.05 * err_plain
+
+
+@pytest.mark.parametrize("t0,steps,d,rotary", [(0, 21, 64, False), (150, 30, 32, True), (96, 14, 128, False)])
+def test_decode_with_half_precision_lookahead_keys(t0, steps, d, rotary):
+    """CASTLE_FLAG_U_HALF: a bf16 cache whose lookahead-key buffer holds fp16 bits of U / 64.  The
+    forward's U output comes in that format, every step's output equals the oracle's, the flushed
+    buffer decodes (64 * fp16) to the oracle's keys, and it does so more closely than the same steps
+    on a plain bf16 buffer (11 instead of 8 significant bits per write-back)."""
+    from lookahead_keys_attention_amd import _native as N
+
+    B, Hh, dtype = 2, 2, torch.bfloat16
+    L = t0 + steps
+    ops, _ = rand_ops(B, Hh, L, d, dtype, seed=11 * L + d)
+    s = d ** -0.5
+    pos = torch.arange(L)
+    ref = [t.double() if (idx == 2 or not rotary) else O.rope(t.double(), pos) for idx, t in enumerate(ops)]
+    ref_out, ref_U = O.parallel_core(*ref, s, want_U=True)
+    dev_ops = [t.to(DEV) for t in ops]
+
+    def fresh(half):
+        bufs = [torch.zeros(B, Hh, L + 3, d, dtype=dtype, device=DEV) for _ in range(4)]
+        if t0:
+            proj = torch.stack([dev_ops[i][:, :, :t0] for i in (3, 4, 5, 0, 1, 2)], 0)   # qu, ku, vu, qc, kc, vc
+            proj = proj.permute(1, 3, 0, 2, 4).reshape(B, t0, 6 * Hh * d).contiguous()
+            _, U0 = H().castle_attention_packed(proj, Hh, s, True, rotary=rotary, u_half=half)
+            bufs[0][:, :, :t0] = U0
+            for buf, src in zip(bufs[1:], (ref[3], ref[1], ref[2])):
+                buf[:, :, :t0] = src[:, :, :t0].to(dtype).to(DEV)
+        return bufs
+
+    half, plain = fresh(True), fresh(False)
+    if t0:   # the forward wrote the same keys in the two formats
+        U0_ref = O.parallel_core(*[t[:, :, :t0] for t in ref], s, want_U=True)[1]
+        assert_close(H().decode_lookahead_keys(half[0][:, :, :t0]), U0_ref, dtype, "prefill U (half format)", 1e-3)
+    rings = [[torch.zeros(B, Hh, N.DECODE_DEFER, d, dtype=dtype, device=DEV),
+              torch.zeros(B, Hh, L + 3, N.DECODE_DEFER, dtype=torch.float32, device=DEV)] for _ in range(2)]
+    ws = H().decode_workspace(B, Hh, d, DEV)
+    outs = []
+    for t in range(t0, L):
+        tok = [x[:, :, t:t + 1] for x in dev_ops]
+        o = torch.empty(B, Hh, 1, d, dtype=dtype, device=DEV)
+        H().castle_decode_step_hip(*half, t, *tok, s, o, ws, rotary=rotary, deferred=H().make_deferred(*rings[0], t0), u_half=True)
+        H().castle_decode_step_hip(*plain, t, *tok, s, torch.empty_like(o), ws, rotary=rotary, deferred=H().make_deferred(*rings[1], t0))
+        outs.append(o)
+    assert_close(torch.cat(outs, 2), ref_out[:, :, t0:], dtype, "decode out", 1e-3)
+    H().castle_decode_flush(half[0], half[1], L, H().make_deferred(*rings[0], t0), s, u_half=True)
+    H().castle_decode_flush(plain[0], plain[1], L, H().make_deferred(*rings[1], t0), s)
+    got = (half[0][:, :, :L].view(torch.float16).double().cpu() * 64.0)
+    err_half = ((got - ref_U).norm() / ref_U.norm()).item()
+    err_plain = ((plain[0][:, :, :L].double().cpu() - ref_U).norm() / ref_U.norm()).item()
+    assert err_half <= 1.5e-3, f"half-precision keys: {err_half:.3e}"
+    assert err_half <= 0.5 * err_plain, f"half format {err_half:.3e} vs bf16 {err_plain:.3e}"
+    # the rows the steps appended are zero in both formats, and fp16 / fp32 tensors reject the flag
+    with pytest.raises(RuntimeError):
+        f16 = [b.half() for b in plain]
+        H().castle_decode_step_hip(*f16, L, *[x[:, :, :1].half() for x in dev_ops], s, torch.empty(B, Hh, 1, d, dtype=torch.float16, device=DEV),
+                                   ws, u_half=True)
+
