@@ -191,6 +191,8 @@ class RotaryFrequencies(nn.Module):
 
 
 class Castle(nn.Module):
+    _warned_dense_step = False   # the grad-mode fallback of the cached step warns once per process
+
     def __init__(self, dim, heads=8, dim_head=64, use_triton=None, rotary_emb=False, prenorm=False):
         super().__init__()
         self.dim, self.heads, self.dim_head = dim, heads, dim_head
@@ -245,7 +247,18 @@ class Castle(nn.Module):
             native = False   # auto-selected kernels that do not cover this head dimension / type: dense as well
         if single and native and torch.is_grad_enabled() and (
                 x.requires_grad or any(p.requires_grad for p in self.parameters())):
-            native = False   # the native step records no autograd graph; the dense step does
+            # the native step records no autograd graph; the dense step does.  A native cache handed to it
+            # is read out into plain tensors that grow by concatenation: O(t) copies per step from here on
+            if self._explicit_native:
+                raise RuntimeError("Castle(use_triton=True): the native single-token step is inference-only; call it under "
+                                   "torch.no_grad() / torch.inference_mode(), or construct with use_triton=None / False "
+                                   "for a differentiable (dense) step")
+            if getattr(cache, "_store", None) is not None and not Castle._warned_dense_step:
+                Castle._warned_dense_step = True
+                warnings.warn("a single-token call with grad mode on takes the dense PyTorch step (the native step is "
+                              "inference-only); its native cache is copied out and every later step stays dense. "
+                              "Decode under torch.no_grad() to keep the HIP kernels", RuntimeWarning, stacklevel=2)
+            native = False
         native_step = single and native
         proj = self._project(self.to_all_qkv, x, native_step, norm=self.norm)
         if not single:

@@ -13,6 +13,13 @@
 #include "castle_profile.h"
 #include <mutex>
 
+#ifndef CASTLE_DEC_PF
+#define CASTLE_DEC_PF 1   // iterations of row pieces requested ahead in the stream kernel
+#endif
+#ifndef CASTLE_DEC_WGS
+#define CASTLE_DEC_WGS 640   // workgroups the stream kernel aims for
+#endif
+
 namespace castle {
 
 template <typename T> __device__ __forceinline__ T* view_row(const View4& v, int b, int h, int64_t row) {
@@ -115,26 +122,32 @@ __global__ __launch_bounds__(kThreads) void decode_stream_kernel(DecodeArgs a) {
   for (int e = 0; e < V; ++e) acc[e] = 0.f;
   float m = -INFINITY, l = 0.f;
 
-  // The row pieces of the NEXT iteration are requested before the current one is processed: twice
-  // the bytes in flight per wave, which is what a latency-bound streaming loop is short of.
-  vt nq, nu, nk, nv;
-  vec<float, 4> ng = {0.f, 0.f, 0.f, 0.f};
+  // The row pieces of the next PF iterations are requested before the current one is processed:
+  // PF + 1 times the bytes in flight per wave, which is what a latency-bound streaming loop is short of.
+  constexpr int PF = CASTLE_DEC_PF;
+  vt nq[PF], nu[PF], nk[PF], nv[PF];
+  vec<float, 4> ng[PF];
+#pragma unroll
+  for (int p = 0; p < PF; ++p) ng[p] = vec<float, 4>{0.f, 0.f, 0.f, 0.f};
   float* const gbase = deferred ? reinterpret_cast<float*>(a.pend_gate.ptr) + (int64_t)b * a.pend_gate.sb + (int64_t)h * a.pend_gate.sh : nullptr;
-  auto request = [&](int k) __attribute__((always_inline)) {
+  auto request = [&](int p, int k) __attribute__((always_inline)) {
     if (k < r1) {
-      nq = *reinterpret_cast<const vt*>(view_row<T>(a.qu_cache, b, h, k) + sub * V);
-      nu = *reinterpret_cast<const vt*>(view_row<T>(a.U, b, h, k) + sub * V);
-      nk = *reinterpret_cast<const vt*>(view_row<T>(a.kc_cache, b, h, k) + sub * V);
-      nv = *reinterpret_cast<const vt*>(view_row<T>(a.vc_cache, b, h, k) + sub * V);
-      if (np > 0) ng = *reinterpret_cast<const vec<float, 4>*>(gbase + (int64_t)k * kDecodeDefer);
+      nq[p] = *reinterpret_cast<const vt*>(view_row<T>(a.qu_cache, b, h, k) + sub * V);
+      nu[p] = *reinterpret_cast<const vt*>(view_row<T>(a.U, b, h, k) + sub * V);
+      nk[p] = *reinterpret_cast<const vt*>(view_row<T>(a.kc_cache, b, h, k) + sub * V);
+      nv[p] = *reinterpret_cast<const vt*>(view_row<T>(a.vc_cache, b, h, k) + sub * V);
+      if (np > 0) ng[p] = *reinterpret_cast<const vec<float, 4>*>(gbase + (int64_t)k * kDecodeDefer);
     }
   };
-  request(r0 + grp);
-  for (int base = r0; base < r1; base += RPI) {
-    const int k = base + grp;
-    const vt cq = nq, cu = nu, ck = nk, cv = nv;
-    const vec<float, 4> g4 = ng;
-    request(k + RPI);
+#pragma unroll
+  for (int p = 0; p < PF; ++p) request(p, r0 + grp + p * RPI);
+  for (int base = r0; base < r1; base += PF * RPI) {
+#pragma unroll
+    for (int p = 0; p < PF; ++p) {
+    const int k = base + p * RPI + grp;
+    const vt cq = nq[p], cu = nu[p], ck = nk[p], cv = nv[p];
+    const vec<float, 4> g4 = ng[p];
+    request(p, k + PF * RPI);
     if (k < r1) {
       float quk[V], uk[V], kck[V], vck[V];
       T* urow = view_row<T>(a.U, b, h, k) + sub * V;
@@ -178,11 +191,12 @@ __global__ __launch_bounds__(kThreads) void decode_stream_kernel(DecodeArgs a) {
       dsc = group_sum<LPR>(dsc);
       const float x = (dsc - dsu * sigmoid_l2(dsu * c1)) * c1;   // score in log2 units
       const float mn = fmaxf(m, x);
-      const float al = fast_exp2(m - mn), p = fast_exp2(x - mn);
-      l = l * al + p;
+      const float al = fast_exp2(m - mn), p_ = fast_exp2(x - mn);
+      l = l * al + p_;
 #pragma unroll
-      for (int e = 0; e < V; ++e) acc[e] = __builtin_fmaf(p, vck[e], acc[e] * al);
+      for (int e = 0; e < V; ++e) acc[e] = __builtin_fmaf(p_, vck[e], acc[e] * al);
       m = mn;
+    }
     }
   }
   (void)c0;
@@ -595,7 +609,7 @@ int decode_static_scratch(float** ptr) {
 // rows of one (b, h) handled per workgroup iteration, needed by the host to size `splits`
 int decode_pick_splits(int BH, int t) {
   if (t <= 0) return 1;
-  int want = (640 + BH - 1) / BH;           // 2-3 workgroups per CU: measured 6.3 TB/s at 512-768 workgroups, 6.0 at 2048, 4.5 at 256
+  int want = (CASTLE_DEC_WGS + BH - 1) / BH;           // 2-3 workgroups per CU: measured 6.3 TB/s at 512-768 workgroups, 6.0 at 2048, 4.5 at 256
   int max_by_rows = (t + 63) / 64;          // at least 64 rows per workgroup
   int s = want < max_by_rows ? want : max_by_rows;
   if (s < 1) s = 1;

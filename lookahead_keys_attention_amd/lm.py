@@ -20,6 +20,7 @@ import torch
 import torch.nn.functional as F
 from torch import nn
 
+from . import _native
 from .castle import Castle
 
 
@@ -189,7 +190,9 @@ class CastleLM(nn.Module):
             x, target = x[:, :-1], x[:, 1:]
         h = self.token_emb(x)
         # one token per sequence, no graph to record: the few rows of every projection go through the small-M kernel
-        token_step = h.shape[1] == 1 and h.is_cuda and not torch.is_grad_enabled()
+        # (only for a model whose layers run the native kernels: one built with use_triton=False stays on
+        # the PyTorch layers throughout, so it remains an independent baseline for the native one)
+        token_step = h.shape[1] == 1 and not torch.is_grad_enabled() and self._native_on_gpu(h.device)
         next_cache = []
         for index, (attention, feed_forward) in enumerate(self.layers):
             layer_cache = cache[index] if cache is not None and index < len(cache) else None
@@ -221,7 +224,7 @@ class CastleLM(nn.Module):
         self.__dict__.pop("_kept_decoder", None)
 
     def _native_on_gpu(self, device) -> bool:
-        return device.type == "cuda" and all(attention.use_triton for attention, _ in self.layers)
+        return device.type == "cuda" and _native.is_built() and all(attention.use_triton for attention, _ in self.layers)
 
     @torch.no_grad()
     def sample(self, prompt, seq_len, temperature=1.0, filter_thres=0.9, generator=None, graph=None):

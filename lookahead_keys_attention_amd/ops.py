@@ -63,9 +63,9 @@ def _check_dims(d: int, dtype: torch.dtype):
         raise ValueError("float32 HIP kernels support dim_head <= 64")
 
 
-def _fwd_raw(qc, kc, vc, qu, ku, vu, scale, out, U, flags=0):
+def _fwd_raw(qc, kc, vc, qu, ku, vu, scale, out, U, flags=0, keep_state=True):
     """Launch castle_fwd; returns (workspace, state): the tensors the backward pass needs back.
-    `state` is an empty tensor when the snapshots are too large to keep (KEEP_STATE_LIMIT_BYTES)."""
+    `state` is an empty tensor when the caller does not keep the snapshots (`keep_state` False)."""
     B, H, L, d = qc.shape
     code = N.dtype_code(qc.dtype)
     lib = N.lib()
@@ -80,7 +80,7 @@ def _fwd_raw(qc, kc, vc, qu, ku, vu, scale, out, U, flags=0):
         rc = lib.castle_fwd(*views, B, H, L, d, code, float(scale), int(flags), vo, vU, ws.data_ptr(), nbytes,
                             state.data_ptr(), sbytes, N.stream_ptr(qc.device))
     N.check(rc, "castle_fwd")
-    if sbytes > KEEP_STATE_LIMIT_BYTES:
+    if not keep_state:
         state = torch.empty(0, dtype=torch.uint8, device=qc.device)   # the caching allocator keeps the block until the stream is done with it
     if CHECK_RANGE:
         status = range_status(ws)
@@ -134,9 +134,26 @@ def _out_like(q):
     return torch.empty((B, L, H, d), dtype=q.dtype, device=q.device).permute(0, 2, 1, 3)
 
 
-def _fake_state(B, H, L, d, like):
-    n = N.check(N.lib().castle_fwd_state_bytes(int(B), int(H), int(L), int(d), N.dtype_code(like.dtype)), "castle_fwd_state_bytes")
-    return torch.empty(n if n <= KEEP_STATE_LIMIT_BYTES else 0, dtype=torch.uint8, device=like.device)
+def _state_bytes(B, H, L, d, dtype):
+    return N.check(N.lib().castle_fwd_state_bytes(int(B), int(H), int(L), int(d), N.dtype_code(dtype)), "castle_fwd_state_bytes")
+
+
+def _fake_state(B, H, L, d, like, keep_state):
+    return torch.empty(_state_bytes(B, H, L, d, like.dtype) if keep_state else 0, dtype=torch.uint8, device=like.device)
+
+
+def state_bytes_formula(B, H, L, d, element_size) -> int:
+    """castle_fwd_state_bytes in plain Python (64-row blocks over L rounded up to 128; one snapshot row
+    of d elements per key and later block), for callers that a tracing compiler looks into."""
+    nblk = (L + 127) // 128 * 2
+    n = B * H * 64 * (nblk * (nblk - 1) // 2) * d * element_size
+    return max(256, (n + 255) // 256 * 256)
+
+
+def keeps_state(B, H, L, d, dtype) -> bool:
+    """The decision KEEP_STATE_LIMIT_BYTES stands for, taken once per call by the Python callers and
+    handed to the registered operators as an argument (so a traced graph and its execution agree)."""
+    return state_bytes_formula(B, H, L, d, dtype.itemsize) <= KEEP_STATE_LIMIT_BYTES
 
 
 def _fwd_ws_bytes(B, H, L, d, dtype):
@@ -146,24 +163,25 @@ def _fwd_ws_bytes(B, H, L, d, dtype):
 
 @torch.library.custom_op("castle_hip::attention", mutates_args=())
 def _attention_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, qu: torch.Tensor, ku: torch.Tensor,
-                  vu: torch.Tensor, scale: float, want_U: bool, flags: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+                  vu: torch.Tensor, scale: float, want_U: bool, flags: int,
+                  keep_state: bool) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     _require_gpu(q, "castle_attention_hip")
     B, H, L, d = q.shape
     _check_dims(d, q.dtype)
     ops = [_as_readable(t) for t in (q, k, v, qu, ku, vu)]
     out = _out_like(q)
     U = torch.empty((B, H, L, d) if want_U else (0,), dtype=q.dtype, device=q.device)
-    ws, state = _fwd_raw(*ops, scale, out, U if want_U else None, flags)
+    ws, state = _fwd_raw(*ops, scale, out, U if want_U else None, flags, keep_state)
     return out, U, ws, state
 
 
 @_attention_op.register_fake
-def _(q, k, v, qu, ku, vu, scale, want_U, flags):
+def _(q, k, v, qu, ku, vu, scale, want_U, flags, keep_state):
     B, H, L, d = q.shape
     _check_dims(d, q.dtype)
     U = torch.empty((B, H, L, d) if want_U else (0,), dtype=q.dtype, device=q.device)
     ws = torch.empty(_fwd_ws_bytes(B, H, L, d, q.dtype), dtype=torch.uint8, device=q.device)
-    return _out_like(q), U, ws, _fake_state(B, H, L, d, q)
+    return _out_like(q), U, ws, _fake_state(B, H, L, d, q, keep_state)
 
 
 @torch.library.custom_op("castle_hip::attention_bwd", mutates_args=())
@@ -183,7 +201,7 @@ def _(q, k, v, qu, ku, vu, out, dout, ws, state, scale, flags):
 
 
 def _attention_setup(ctx, inputs, output):
-    q, k, v, qu, ku, vu, scale, want_U, flags = inputs
+    q, k, v, qu, ku, vu, scale, want_U, flags, keep_state = inputs
     out, U, ws, state = output
     ctx.save_for_backward(q, k, v, qu, ku, vu, out, ws, state)
     ctx.scale, ctx.flags = scale, flags
@@ -198,7 +216,7 @@ def _attention_backward(ctx, dout, dU, dws, dstate):
     if dout is None:
         dout = torch.zeros_like(out)
     grads = torch.ops.castle_hip.attention_bwd(q, k, v, qu, ku, vu, out, dout, ws, state, ctx.scale, ctx.flags)
-    return (*grads.unbind(0), None, None, None)
+    return (*grads.unbind(0), None, None, None, None)
 
 
 _attention_op.register_autograd(_attention_backward, setup_context=_attention_setup)
@@ -217,7 +235,7 @@ def _packed_ok(t):
 
 @torch.library.custom_op("castle_hip::attention_packed", mutates_args=())
 def _attention_packed_op(proj: torch.Tensor, heads: int, scale: float, want_U: bool, row_capacity: int,
-                         flags: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+                         flags: int, keep_state: bool) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     # The lookahead keys come back as the first L rows of a (B, H, row_capacity, d) buffer, so that a
     # caller can hand over the U buffer of a decode cache without copying (row_capacity >= L).
     _require_gpu(proj, "castle_attention_packed")
@@ -228,18 +246,18 @@ def _attention_packed_op(proj: torch.Tensor, heads: int, scale: float, want_U: b
     merged = torch.empty((B, L, heads * d), dtype=proj.dtype, device=proj.device)
     out = merged.view(B, L, heads, d).permute(0, 2, 1, 3)
     U = torch.empty((B, heads, max(row_capacity, L), d) if want_U else (0,), dtype=proj.dtype, device=proj.device)
-    ws, state = _fwd_raw(qc, kc, vc, qu, ku, vu, scale, out, U[:, :, :L] if want_U else None, flags)
+    ws, state = _fwd_raw(qc, kc, vc, qu, ku, vu, scale, out, U[:, :, :L] if want_U else None, flags, keep_state)
     return merged, U, ws, state
 
 
 @_attention_packed_op.register_fake
-def _(proj, heads, scale, want_U, row_capacity, flags):
+def _(proj, heads, scale, want_U, row_capacity, flags, keep_state):
     B, L, width = proj.shape
     d = width // (6 * heads)
     _check_dims(d, proj.dtype)
     ws = torch.empty(_fwd_ws_bytes(B, heads, L, d, proj.dtype), dtype=torch.uint8, device=proj.device)
     U = torch.empty((B, heads, max(row_capacity, L), d) if want_U else (0,), dtype=proj.dtype, device=proj.device)
-    return torch.empty((B, L, heads * d), dtype=proj.dtype, device=proj.device), U, ws, _fake_state(B, heads, L, d, proj)
+    return torch.empty((B, L, heads * d), dtype=proj.dtype, device=proj.device), U, ws, _fake_state(B, heads, L, d, proj, keep_state)
 
 
 @torch.library.custom_op("castle_hip::attention_packed_bwd", mutates_args=())
@@ -262,7 +280,7 @@ def _(proj, merged, dmerged, ws, state, heads, scale, flags):
 
 
 def _packed_setup(ctx, inputs, output):
-    proj, heads, scale, want_U, row_capacity, flags = inputs
+    proj, heads, scale, want_U, row_capacity, flags, keep_state = inputs
     merged, U, ws, state = output
     ctx.save_for_backward(proj, merged, ws, state)
     ctx.heads, ctx.scale, ctx.flags = heads, scale, flags
@@ -275,7 +293,7 @@ def _packed_backward(ctx, dmerged, dU, dws, dstate):
     if dmerged is None:
         dmerged = torch.zeros_like(merged)
     dproj = torch.ops.castle_hip.attention_packed_bwd(proj, merged, dmerged, ws, state, ctx.heads, ctx.scale, ctx.flags)
-    return dproj, None, None, None, None, None
+    return dproj, None, None, None, None, None, None
 
 
 _attention_packed_op.register_autograd(_packed_backward, setup_context=_packed_setup)
@@ -285,7 +303,10 @@ def castle_attention_hip(q, k, v, qu, ku, vu, scale, return_U_for_cache=False, r
     """Drop-in for castle_attention_triton: returns out, or (out, U).  rotary=True applies the
     rotary position embedding (positions 0..L-1) to q, k, qu, ku, vu inside the kernels."""
     flags = DEFAULT_FLAGS | (N.FLAG_ROTARY if rotary else 0)
-    out, U, _, _ = torch.ops.castle_hip.attention(q, k, v, qu, ku, vu, float(scale), bool(return_U_for_cache), int(flags))
+    B, H, L, d = q.shape
+    _check_dims(d, q.dtype)
+    out, U, _, _ = torch.ops.castle_hip.attention(q, k, v, qu, ku, vu, float(scale), bool(return_U_for_cache), int(flags),
+                                                  keeps_state(B, H, L, d, q.dtype))
     return (out, U) if return_U_for_cache else out
 
 
@@ -296,8 +317,11 @@ def castle_attention_packed(proj, heads, scale, return_U_for_cache=False, row_ca
     `u_half` (bf16 only): U comes back in the half-precision cache format (`decode_lookahead_keys`
     reads it), the format the cached step then keeps it in."""
     flags = DEFAULT_FLAGS | (N.FLAG_ROTARY if rotary else 0) | (N.FLAG_U_HALF if u_half and return_U_for_cache else 0)
+    B, L, width = proj.shape
+    _check_dims(width // (6 * int(heads)), proj.dtype)
     merged, U, _, _ = torch.ops.castle_hip.attention_packed(proj, int(heads), float(scale), bool(return_U_for_cache),
-                                                         int(row_capacity), int(flags))
+                                                         int(row_capacity), int(flags),
+                                                         keeps_state(B, int(heads), L, width // (6 * int(heads)), proj.dtype))
     return (merged, U[:, :, : proj.shape[1]]) if return_U_for_cache else merged
 
 
@@ -368,7 +392,7 @@ SMALL_LINEAR_MAX_ROWS = 64
 def small_linear_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:
     """True if `small_linear` can replace F.linear(x, weight) for this call: a few rows, 16-bit GPU
     tensors, K-contiguous rows that the kernels can read 16 bytes at a time."""
-    return (x.is_cuda and x.dtype in (torch.bfloat16, torch.float16) and weight.dtype == x.dtype
+    return (N.is_built() and x.is_cuda and x.dtype in (torch.bfloat16, torch.float16) and weight.dtype == x.dtype
             and x.dim() == 3 and x.shape[1] == 1 and x.shape[0] <= SMALL_LINEAR_MAX_ROWS
             and x.stride(2) == 1 and weight.stride(1) == 1 and x.shape[2] % 8 == 0 and weight.shape[0] % 2 == 0
             and x.stride(0) % 8 == 0 and weight.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)

@@ -60,6 +60,14 @@ def test_workspace_sizes(lib):
     assert lib.castle_decode_workspace_bytes(32, 8, 64, 4096) > 0
 
 
+def test_state_size_formula_of_the_python_callers_matches_the_library(lib):
+    from lookahead_keys_attention_amd import ops
+
+    for B, H, L, d, dtype, es in ((4, 8, 4096, 64, 1, 2), (1, 16, 16384, 128, 1, 2), (2, 2, 100, 32, 0, 4), (1, 1, 129, 16, 2, 2),
+                                  (3, 5, 128, 64, 0, 4)):
+        assert ops.state_bytes_formula(B, H, L, d, es) == lib.castle_fwd_state_bytes(B, H, L, d, dtype)
+
+
 def test_rejects_bad_shapes_and_types(lib):
     assert lib.castle_fwd_workspace_bytes(1, 1, 16, 48, 1) == -2      # head dim not supported
     assert lib.castle_fwd_workspace_bytes(1, 1, 16, 128, 0) == -2     # fp32 needs d <= 64

@@ -13,6 +13,9 @@ def test_operators_are_registered_with_schemas():
         assert hasattr(torch.ops.castle_hip, name)
     schema = str(torch.ops.castle_hip.attention.default._schema)
     assert "Tensor q" in schema and "float scale" in schema and "bool want_U" in schema
+    # whether the forward keeps its state snapshots is an argument, not a global read inside the operator:
+    # the fake and the real implementation cannot disagree about the size of the `state` output
+    assert "bool keep_state" in schema and "bool keep_state" in str(torch.ops.castle_hip.attention_packed.default._schema)
     assert "!" not in schema and "!" not in str(torch.ops.castle_hip.attention_packed.default._schema)   # functional
 
 
@@ -34,6 +37,10 @@ def test_fake_tensor_forward_and_backward_of_the_six_operand_operator():
         assert merged.shape == (2, 100, 3 * 64) and U.shape == (2, 3, 100, 64) and U._base.shape == (2, 3, 150, 64)
         merged.sum().backward()
         assert proj.grad.shape == proj.shape
+        # the state output follows the argument, in the fake implementation as in the real one
+        for keep in (True, False):
+            _, _, _, state = torch.ops.castle_hip.attention_packed(proj.detach(), 3, 0.125, False, 0, 0, keep)
+            assert (state.numel() > 0) == keep
 
 
 def test_fake_tensor_trace_of_the_module():
@@ -55,10 +62,10 @@ def test_fake_tensor_trace_of_the_module():
 def test_opcheck_on_the_gpu():
     g = torch.Generator().manual_seed(0)
     six = [(torch.randn(1, 2, 96, 32, generator=g) * 0.6).to("cuda").requires_grad_() for _ in range(6)]
-    torch.library.opcheck(torch.ops.castle_hip.attention.default, (*six, 32 ** -0.5, True, 0),
+    torch.library.opcheck(torch.ops.castle_hip.attention.default, (*six, 32 ** -0.5, True, 0, True),
                           test_utils=("test_schema", "test_faketensor", "test_autograd_registration"))
     proj = (torch.randn(2, 70, 6 * 2 * 32, generator=g) * 0.6).to("cuda").requires_grad_()
-    torch.library.opcheck(torch.ops.castle_hip.attention_packed.default, (proj, 2, 32 ** -0.5, True, 128, 0),
+    torch.library.opcheck(torch.ops.castle_hip.attention_packed.default, (proj, 2, 32 ** -0.5, True, 128, 0, True),
                           test_utils=("test_schema", "test_faketensor", "test_autograd_registration"))
 
 

@@ -126,6 +126,35 @@ def test_reading_the_lookahead_keys_mid_window_completes_them():
             assert (U.cpu() - oc.U).abs().max() <= 1e-3 and (kc_c.cpu() - oc.kc_cache).abs().max() <= 1e-5
 
 
+def test_single_token_step_with_grad_mode_on():
+    """The native cached step is inference-only.  Castle(use_triton=True) says so when a single-token
+    call would need a graph (grad mode on, parameters requiring grad) instead of silently going
+    dense; an auto-selected module (use_triton=None) takes the differentiable dense step, as the
+    reference's module would, and warns once that the native cache is copied out."""
+    from lookahead_keys_attention_amd import Castle
+
+    m = make(32, 2, 16)
+    x = torch.randn(1, 6, 32).to(DEV)
+    with torch.no_grad():
+        _, cache = m(x[:, :5], return_next_cache=True)
+    with pytest.raises(RuntimeError, match="inference-only"):
+        m(x[:, 5:], cache=cache)
+    with torch.no_grad():
+        want, _ = m(x[:, 5:], cache=cache)
+    torch.manual_seed(0)
+    auto = Castle(32, heads=2, dim_head=16, use_triton=None).to(DEV)
+    auto.load_state_dict(m.state_dict())
+    with torch.no_grad():
+        _, cache = auto(x[:, :5], return_next_cache=True)
+    Castle._warned_dense_step = False
+    with pytest.warns(RuntimeWarning, match="dense PyTorch step"):
+        got, nxt = auto(x[:, 5:], cache=cache)
+    assert got.requires_grad and nxt.U.shape[-2] == 6
+    got.sum().backward()
+    assert auto.to_all_qkv.weight.grad is not None
+    assert (got.detach() - want).abs().max() <= 1e-4
+
+
 def test_multi_token_with_cache_is_rejected():
     m = make(32, 2, 16)
     x = torch.randn(1, 4, 32).to(DEV)

@@ -536,3 +536,47 @@ def test_decode_with_half_precision_lookahead_keys(t0, steps, d, rotary):
         H().castle_decode_step_hip(*f16, L, *[x[:, :, :1].half() for x in dev_ops], s, torch.empty(B, Hh, 1, d, dtype=torch.float16, device=DEV),
                                    ws, u_half=True)
 
+
+
+def test_flush_then_step_needs_the_base_moved_to_the_row_count():
+    """castle_decode_flush folds the pending sources into U and leaves the castle_deferred struct alone:
+    the caller moves `base` to the row count.  Steps that follow a flush with the base moved equal the
+    steps of a cache that was never flushed; with the old base the pending terms would be added twice
+    (shown here on the stored keys, which is why the header calls the update a postcondition)."""
+    from lookahead_keys_attention_amd import _native as N
+
+    B, Hh, d, dtype, t0, t_flush, L = 1, 2, 32, torch.float32, 8, 14, 21
+    ops, _ = rand_ops(B, Hh, L, d, dtype, seed=5)
+    s = d ** -0.5
+    ref = [t.double() for t in ops]
+    ref_out, ref_U = O.parallel_core(*ref, s, want_U=True)
+    _, U0 = O.parallel_core(*[t[:, :, :t0] for t in ref], s, want_U=True)
+    dev_ops = [t.to(DEV) for t in ops]
+    ws = H().decode_workspace(B, Hh, d, DEV)
+
+    def run(flush, move_base):
+        bufs = [torch.zeros(B, Hh, L + 3, d, dtype=dtype, device=DEV) for _ in range(4)]
+        for buf, src in zip(bufs, (U0, ref[3][:, :, :t0], ref[1][:, :, :t0], ref[2][:, :, :t0])):
+            buf[:, :, :t0] = src.to(dtype).to(DEV)
+        rings = [torch.zeros(B, Hh, N.DECODE_DEFER, d, dtype=dtype, device=DEV),
+                 torch.zeros(B, Hh, L + 3, N.DECODE_DEFER, dtype=torch.float32, device=DEV)]
+        base, outs = t0, []
+        for t in range(t0, L):
+            if flush and t == t_flush:
+                assert t % N.DECODE_DEFER != 0   # something is pending here
+                H().castle_decode_flush(bufs[0], bufs[1], t, H().make_deferred(*rings, base), s)
+                if move_base:
+                    base = t
+            o = torch.empty(B, Hh, 1, d, dtype=dtype, device=DEV)
+            H().castle_decode_step_hip(*bufs, t, *[x[:, :, t:t + 1] for x in dev_ops], s, o, ws, deferred=H().make_deferred(*rings, base))
+            outs.append(o)
+        H().castle_decode_flush(bufs[0], bufs[1], L, H().make_deferred(*rings, base), s)
+        return torch.cat(outs, 2), bufs[0][:, :, :L].clone()
+
+    out_plain, U_plain = run(False, False)
+    out_moved, U_moved = run(True, True)
+    assert_close(out_plain, ref_out[:, :, t0:], dtype, "never flushed", 1e-3)
+    assert (out_moved - out_plain).abs().max() <= 1e-5 and (U_moved - U_plain).abs().max() <= 1e-5
+    assert_close(U_moved, ref_U, dtype, "U, base moved after the flush", 1e-3)
+    _, U_stale = run(True, False)
+    assert (U_stale.cpu().double() - ref_U).abs().max() > 1e-2   # the pending terms went in twice
