@@ -606,7 +606,7 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_key2_kernel(BwdArgs a) {
       }                                                                                              \
       fa[jt][0] = chain<T>(aT, 0);                                                                   \
       fa[jt][1] = chain<T>(aT, 1);                                                                   \
-      _Pragma("unroll") for (int r = 0; r < 16; ++r) aT[r] = aT[r] * (1.f - aT[r]);                  \
+      _Pragma("unroll") for (int r = 0; r < 16; ++r) aT[r] = __builtin_fmaf(-aT[r], aT[r], aT[r]);         \
       _Pragma("unroll") for (int q = 0; q < 4; ++q)                                                  \
         st4<T>(w_tile_ + c * LDX + 32 * jt + 8 * q + 4 * g, pack4<T>(aT, q));                        \
     }                                                                                                \
@@ -1426,7 +1426,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
       }
       acc_t dz;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) dz[r] = (dA[r] + dA2[r]) * aK[r] * (1.f - aK[r]);
+      for (int r = 0; r < 16; ++r) dz[r] = (dA[r] + dA2[r]) * __builtin_fmaf(-aK[r], aK[r], aK[r]);   // A (1 - A) in one instruction
       {
         constexpr int SB = LDS_ROWS ? 1 : 2;
 #pragma unroll
