@@ -21,7 +21,7 @@ import torch.nn.functional as F
 from torch import nn
 
 from . import _native
-from .castle import Castle
+from .castle import Castle, _linear
 
 
 # -- sampling helpers (train_triton.py:56-71) ------------------------------------------------
@@ -53,6 +53,13 @@ def token_feed_forward(feed_forward: nn.Sequential, h: torch.Tensor) -> torch.Te
     norm, up, act, down = feed_forward
     hidden = Castle._project(up, h, True, norm=norm, activation="gelu")
     return Castle._project(down, hidden, True, residual=h)
+
+
+def block_feed_forward(feed_forward: nn.Sequential, h: torch.Tensor) -> torch.Tensor:
+    """feed_forward(h) for the block [norm, linear, GELU, linear] over many rows: the layers themselves,
+    with the two weight gradients formed in row ranges where that pays (castle._linear)."""
+    norm, up, act, down = feed_forward
+    return _linear(down, act(_linear(up, norm(h))))
 
 
 class GraphedDecoder:
@@ -202,7 +209,7 @@ class CastleLM(nn.Module):
             else:
                 attended = attention(h, cache=layer_cache, return_next_cache=False)
             h = h + attended
-            h = token_feed_forward(feed_forward, h) if token_step else h + feed_forward(h)
+            h = token_feed_forward(feed_forward, h) if token_step else h + block_feed_forward(feed_forward, h)
         logits = Castle._project(self.to_logits, h, token_step, norm=self.final_norm)
         if return_loss:
             return F.cross_entropy(logits.transpose(1, 2), target)

@@ -155,6 +155,34 @@ def test_single_token_step_with_grad_mode_on():
     assert (got.detach() - want).abs().max() <= 1e-4
 
 
+def test_projection_over_many_rows_forms_its_weight_gradient_in_row_ranges():
+    """castle._linear: above SPLIT_WGRAD_MIN_ROWS rows the weight gradient of a bias-free projection is
+    summed from partial products over row ranges; output and both gradients equal nn.Linear's (the
+    partial products are kept in fp32, so the one rounding at the end is the same)."""
+    from lookahead_keys_attention_amd import castle as C
+
+    torch.manual_seed(5)
+    layer = torch.nn.Linear(96, 160, bias=False).to(DEV).bfloat16()
+    x = torch.randn(4, C.SPLIT_WGRAD_MIN_ROWS // 4, 96, device=DEV).bfloat16().requires_grad_()
+    gy = torch.randn(4, C.SPLIT_WGRAD_MIN_ROWS // 4, 160, device=DEV).bfloat16()
+    y = C._linear(layer, x)
+    assert y.grad_fn is not None and "ManyRowLinear" in type(y.grad_fn).__name__
+    y.backward(gy)
+    got = (y.detach(), x.grad.clone(), layer.weight.grad.clone())
+    x.grad, layer.weight.grad = None, None
+    y2 = layer(x)
+    y2.backward(gy)
+    assert torch.equal(got[0], y2.detach()) and torch.equal(got[1], x.grad)
+    ref = gy.float().flatten(0, 1).t() @ x.detach().float().flatten(0, 1)
+    bf16_close(got[2], ref, "weight gradient in row ranges")
+    assert (got[2].float() - ref).norm() <= 1.05 * (layer.weight.grad.float() - ref).norm()
+    # few rows, no grad mode, fp32: the layer itself
+    small = C._linear(layer, x[:, :8])
+    assert "ManyRowLinear" not in type(small.grad_fn).__name__
+    with torch.no_grad():
+        assert C._linear(layer, x).grad_fn is None
+
+
 def test_multi_token_with_cache_is_rejected():
     m = make(32, 2, 16)
     x = torch.randn(1, 4, 32).to(DEV)
