@@ -84,8 +84,8 @@ struct BwdArgs {
 // rounds every U row once per write-back; bf16 keeps 8 significant bits, fp16 keeps 11, so the
 // rounding noise a long decode accumulates is 8 times smaller.  The power-of-two factor moves the
 // fp16 window to |U| in [2^-18, 4.2e6]: below it the absolute error (4e-6) is far under what a bf16
-// value of any score-relevant size carries; above it the silu term of that key's score has long
-// saturated (the key is masked out either way).
+// value of any score-relevant size carries; above it the keys saturate instead of becoming infinite
+// (lookahead scores of that size are beyond what any 16-bit cache resolves).
 constexpr float kUHalfScale = 0.015625f;   // 2^-6
 constexpr float kUHalfUnscale = 64.f;
 

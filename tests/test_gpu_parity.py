@@ -580,3 +580,39 @@ def test_flush_then_step_needs_the_base_moved_to_the_row_count():
     assert_close(U_moved, ref_U, dtype, "U, base moved after the flush", 1e-3)
     _, U_stale = run(True, False)
     assert (U_stale.cpu().double() - ref_U).abs().max() > 1e-2   # the pending terms went in twice
+
+
+def test_half_precision_lookahead_keys_saturate_instead_of_overflowing():
+    """Lookahead keys beyond the window of the half-precision cache format (|U| > 4.2e6) are stored
+    saturated, never as infinities: the steps stay finite (each output row a convex combination of
+    value rows) and the keys inside the window are still the oracle's.  (Lookahead scores built from
+    keys of that size are millions wide; no 16-bit cache resolves them, so the outputs themselves are
+    not compared here.)"""
+    from lookahead_keys_attention_amd import _native as N
+
+    B, Hh, d, L, dtype = 1, 2, 32, 260, torch.bfloat16
+    ops, _ = rand_ops(B, Hh, L, d, dtype, seed=77)
+    ops[5] = (ops[5].float().abs() * 6.0e4 + 2.0e4).clamp(0, 6.5e4).to(dtype)     # vu: a few hundred of these add up past 4.2e6
+    s = d ** -0.5
+    ref_out, ref_U = O.parallel_core(*[t.double() for t in ops], s, want_U=True)
+    assert ref_U.abs().max() > 4.5e6
+    dev_ops = [t.to(DEV) for t in ops]
+    bufs = [torch.zeros(B, Hh, L + 1, d, dtype=dtype, device=DEV) for _ in range(4)]
+    rings = [torch.zeros(B, Hh, N.DECODE_DEFER, d, dtype=dtype, device=DEV),
+             torch.zeros(B, Hh, L + 1, N.DECODE_DEFER, dtype=torch.float32, device=DEV)]
+    ws = H().decode_workspace(B, Hh, d, DEV)
+    outs = []
+    for t in range(L):
+        o = torch.empty(B, Hh, 1, d, dtype=dtype, device=DEV)
+        H().castle_decode_step_hip(*bufs, t, *[x[:, :, t:t + 1] for x in dev_ops], s, o, ws,
+                                   deferred=H().make_deferred(*rings, 0), u_half=True)
+        outs.append(o)
+    got = torch.cat(outs, 2)
+    assert torch.isfinite(got).all()
+    assert got.float().abs().max() <= dev_ops[2].float().abs().max() * 1.01
+    H().castle_decode_flush(bufs[0], bufs[1], L, H().make_deferred(*rings, 0), s, u_half=True)
+    stored = bufs[0][:, :, :L].view(torch.float16).float().cpu() * 64.0
+    assert torch.isfinite(stored).all() and stored.abs().max() <= 65504.0 * 64.0
+    small = ref_U.abs() < 4.0e6     # inside the window the keys are the oracle's
+    assert ((stored.double() - ref_U)[small].abs() <= 2e-3 * ref_U.abs().max()).all()
+
