@@ -12,6 +12,12 @@
 //   bwd_query_kernel  query-stationary, 128 rows per workgroup (32 per wave, rows on lanes),
 //                     keys streamed in chunks of 32: dQc (rows as queries) and dKu, dVu
 //                     (rows as lookahead sources), using the forward snapshots usnap and gsnap.
+// Those two are the single-role kernels (fp32 tensors; 16-bit at d = 128 without room for score
+// tiles).  16-bit tensors otherwise run workgroups of 512 threads in two wave roles that share a
+// SIMD pairwise, and hand dS / dSu from the key side to the query side as 32 x 32 tiles in HBM:
+//   bwd_key2_kernel   (d <= 64) score waves + gradient waves, one launch
+//   bwd_keyw1_kernel, bwd_keyw2_kernel  (d = 128) the same split over two launches
+//   bwd_query2_kernel source-row waves + query-row waves; one launch up to d = 64, two at d = 128
 //
 // Units (s = softmax scale, c1 = s log2 e).  As in the forward pass the resident query operand is
 // Qc' = c1 Qc, the stored T blocks are T' = c1 tril(Qc Vu^T) and the resident gate operand is
@@ -126,12 +132,11 @@ template <typename T, int HD> constexpr int bwd_key_lds_bytes() {
 
 // PART selects the outputs of a launch: 0 = all (d <= 64); 1 = dVc, dKc; 2 = dQu and the reverse
 // state (gsnap).  At d = 128 the four accumulator sets do not fit the register file together, so
-// the kernel runs once with PART 1 and once with PART 2.  The PART 1 launch hands dS / dSu to the
-// query-stationary kernel as tiles when there is room for them; a PART 2 launch with TILES_IN
-// (after it) reads dSu from those tiles instead of evaluating the score chain a second time.
-template <typename T, typename TI, int HD, int PART, bool TILES_IN = false>
+// the kernel runs once with PART 1 and once with PART 2.  This is the kernel of fp32 tensors, and
+// of 16-bit tensors at d = 128 when there is no room for the dS / dSu tiles (otherwise the two-role
+// kernels below run).
+template <typename T, typename TI, int HD, int PART>
 __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
-  static_assert(!TILES_IN || (PART == 2 && sizeof(T) == 2), "only the dQu / reverse-state pass reads tiles");
   constexpr bool DO_KV = PART != 2, DO_QG = PART != 1;
   constexpr int KS = HD / 16;
   constexpr int HDP = HD < 32 ? 32 : HD;
@@ -149,7 +154,7 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   float* s_delta = cv.take<float>(kNB);
   // At d = 128 the score chain takes the kc / vc rows of the workgroup's keys from LDS instead of
   // holding them in registers: that is what leaves room for the register prefetch of the next block.
-  constexpr bool KV_LDS = HD > 64 && !TILES_IN;
+  constexpr bool KV_LDS = HD > 64;
   T* s_kcw = KV_LDS ? cv.take<T>(128 * LDK) : nullptr;
   T* s_vcw = KV_LDS ? cv.take<T>(128 * LDK) : nullptr;
 
@@ -176,29 +181,23 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   const float* lse = a.ws.lse + (int64_t)bh * a.s.Lp;
   const float* delta = a.delta + (int64_t)bh * a.s.Lp;
 
-  constexpr int NSC = TILES_IN ? 1 : KS;   // the score-chain operands are not needed when dSu is read
-  constexpr int NKV = (TILES_IN || KV_LDS) ? 1 : KS;
-  frag<T> fkc[NKV], fvc[NKV], fqu[KS], fub[NSC];
+  constexpr int NKV = KV_LDS ? 1 : KS;
+  frag<T> fkc[NKV], fvc[NKV], fqu[KS], fub[KS];
 #pragma unroll
   for (int s = 0; s < KS; ++s) fqu[s] = ldg_nat_scaled<T, T>(qu, HD, k, 16 * s + 8 * g, true, -c1);
-  if constexpr (!TILES_IN) {
 #pragma unroll
-    for (int s = 0; s < KS; ++s) fub[s] = zero_frag<T>();
-    if constexpr (KV_LDS) {   // visible after the first barrier of the block loop
-      RowStage<T, T, 128, HD> st;
-      st.load_flat(kc + (int64_t)kb * 128 * HD); st.store(s_kcw, LDK);
-      st.load_flat(vc + (int64_t)kb * 128 * HD); st.store(s_vcw, LDK);
-    } else {
+  for (int s = 0; s < KS; ++s) fub[s] = zero_frag<T>();
+  if constexpr (KV_LDS) {   // visible after the first barrier of the block loop
+    RowStage<T, T, 128, HD> st;
+    st.load_flat(kc + (int64_t)kb * 128 * HD); st.store(s_kcw, LDK);
+    st.load_flat(vc + (int64_t)kb * 128 * HD); st.store(s_vcw, LDK);
+  } else {
 #pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        fkc[s] = ldg_nat<T>(kc, HD, k, 16 * s + 8 * g, true);
-        fvc[s] = ldg_nat<T>(vc, HD, k, 16 * s + 8 * g, true);
-      }
+    for (int s = 0; s < KS; ++s) {
+      fkc[s] = ldg_nat<T>(kc, HD, k, 16 * s + 8 * g, true);
+      fvc[s] = ldg_nat<T>(vc, HD, k, 16 * s + 8 * g, true);
     }
   }
-  const T* dsu_tiles = TILES_IN ? reinterpret_cast<const T*>(a.dsu_mat) + (int64_t)bh * a.s.Lp * a.s.Lp +
-                                      (int64_t)(kw0 / 32) * (a.s.Lp / 32) * 1024 + c * 16 + 8 * g
-                                : nullptr;
   acc_t dvc[NT], dkc[NT], dqu[NT], G[NT];   // [n rows, k lanes]
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) { zero(dvc[nt]); zero(dkc[nt]); zero(dqu[nt]); zero(G[nt]); }
@@ -210,7 +209,7 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
   do {                                                       \
     const int64_t r_ = (int64_t)(I_) * kNB;                  \
     pqc.load_flat(qc + r_ * HD);                            \
-    if (!TILES_IN) pdo.load_flat(dout + r_ * HD);           \
+    pdo.load_flat(dout + r_ * HD);                          \
     pku.load_flat(ku + r_ * HD);                            \
     pvu.load_flat(vu + r_ * HD);                            \
     ptb.load(tb, kNB, r_, (int64_t)1 << 40);                 \
@@ -226,35 +225,20 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
     if (DO_QG && active && I <= a.s.nblk - 2 && (a.ds_mat == nullptr || (I & 1))) {
       store_snap_tile<T, HD, NT>(gsnap + (gsnap_off(I) + kw0) * HD, G, c, g);
     }
-    if constexpr (!TILES_IN) {
-      if (I > Iw) {
+    if (I > Iw) {
 #pragma unroll
-        for (int s = 0; s < KS; ++s) fub[s] = ldg_snap_nat<T>(usnap + (usnap_off(I) + kw0) * HD, c, 16 * s + 8 * g);
-      }
-    }
-    // dSu fragments of the block's sub-tiles straight from the tiles (natural order: lane = key,
-    // 8 consecutive queries), requested here and used behind the gate
-    frag<T> tdsu[TILES_IN ? BT : 1][2];
-    if constexpr (TILES_IN) {
-#pragma unroll
-      for (int it = 0; it < BT; ++it) {
-        const int i0 = I * kNB + 32 * it;
-#pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2)
-          tdsu[it][s2] = (active && i0 + 31 >= kw0) ? __builtin_nontemporal_load(reinterpret_cast<const frag_mem<T>*>(dsu_tiles + (int64_t)(i0 / 32) * 1024 + s2 * 512))
-                                                   : zero_frag<T>();
-      }
+      for (int s = 0; s < KS; ++s) fub[s] = ldg_snap_nat<T>(usnap + (usnap_off(I) + kw0) * HD, c, 16 * s + 8 * g);
     }
     __syncthreads();
     const int64_t r0 = (int64_t)I * kNB;
     if (!PF) CASTLE_BK_LOAD(I);
     pqc.store(s_qc, LDK);
-    if (!TILES_IN) pdo.store(s_do, LDK);
+    pdo.store(s_do, LDK);
     pku.store(s_ku, LDK);
     pvu.store_halves(s_vu, LDU);
     ptb.store_halves(s_t, LDT);
     if (PF && I > I0) CASTLE_BK_LOAD(I - 1);   // in flight while this block is processed
-    if (!TILES_IN && threadIdx.x < kNB) {
+    if (threadIdx.x < kNB) {
       const int64_t i = r0 + threadIdx.x;
       s_lse[threadIdx.x] = i < L ? lse[i] * kLog2e : INFINITY;
       s_delta[threadIdx.x] = i < L ? delta[i] : 0.f;
@@ -306,28 +290,6 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
     for (int it = 0; it < BT; ++it) {
       const int i0 = I * kNB + 32 * it;
       if (i0 + 31 < kw0) continue;   // every query precedes every key of this wave
-      if constexpr (TILES_IN) {
-        frag<T> oqt[2][NT], ott[2][BT];
-#pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2) {
-          const int ic = 32 * it + 16 * s2;
-#pragma unroll
-          for (int nt = 0; nt < NT; ++nt) oqt[s2][nt] = ld_free<T, false>(s_qc, LDK, 32 * nt, HD, ic, c, g);
-#pragma unroll
-          for (int jt = 0; jt < BT; ++jt)
-            if (jt <= it) ott[s2][jt] = ld_free<T, false>(s_t, LDT, 32 * jt, kNB, ic, c, g);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2) {
-#pragma unroll
-          for (int nt = 0; nt < NT; ++nt) mma(G[nt], oqt[s2][nt], tdsu[it][s2]);
-#pragma unroll
-          for (int jt = 0; jt < BT; ++jt)
-            if (jt <= it) mma(dA[jt], ott[s2][jt], tdsu[it][s2]);
-        }
-        continue;
-      }
       acc_t sc, su, dp;
       zero(sc); zero(su); zero(dp);
       {
@@ -380,18 +342,6 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_key_kernel(BwdArgs a) {
         sc[r] = p;
         ds[r] = dsv;
         dsu[r] = -dsv * sp * su_mul;                      // gradient of the product built from vu * vu_scale
-      }
-      if constexpr (DO_KV && sizeof(T) == 2) {
-        if (a.ds_mat != nullptr) {   // hand the tile to the tile-consuming query kernel: element (k, i) at (i/16)*512 + k*16 + i%16
-          T* ds_mat = reinterpret_cast<T*>(a.ds_mat) + (int64_t)bh * a.s.Lp * a.s.Lp;
-          T* dsu_mat = reinterpret_cast<T*>(a.dsu_mat) + (int64_t)bh * a.s.Lp * a.s.Lp;
-          const int64_t tile = ((int64_t)(kw0 / 32) * (a.s.Lp / 32) + i0 / 32) * 1024 + c * 16 + 4 * g;
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {   // registers 4q .. 4q+3: queries 8q + 4g .. + 3 of the tile
-            st4_stream<T>(ds_mat + tile + (q / 2) * 512 + 8 * (q % 2), pack4<T>(ds, q));
-            st4_stream<T>(dsu_mat + tile + (q / 2) * 512 + 8 * (q % 2), pack4<T>(dsu, q));
-          }
-        }
       }
       {
         frag<T> odt[2][NT], oqt[2][NT], ott[2][BT];
@@ -825,6 +775,517 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_key2_kernel(BwdArgs a) {
 }
 
 // ---------------------------------------------------------------------------
+// Key-stationary backward for head dimensions above 64 (16-bit compute types) with two wave roles,
+// in two launches: no wave can hold the four accumulator sets of its keys at d = 128, and a wave
+// of either role must stay within half a SIMD's registers so that two of them share it.
+//   launch 1 (bwd_keyw1_kernel):  score waves   Kc, Vc, -c1 Qu and the lookahead state of their 32 keys
+//                                               in registers; per 32-query sub-tile the scores, P, dS,
+//                                               dSu -> LDS for the partner and the dS / dSu tiles -> HBM
+//                                 gradient waves  all staging of the block tiles; dVc, dKc
+//   launch 2 (bwd_keyw2_kernel):  gate waves    staging; gate A of a block, then dZ = dA A (1 - A) and
+//                                               dQu one block later
+//                                 state waves   dSu fragments straight from the tiles; reverse state G
+//                                               (snapshots), dA = G Vu^T + dSu^T T' -> LDS for the partner
+// Pair (w, w + 4) owns keys kb*128 + 32 w .. + 31, as in bwd_key2_kernel.
+template <typename T, int HD> constexpr int bwd_keyw1_lds_bytes() {
+  int b = 3 * a16((int)sizeof(T) * kNB * lds_ld<T>(HD));    // qc, do, ku
+  b += a16((int)sizeof(T) * kNB * lds_ld_chain<T>(kNB));    // T'
+  b += 2 * a16(4 * kNB);                                    // lse, delta
+  b += 4 * 3 * a16((int)sizeof(T) * 32 * lds_ld<T>(kNB));   // P, dS, dSu per wave pair
+  return b;
+}
+template <typename T, int HD> constexpr int bwd_keyw2_lds_bytes() {
+  int b = 3 * a16((int)sizeof(T) * kNB * lds_ld<T>(HD));    // qc, ku (two blocks)
+  b += a16((int)sizeof(T) * kNB * lds_ld_chain<T>(HD));     // vu
+  b += a16((int)sizeof(T) * kNB * lds_ld_chain<T>(kNB));    // T'
+  b += 2 * 4 * a16((int)sizeof(T) * 32 * lds_ld<T>(kNB));   // dA per wave pair, two blocks
+  return b;
+}
+
+template <typename T, typename TI, int HD>
+__global__ __launch_bounds__(2 * kThreads, 1) void bwd_keyw1_kernel(BwdArgs a) {
+  static_assert(sizeof(T) == 2 && HD > 64, "two-role kernel for wide heads: 16-bit operands");
+  constexpr int KS = HD / 16;
+  constexpr int NT = HD / 32;
+  constexpr int BT = kNB / 32;
+  constexpr int LDK = lds_ld<T>(HD), LDT = lds_ld_chain<T>(kNB), LDX = lds_ld<T>(kNB);
+
+  Carver cv{castle_smem};
+  T* s_qc = cv.take<T>(kNB * LDK);
+  T* s_do = cv.take<T>(kNB * LDK);
+  T* s_ku = cv.take<T>(kNB * LDK);   // one buffer: only the gate reads it, between barriers 3 and 4
+  T* s_t = cv.take<T>(kNB * LDT);
+  float* s_lse = cv.take<float>(kNB);
+  float* s_delta = cv.take<float>(kNB);
+  T* s_x = cv.take<T>(4 * 3 * 32 * LDX);
+
+  int kb, bh;
+  work_item(a.s.B * a.s.H, kb, bh);
+  const int b = bh / a.s.H, h = bh % a.s.H;
+  const int lane = lane_id(), wave = wave_id(), c = lane & 31, g = lane >> 5;
+  const bool scorer = wave < 4;
+  const int pw = wave & 3;
+  const int L = a.s.L;
+  const float c1 = a.s.scale * kLog2e;
+  const float su_mul = a.ws.hdr->su_mul, gun = a.bhdr->grad_unscale;
+  const int kw0 = kb * 128 + 32 * pw;
+  const int k = kw0 + c;
+  const int Iw = kw0 / kNB;
+  const int I0 = (kb * 128) / kNB;
+  const int Ilast = a.s.nblk - 1;
+  T* x_p = s_x + pw * 3 * 32 * LDX;   // [key][query of the block]
+  T* x_ds = x_p + 32 * LDX;
+  T* x_dsu = x_ds + 32 * LDX;
+
+  if (scorer) {
+    const T* kc = prep_ptr<T>(a.ws.kc_p, bh, a.s.Lp, HD);
+    const T* vc = prep_ptr<T>(a.ws.vc_p, bh, a.s.Lp, HD);
+    const T* qu = prep_ptr<T>(a.ws.qu_p, bh, a.s.Lp, HD);
+    const T* usnap = reinterpret_cast<const T*>(a.ws.usnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
+    T* ds_mat = reinterpret_cast<T*>(a.ds_mat) + (int64_t)bh * a.s.Lp * a.s.Lp;
+    T* dsu_mat = reinterpret_cast<T*>(a.dsu_mat) + (int64_t)bh * a.s.Lp * a.s.Lp;
+
+    frag<T> fkc[KS], fvc[KS], fqu[KS], fub[KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      fkc[s] = ldg_nat<T>(kc, HD, k, 16 * s + 8 * g, true);
+      fvc[s] = ldg_nat<T>(vc, HD, k, 16 * s + 8 * g, true);
+      fqu[s] = ldg_nat_scaled<T, T>(qu, HD, k, 16 * s + 8 * g, true, -c1);
+      fub[s] = zero_frag<T>();
+    }
+    frag<T> fa[BT][2];
+    // gate tiles A^T[j rows, k lanes] of source block J as operand fragments of its score tiles
+#define CASTLE_BKW_GATE(J_)                                                                          \
+  do {                                                                                               \
+    _Pragma("unroll") for (int jt = 0; jt < BT; ++jt) {                                              \
+      acc_t aT;                                                                                      \
+      zero(aT);                                                                                      \
+      _Pragma("unroll") for (int s0 = 0; s0 < KS; s0 += 4) {                                         \
+        frag<T> oku[4];                                                                              \
+        _Pragma("unroll") for (int u = 0; u < 4; ++u)                                                \
+          oku[u] = ld_nat<T>(s_ku, LDK, 32 * jt + c, 16 * (s0 + u) + 8 * g);                         \
+        __builtin_amdgcn_sched_barrier(0);                                                           \
+        _Pragma("unroll") for (int u = 0; u < 4; ++u) mma(aT, oku[u], fqu[s0 + u]);                  \
+      }                                                                                              \
+      const int j0 = (J_) * kNB + 32 * jt;                                                           \
+      _Pragma("unroll") for (int r = 0; r < 16; ++r) aT[r] = fast_rcp(1.f + fast_exp2(aT[r]));       \
+      if (j0 <= kw0 + 31) { /* tile touches the diagonal: keep j > k only */                         \
+        _Pragma("unroll") for (int r = 0; r < 16; ++r)                                               \
+          if (j0 + acc_row(r, g) <= k) aT[r] = 0.f;                                                  \
+      }                                                                                              \
+      fa[jt][0] = chain<T>(aT, 0);                                                                   \
+      fa[jt][1] = chain<T>(aT, 1);                                                                   \
+    }                                                                                                \
+  } while (0)
+
+    if (Ilast > Iw) {
+#pragma unroll
+      for (int s = 0; s < KS; ++s) fub[s] = ldg_snap_nat<T>(usnap + (usnap_off(Ilast) + kw0) * HD, c, 16 * s + 8 * g);
+    }
+    __syncthreads();   // 0: first Ku tile staged
+    if (Ilast >= Iw) CASTLE_BKW_GATE(Ilast);
+    for (int I = Ilast; I >= I0; --I) {
+      const bool active = I >= Iw;
+      const bool inter = I > Iw;   // lookahead state from earlier blocks exists
+      __syncthreads();   // 1: tiles staged
+#pragma unroll
+      for (int it = 0; it < BT; ++it) {
+        const int i0 = I * kNB + 32 * it;
+        if (active && i0 + 31 >= kw0) {   // else every query precedes every key of this wave
+          acc_t sc, su, dp;   // sc starts from -lse, dp from -delta of its row
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const vec<float, 4> nl = *reinterpret_cast<const vec<float, 4>*>(s_lse + 32 * it + 8 * q + 4 * g);
+            const vec<float, 4> nd = *reinterpret_cast<const vec<float, 4>*>(s_delta + 32 * it + 8 * q + 4 * g);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              sc[4 * q + e] = nl[e];
+              dp[4 * q + e] = nd[e];
+              su[4 * q + e] = 0.f;
+            }
+          }
+#pragma unroll
+          for (int s0 = 0; s0 < KS; s0 += 4) {   // operand fragments in batches of four
+            frag<T> oq[4], od[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              oq[u] = ld_nat<T>(s_qc, LDK, 32 * it + c, 16 * (s0 + u) + 8 * g);
+              od[u] = ld_nat<T>(s_do, LDK, 32 * it + c, 16 * (s0 + u) + 8 * g);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              mma(sc, oq[u], fkc[s0 + u]);
+              mma(dp, od[u], fvc[s0 + u]);
+              if (inter) mma(su, oq[u], fub[s0 + u]);
+            }
+          }
+          {
+            frag<T> ot[BT][2];
+#pragma unroll
+            for (int jt = 0; jt < BT; ++jt)
+#pragma unroll
+              for (int s2 = 0; s2 < 2; ++s2)
+                if (jt <= it) ot[jt][s2] = ld_chain<T>(s_t, LDT, 32 * it + c, 32 * jt + 16 * s2, g);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int jt = 0; jt < BT; ++jt)
+#pragma unroll
+              for (int s2 = 0; s2 < 2; ++s2)
+                if (jt <= it) mma(su, ot[jt][s2], fa[jt][s2]);
+          }
+          acc_t ds, dsu;
+          if (i0 < kw0 + 31) {   // tile touches the diagonal: queries before the key see nothing
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+              if (i0 + acc_row(r, g) < k) sc[r] = -INFINITY;
+          }
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float sut = su[r] * su_mul;                 // log2(e) * Su
+            const float sg = fast_rcp(1.f + fast_exp2(-sut));
+            const float p = fast_exp2(__builtin_fmaf(-sut, sg, sc[r]));   // sc carries -lse
+            const float dsv = p * dp[r];                      // dp carries -delta
+            const float y = sut * kLn2;                       // true Su
+            const float t = __builtin_fmaf(-y, sg, y);        // y (1 - sigmoid)
+            const float sp = __builtin_fmaf(sg, t, sg);       // silu'(y)
+            sc[r] = p;
+            ds[r] = dsv;
+            dsu[r] = -dsv * sp * su_mul;                      // gradient of the product built from vu * vu_scale
+          }
+          // For the partner through LDS; for the query-stationary kernel and the second launch as 32 x 32
+          // tiles in HBM.  A tile is two runs of 16 queries, 16 bytes per key and lane half in each; the 8
+          // values of a lane are its accumulator registers as they are (chained order: queries 4g..4g+3
+          // and 8+4g..8+4g+3 of the run), so that one store instruction covers 1 KB of whole lines.
+          const int64_t tile = ((int64_t)(kw0 / 32) * (a.s.Lp / 32) + i0 / 32) * 1024 + c * 16 + 8 * g;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int o = c * LDX + 32 * it + 8 * q + 4 * g;
+            st4<T>(x_p + o, pack4<T>(sc, q));
+            st4<T>(x_ds + o, pack4<T>(ds, q));
+            st4<T>(x_dsu + o, pack4<T>(dsu, q));
+          }
+#pragma unroll
+          for (int s2 = 0; s2 < 2; ++s2) {
+            __builtin_nontemporal_store(chain<T>(ds, s2), reinterpret_cast<frag_mem<T>*>(ds_mat + tile + s2 * 512));
+            __builtin_nontemporal_store(chain<T>(dsu, s2), reinterpret_cast<frag_mem<T>*>(dsu_mat + tile + s2 * 512));
+          }
+        }
+        __syncthreads();   // 2, 3: sub-tile handed over
+      }
+      if (I > I0) {
+        if (I - 1 > Iw) {   // lookahead state as of the next block: in flight behind the gate
+#pragma unroll
+          for (int s = 0; s < KS; ++s) fub[s] = ldg_snap_nat<T>(usnap + (usnap_off(I - 1) + kw0) * HD, c, 16 * s + 8 * g);
+        }
+        if (I - 1 >= Iw) CASTLE_BKW_GATE(I - 1);   // its Ku tile was staged before barrier 3
+      }
+      __syncthreads();   // 4: tiles free
+    }
+#undef CASTLE_BKW_GATE
+  } else {
+    const T* qc = prep_ptr<T>(a.ws.qc_p, bh, a.s.Lp, HD);
+    const T* ku = prep_ptr<T>(a.ws.ku_p, bh, a.s.Lp, HD);
+    const T* dout = prep_ptr<T>(a.dout_p, bh, a.s.Lp, HD);
+    const T* tb = reinterpret_cast<const T*>(a.ws.t_blk) + (int64_t)bh * a.s.Lp * kNB;
+    const float* lse = a.ws.lse + (int64_t)bh * a.s.Lp;
+    const float* delta = a.delta + (int64_t)bh * a.s.Lp;
+    const int tid = threadIdx.x - kThreads;   // thread index inside the role
+    acc_t dvc[NT], dkc[NT];   // [n rows, k lanes]
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) { zero(dvc[nt]); zero(dkc[nt]); }
+    // These waves issue no global stores inside the loop, so the pieces of the next block can stay in
+    // flight for a whole block without anything queueing behind them in the in-order memory counter.
+    RowStage<T, T, kNB, HD> pku, pqc, pdo;
+    RowStage<T, T, kNB, kNB> ptb;
+    float plse = 0.f, pdelta = 0.f;
+#define CASTLE_BKW_LOAD(I_)                                  \
+  do {                                                       \
+    const int64_t r_ = (int64_t)(I_) * kNB;                  \
+    pku.load_flat(ku + r_ * HD, tid);                        \
+    pqc.load_flat(qc + r_ * HD, tid);                        \
+    pdo.load_flat(dout + r_ * HD, tid);                      \
+    ptb.load_flat(tb + r_ * kNB, tid);                       \
+    if (tid < kNB) {                                         \
+      const int64_t i_ = r_ + tid;                           \
+      plse = i_ < L ? lse[i_] : INFINITY;                    \
+      pdelta = i_ < L ? delta[i_] : 0.f;                     \
+    }                                                        \
+  } while (0)
+    CASTLE_BKW_LOAD(Ilast);
+    pku.store(s_ku, LDK, tid);
+    __syncthreads();   // 0
+    for (int I = Ilast; I >= I0; --I) {
+      const bool active = I >= Iw;
+      pqc.store(s_qc, LDK, tid);
+      pdo.store(s_do, LDK, tid);
+      ptb.store_halves(s_t, LDT, tid);
+      if (tid < kNB) {
+        s_lse[tid] = -plse * kLog2e;
+        s_delta[tid] = -pdelta;
+      }
+      __syncthreads();   // 1: tiles staged
+      if (I > I0) CASTLE_BKW_LOAD(I - 1);   // in flight for the whole block
+#pragma unroll
+      for (int it = 0; it < BT; ++it) {
+        if (it == 1 && I > I0) pku.store(s_ku, LDK, tid);   // the gate of block I finished before barrier 4 of block I + 1
+        __syncthreads();   // 2, 3: sub-tile `it` is there
+        const int i0 = I * kNB + 32 * it;
+        if (active && i0 + 31 >= kw0) {
+#pragma unroll
+          for (int s2 = 0; s2 < 2; ++s2) {
+            const int ic = 32 * it + 16 * s2;
+            frag<T> odt[NT], oqt[NT];
+            const frag<T> fp = ld_nat<T>(x_p, LDX, c, ic + 8 * g);
+            const frag<T> fds = ld_nat<T>(x_ds, LDX, c, ic + 8 * g);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+              odt[nt] = ld_free<T, false>(s_do, LDK, 32 * nt, HD, ic, c, g);
+              oqt[nt] = ld_free<T, false>(s_qc, LDK, 32 * nt, HD, ic, c, g);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+              mma(dvc[nt], odt[nt], fp);
+              mma(dkc[nt], oqt[nt], fds);
+            }
+          }
+        }
+      }
+      __syncthreads();   // 4
+    }
+#undef CASTLE_BKW_LOAD
+    if (k < L) {
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dkc, b, h) + (int64_t)k * a.dkc.sl, dkc, kLn2 * gun, g, a.s.rotary ? k : -1);
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvc, b, h) + (int64_t)k * a.dvc.sl, dvc, gun, g);
+    }
+  }
+}
+
+template <typename T, typename TI, int HD>
+__global__ __launch_bounds__(2 * kThreads, 1) void bwd_keyw2_kernel(BwdArgs a) {
+  static_assert(sizeof(T) == 2 && HD > 64, "two-role kernel for wide heads: 16-bit operands");
+  constexpr int KS = HD / 16;
+  constexpr int NT = HD / 32;
+  constexpr int BT = kNB / 32;
+  constexpr int LDK = lds_ld<T>(HD), LDU = lds_ld_chain<T>(HD), LDT = lds_ld_chain<T>(kNB), LDX = lds_ld<T>(kNB);
+  // dA crosses the LDS as a 16-bit value: a quarter of it, so that it needs no more range than
+  // dZ = dA A (1 - A) <= dA / 4, which is a 16-bit MFMA operand in every variant of this kernel
+  constexpr float kHand = 0.25f, kUnhand = 4.f;
+
+  Carver cv{castle_smem};
+  T* s_qc = cv.take<T>(kNB * LDK);
+  T* s_ku0 = cv.take<T>(kNB * LDK);
+  T* s_ku1 = cv.take<T>(kNB * LDK);
+  T* s_vu = cv.take<T>(kNB * LDU);
+  T* s_t = cv.take<T>(kNB * LDT);
+  T* s_da = cv.take<T>(2 * 4 * 32 * LDX);
+
+  int kb, bh;
+  work_item(a.s.B * a.s.H, kb, bh);
+  const int b = bh / a.s.H, h = bh % a.s.H;
+  const int lane = lane_id(), wave = wave_id(), c = lane & 31, g = lane >> 5;
+  const bool gater = wave < 4;
+  const int pw = wave & 3;
+  const int L = a.s.L;
+  const float c0 = a.s.scale, c1 = a.s.scale * kLog2e;
+  const float gun = a.bhdr->grad_unscale;
+  const int kw0 = kb * 128 + 32 * pw;
+  const int k = kw0 + c;
+  const int Iw = kw0 / kNB;
+  const int I0 = (kb * 128) / kNB;
+  const int Ilast = a.s.nblk - 1;
+  T* x_da = s_da + pw * 32 * LDX;   // [key][source of the block], + 4*32*LDX for odd blocks
+#define CASTLE_BKW_KU(I_) (((I_) & 1) ? s_ku1 : s_ku0)
+#define CASTLE_BKW_DA(I_) (x_da + ((I_) & 1) * 4 * 32 * LDX)
+
+  if (gater) {
+    const T* qc = prep_ptr<T>(a.ws.qc_p, bh, a.s.Lp, HD);
+    const T* qu = prep_ptr<T>(a.ws.qu_p, bh, a.s.Lp, HD);
+    const T* ku = prep_ptr<T>(a.ws.ku_p, bh, a.s.Lp, HD);
+    const T* vu = prep_ptr<T>(a.ws.vu_p, bh, a.s.Lp, HD);
+    const T* tb = reinterpret_cast<const T*>(a.ws.t_blk) + (int64_t)bh * a.s.Lp * kNB;
+    frag<T> fqu[KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) fqu[s] = ldg_nat_scaled<T, T>(qu, HD, k, 16 * s + 8 * g, true, -c1);
+    acc_t dqu[NT];   // [n rows, k lanes]
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) zero(dqu[nt]);
+    vec<T, 4> w[BT][4];   // 4 A (1 - A) of the block whose dA is still to come, [j rows, k lanes], packed
+#pragma unroll
+    for (int jt = 0; jt < BT; ++jt)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) w[jt][q] = vec<T, 4>{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+    RowStage<T, T, kNB, HD> pku, pqc, pvu;
+    RowStage<T, T, kNB, kNB> ptb;
+#define CASTLE_BKW_LOAD(I_)                                  \
+  do {                                                       \
+    const int64_t r_ = (int64_t)(I_) * kNB;                  \
+    pku.load_flat(ku + r_ * HD);                             \
+    pqc.load_flat(qc + r_ * HD);                             \
+    pvu.load_flat(vu + r_ * HD);                             \
+    ptb.load_flat(tb + r_ * kNB);                            \
+  } while (0)
+    // dZ^T = dA^T * A (1 - A)  ->  dQu, for source block J: its Ku tile is still in its buffer
+#define CASTLE_BKW_DQU(J_)                                                                           \
+  do {                                                                                               \
+    const T* ku_tile_ = CASTLE_BKW_KU(J_);                                                           \
+    const T* da_tile_ = CASTLE_BKW_DA(J_);                                                           \
+    _Pragma("unroll") for (int jt = 0; jt < BT; ++jt) {                                              \
+      acc_t dz;                                                                                      \
+      _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                                \
+        const vec<T, 4> d4 = *reinterpret_cast<const vec4_mem<T>*>(da_tile_ + c * LDX + 32 * jt + 8 * q + 4 * g); \
+        _Pragma("unroll") for (int e = 0; e < 4; ++e) dz[4 * q + e] = (float)d4[e] * (float)w[jt][q][e]; \
+      }                                                                                              \
+      _Pragma("unroll") for (int s2 = 0; s2 < 2; ++s2) {                                             \
+        frag<T> okt[NT];                                                                             \
+        _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                            \
+          okt[nt] = ld_free<T, true>(ku_tile_, LDK, 32 * nt, HD, 32 * jt + 16 * s2, c, g);           \
+        __builtin_amdgcn_sched_barrier(0);                                                           \
+        const frag<T> fdz = chain<T>(dz, s2);                                                        \
+        _Pragma("unroll") for (int nt = 0; nt < NT; ++nt) mma(dqu[nt], okt[nt], fdz);                \
+      }                                                                                              \
+    }                                                                                                \
+  } while (0)
+
+    CASTLE_BKW_LOAD(Ilast);
+    for (int I = Ilast; I >= I0; --I) {
+      // every wave has passed the end barrier of block I + 1: its tiles are free, and so is the Ku
+      // buffer of block I + 2, which block I takes over
+      pqc.store(s_qc, LDK);
+      pvu.store_halves(s_vu, LDU);
+      ptb.store_halves(s_t, LDT);
+      pku.store(CASTLE_BKW_KU(I), LDK);
+      __syncthreads();   // 1: tiles staged
+      if (I > I0) CASTLE_BKW_LOAD(I - 1);   // in flight for the whole block
+      if (I < Ilast && I + 1 >= Iw) CASTLE_BKW_DQU(I + 1);   // finish the previous block
+      if (I >= Iw) {   // gate of this block: 4 A (1 - A) stays in registers until its dA arrives
+        const T* ku_tile = CASTLE_BKW_KU(I);
+#pragma unroll
+        for (int jt = 0; jt < BT; ++jt) {
+          acc_t aT;
+          zero(aT);
+#pragma unroll
+          for (int s0 = 0; s0 < KS; s0 += 2) {   // operand fragments in pairs: this role is at the register limit
+            frag<T> oku[2];
+#pragma unroll
+            for (int u = 0; u < 2; ++u) oku[u] = ld_nat<T>(ku_tile, LDK, 32 * jt + c, 16 * (s0 + u) + 8 * g);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < 2; ++u) mma(aT, oku[u], fqu[s0 + u]);
+          }
+          const int j0 = I * kNB + 32 * jt;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float av = fast_rcp(1.f + fast_exp2(aT[r]));
+            aT[r] = kUnhand * __builtin_fmaf(-av, av, av);
+          }
+          if (j0 <= kw0 + 31) {   // tile touches the diagonal: keep j > k only
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+              if (j0 + acc_row(r, g) <= k) aT[r] = 0.f;
+          }
+#pragma unroll
+          for (int q = 0; q < 4; ++q) w[jt][q] = pack4<T>(aT, q);
+        }
+      }
+      __syncthreads();   // 2: block done, dA of block I written
+    }
+    if (I0 >= Iw) CASTLE_BKW_DQU(I0);
+#undef CASTLE_BKW_LOAD
+#undef CASTLE_BKW_DQU
+    if (k < L) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqu, b, h) + (int64_t)k * a.dqu.sl, dqu, c0 * kLn2 * gun, g, a.s.rotary ? k : -1);
+  } else {
+    T* gsnap = reinterpret_cast<T*>(a.gsnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
+    const T* dsu_tiles = reinterpret_cast<const T*>(a.dsu_mat) + (int64_t)bh * a.s.Lp * a.s.Lp +
+                         (int64_t)(kw0 / 32) * (a.s.Lp / 32) * 1024 + c * 16 + 8 * g;
+    acc_t G[NT];   // [n rows, k lanes]
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) zero(G[nt]);
+    // dSu fragments of a block's sub-tiles straight from the tiles (lane = key, 8 queries in the
+    // chained order the first launch stored them in); those of the next block are requested a block ahead
+    frag<T> tdsu[BT][2], tnext[BT][2];
+#define CASTLE_BKW_TILES(DST, I_)                                                                     \
+  do {                                                                                                \
+    _Pragma("unroll") for (int it = 0; it < BT; ++it) {                                               \
+      const int i0_ = (I_) * kNB + 32 * it;                                                           \
+      _Pragma("unroll") for (int s2 = 0; s2 < 2; ++s2)                                                \
+        DST[it][s2] = ((I_) >= Iw && i0_ + 31 >= kw0)                                                 \
+                          ? __builtin_nontemporal_load(reinterpret_cast<const frag_mem<T>*>(dsu_tiles + (int64_t)(i0_ / 32) * 1024 + s2 * 512)) \
+                          : zero_frag<T>();                                                           \
+    }                                                                                                 \
+  } while (0)
+    CASTLE_BKW_TILES(tnext, Ilast);
+    for (int I = Ilast; I >= I0; --I) {
+      const bool active = I >= Iw;
+      // the fragments requested a block ago are waited for here, ahead of the stores below: behind
+      // them the wait would cover the stores too
+#pragma unroll
+      for (int it = 0; it < BT; ++it)
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+          tdsu[it][s2] = tnext[it][s2];
+          asm volatile("" : "+v"(tdsu[it][s2]));
+        }
+      // reverse state as of block I; the query-stationary kernel reads those behind a pair of blocks
+      if (active && I <= a.s.nblk - 2 && (I & 1)) store_snap_tile<T, HD, NT>(gsnap + (gsnap_off(I) + kw0) * HD, G, c, g);
+      __syncthreads();   // 1: tiles staged
+      if (I > I0) CASTLE_BKW_TILES(tnext, I - 1);
+      if (active) {
+        // dA^T[j rows, k lanes] of this block, second term first: G (before this block) times Vu^T
+        acc_t dA[BT];
+#pragma unroll
+        for (int jt = 0; jt < BT; ++jt) {
+          zero(dA[jt]);
+#pragma unroll
+          for (int s0 = 0; s0 < KS; s0 += 4) {
+            frag<T> ovu[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) ovu[u] = ld_chain<T>(s_vu, LDU, 32 * jt + c, 16 * (s0 + u), g);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) mma(dA[jt], ovu[u], chain<T>(G[(s0 + u) / 2], (s0 + u) % 2));
+          }
+        }
+#pragma unroll
+        for (int it = 0; it < BT; ++it) {
+          const int i0 = I * kNB + 32 * it;
+          if (i0 + 31 < kw0) continue;   // every query precedes every key of this wave
+#pragma unroll
+          for (int s2 = 0; s2 < 2; ++s2) {
+            const int ic = 32 * it + 16 * s2;
+            frag<T> oqt[NT], ott[BT];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) oqt[nt] = ld_free<T, true>(s_qc, LDK, 32 * nt, HD, ic, c, g);
+#pragma unroll
+            for (int jt = 0; jt < BT; ++jt)
+              if (jt <= it) ott[jt] = ld_free<T, true>(s_t, LDT, 32 * jt, kNB, ic, c, g);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) mma(G[nt], oqt[nt], tdsu[it][s2]);
+#pragma unroll
+            for (int jt = 0; jt < BT; ++jt)
+              if (jt <= it) mma(dA[jt], ott[jt], tdsu[it][s2]);
+          }
+        }
+        T* da_tile = CASTLE_BKW_DA(I);
+#pragma unroll
+        for (int jt = 0; jt < BT; ++jt) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) dA[jt][r] *= kHand;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) st4<T>(da_tile + c * LDX + 32 * jt + 8 * q + 4 * g, pack4<T>(dA[jt], q));
+        }
+      }
+      __syncthreads();   // 2: block done
+    }
+#undef CASTLE_BKW_TILES
+  }
+#undef CASTLE_BKW_KU
+#undef CASTLE_BKW_DA
+}
+
+// ---------------------------------------------------------------------------
 constexpr int kCK = 32;   // keys per chunk in the query-stationary backward
 
 template <typename T, int HD> constexpr int bwd_query_lds_bytes() {
@@ -1187,7 +1648,9 @@ template <typename T, int HD> constexpr int bwd_query2_lds_bytes() {
 // Staging of the 4 consecutive 32x32 tiles (8 KB) that one chunk of 32 keys shares with the 128
 // queries of a workgroup, one 16-byte piece per thread (512 threads).  Every wave instruction
 // reads 1 KB contiguous; within 16 lanes the LDS rows differ, which keeps the stores conflict free.
-template <typename T>
+// CHAINED: the 8 values of a piece are queries 4g..4g+3 and 8+4g..8+4g+3 of their run of 16 (tiles
+// written from accumulator registers by bwd_keyw1_kernel); the LDS tile is in natural order either way.
+template <typename T, bool CHAINED>
 struct TileStage {
   vec<T, 8> r;
   __device__ __forceinline__ void load(const T* src) {
@@ -1198,7 +1661,15 @@ struct TileStage {
   __device__ __forceinline__ void store(T* dst) const {
     const int slab = threadIdx.x >> 6, l = threadIdx.x & 63;
     const int g = (l >> 4) & 1, k = (l & 15) + 16 * (l >> 5);
-    *reinterpret_cast<frag_mem<T>*>(dst + k * kLdD<T> + 16 * slab + 8 * g) = r;
+    if constexpr (CHAINED) {
+      vec<T, 4> lo, hi;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { lo[e] = r[e]; hi[e] = r[4 + e]; }
+      st4<T>(dst + k * kLdD<T> + 16 * slab + 4 * g, lo);
+      st4<T>(dst + k * kLdD<T> + 16 * slab + 8 + 4 * g, hi);
+    } else {
+      *reinterpret_cast<frag_mem<T>*>(dst + k * kLdD<T> + 16 * slab + 8 * g) = r;
+    }
   }
 };
 
@@ -1276,7 +1747,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
   const T* dsum = reinterpret_cast<const T*>(a.dsu_mat) + (int64_t)bh * a.s.Lp * a.s.Lp + (int64_t)qb * 4 * 1024;
   int kend = qb * QB + QB;
   if (kend > a.s.Lp) kend = a.s.Lp;
-  TileStage<T> pds, pdsu;   // every thread: one piece of each
+  TileStage<T, (HD > 64)> pds, pdsu;   // every thread: one piece of each
 
   if constexpr (LDS_ROWS && DO_S) {
     // rows j of the pair: T'^T[j][i] over the pair's queries (own block from tt_blk; for the first
@@ -1330,7 +1801,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
     if (DO_Q) pkc.load_flat(kc + (int64_t)(K0) * HD, tid);                               \
     pqu.load_flat(qu + (int64_t)(K0) * HD, tid);                                         \
     if (DO_Q && (K0) / kNB < blk0) pu.load(usnap + (usnap_off(blk0) + (K0)) * HD, tid);  \
-    pds.load(dsm + (int64_t)((K0) / 32) * tile_row);                                     \
+    if (DO_Q) pds.load(dsm + (int64_t)((K0) / 32) * tile_row);                           \
     pdsu.load(dsum + (int64_t)((K0) / 32) * tile_row);                                   \
   } while (0)
     CASTLE_BQ2_LOAD_A(0);
@@ -1340,7 +1811,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
       if (DO_Q) pkc.store(s_kc, LDK, tid);
       pqu.store(s_qu, LDK, tid);
       if (DO_Q && Kb < blk0) pu.store(s_ub, LDK, tid);
-      pds.store(s_ds);
+      if (DO_Q) pds.store(s_ds);   // only the dQc product reads dS
       pdsu.store(s_dsu);
       if (k0 + kCK < kend) CASTLE_BQ2_LOAD_A(k0 + kCK);   // in flight while this chunk is processed
       __syncthreads();   // 2: tiles staged
@@ -1473,7 +1944,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
 #define CASTLE_BQ2_LOAD_B(K0)                                                                             \
   do {                                                                                                    \
     if (has_g) pg.load(gsnap + (gsnap_off(blk1) + (K0)) * HD, tid);                                       \
-    pds.load(dsm + (int64_t)((K0) / 32) * tile_row);                                                      \
+    if (DO_Q) pds.load(dsm + (int64_t)((K0) / 32) * tile_row);                                            \
     pdsu.load(dsum + (int64_t)((K0) / 32) * tile_row);                                                    \
   } while (0)
     CASTLE_BQ2_LOAD_B(0);
@@ -1481,7 +1952,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
       const int Kb = k0 / kNB;
       __syncthreads();   // 1
       if (has_g) pg.store(s_g, LDK, tid);
-      pds.store(s_ds);
+      if (DO_Q) pds.store(s_ds);   // only the dQc product reads dS
       pdsu.store(s_dsu);
       if (k0 + kCK < kend) CASTLE_BQ2_LOAD_B(k0 + kCK);
       __syncthreads();   // 2
@@ -1629,7 +2100,11 @@ template <typename T, typename TI, int HD> static int launch_bwd_t(const BwdArgs
     if (!configured3) {
       if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_query2_kernel<T, TI, HD, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_query2_lds_bytes<T, HD>()) != hipSuccess) return -3;
       if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_query2_kernel<T, TI, HD, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_query2_lds_bytes<T, HD>()) != hipSuccess) return -3;
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_key_kernel<T, TI, HD, 2, true>), hipFuncAttributeMaxDynamicSharedMemorySize, key_lds) != hipSuccess) return -3;
+      if constexpr (SPLIT) {
+        static_assert(bwd_keyw1_lds_bytes<T, HD>() <= kMaxLds && bwd_keyw2_lds_bytes<T, HD>() <= kMaxLds, "wide-head key kernels do not fit the LDS");
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_keyw1_kernel<T, TI, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_keyw1_lds_bytes<T, HD>()) != hipSuccess) return -3;
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_keyw2_kernel<T, TI, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_keyw2_lds_bytes<T, HD>()) != hipSuccess) return -3;
+      }
       configured3 = true;
     }
   }
@@ -1653,15 +2128,19 @@ template <typename T, typename TI, int HD> static int launch_bwd_t(const BwdArgs
   {
     ProfScope ps(kSlotBwdKey, stream);
     if constexpr (SPLIT) {
-      hipLaunchKernelGGL((bwd_key_kernel<T, TI, HD, 1>), grid, block, key_lds, stream, a);   // also writes the tiles
       bool from_tiles = false;
       if constexpr (TILES) {
-        if (a.ds_mat != nullptr) {
-          hipLaunchKernelGGL((bwd_key_kernel<T, TI, HD, 2, true>), grid, block, key_lds, stream, a);
+        if (a.ds_mat != nullptr) {   // room for the dS / dSu tiles: the two-role launches
+          constexpr int w1_lds = bwd_keyw1_lds_bytes<T, HD>(), w2_lds = bwd_keyw2_lds_bytes<T, HD>();
+          hipLaunchKernelGGL((bwd_keyw1_kernel<T, TI, HD>), grid, dim3(2 * kThreads), w1_lds, stream, a);
+          hipLaunchKernelGGL((bwd_keyw2_kernel<T, TI, HD>), grid, dim3(2 * kThreads), w2_lds, stream, a);
           from_tiles = true;
         }
       }
-      if (!from_tiles) hipLaunchKernelGGL((bwd_key_kernel<T, TI, HD, 2>), grid, block, key_lds, stream, a);
+      if (!from_tiles) {
+        hipLaunchKernelGGL((bwd_key_kernel<T, TI, HD, 1>), grid, block, key_lds, stream, a);
+        hipLaunchKernelGGL((bwd_key_kernel<T, TI, HD, 2>), grid, block, key_lds, stream, a);
+      }
     } else if constexpr (TWO_ROLE) {
       constexpr int key2_lds = bwd_key2_lds_bytes<T, HD>();
       hipLaunchKernelGGL((bwd_key2_kernel<T, TI, HD>), grid, dim3(2 * kThreads), key2_lds, stream, a);

@@ -10,7 +10,7 @@
 //                The state as of the start of block I is stored as snapshot
 //                usnap[I][k]; the final state is the cache tensor U.
 //   attn_kernel  query-stationary: 128 queries per workgroup (two 64-row blocks),
-//                keys streamed in chunks of 64:
+//                keys streamed in chunks of 64 or 32:
 //                  Su = Qc_I usnap[I][K]^T + T_II A_KI^T,  S = s(Sc - Su sigmoid(s Su)),
 //                online softmax over keys, O = P Vc.
 // The math follows the dense definition at lookahead_keys_attention.py:132-164 of the
@@ -38,8 +38,16 @@ template <typename T, int HD> constexpr int vtile_elems() {
 template <typename T, int HD> constexpr int scan_lds_bytes() {
   return (int)sizeof(T) * (kNB * lds_ld<T>(HD) + vtile_elems<T, HD>());
 }
+// keys per chunk of the attention kernel: 32 for 16-bit operands from d = 64 up.  At d = 128 the smaller
+// tiles and staging registers are what lets two workgroups share a CU (two waves per SIMD instead of
+// one: 5.6 -> 3.8 ms at 16 heads x 16384 tokens); at d = 64 they are worth 1.5 %.
+template <typename T, int HD> constexpr int attn_chunk() { return sizeof(T) == 2 && HD >= 64 ? 32 : kNB; }
+// at d = 128 the T' rows of a wave live in LDS instead of registers (each lane reads back what it wrote)
+template <typename T, int HD> constexpr bool attn_t_in_lds() { return sizeof(T) == 2 && HD == 128; }
 template <typename T, int HD> constexpr int attn_lds_bytes() {
-  return (int)sizeof(T) * (4 * kNB * lds_ld<T>(HD) + vtile_elems<T, HD>() + kNB * lds_ld<T>(128));
+  constexpr int CK = attn_chunk<T, HD>();
+  return (int)sizeof(T) * (4 * CK * lds_ld<T>(HD) + (sizeof(T) == 2 ? CK * lds_ld<T>(HD) : vtile_elems<T, HD>()) + CK * lds_ld<T>(128) +
+                           (attn_t_in_lds<T, HD>() ? 128 * lds_ld<T>(kNB) : 0));
 }
 // register prefetch of the next tile is affordable for 16-bit operands up to d = 64
 template <typename T, int HD> constexpr bool use_prefetch() { return sizeof(T) == 2; }
@@ -311,21 +319,25 @@ __global__ __launch_bounds__(kThreads, (scan_waves_per_simd<T, HD>())) void scan
 
 // ---------------------------------------------------------------------------
 template <typename T, typename TI, int HD>
-__global__ __launch_bounds__(kThreads, (sizeof(T) == 2 && HD <= 64) ? 2 : 1) void attn_kernel(FwdArgs a) {
+__global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void attn_kernel(FwdArgs a) {
   constexpr int KS = HD / 16;
   constexpr int HDP = HD < 32 ? 32 : HD;
   constexpr int NT = HDP / 32;
-  constexpr int KT = kNB / 32;
+  constexpr int CK = attn_chunk<T, HD>();   // keys per chunk
+  constexpr int KT = CK / 32;
   constexpr int QB = 128;
   constexpr int NBLK_Q = QB / kNB;   // snapshot blocks per workgroup
   constexpr int LDK = lds_ld<T>(HD), LDV = lds_ld_chain<T>(kNB), LDA = lds_ld<T>(QB);
   constexpr bool PF = use_prefetch<T, HD>();
-  T* s_kc = reinterpret_cast<T*>(castle_smem);   // [kNB][LDK]
-  T* s_qu = s_kc + kNB * LDK;                    // [kNB][LDK]
-  T* s_ub0 = s_qu + kNB * LDK;                   // [NBLK_Q][kNB][LDK]
-  T* s_vct = s_ub0 + NBLK_Q * kNB * LDK;         // fp32: [HDP][LDV] (transposed); 16-bit: [kNB][LDK]
-  T* s_a = s_vct + vtile_elems<T, HD>();         // [kNB][LDA]
   constexpr bool TRV = sizeof(T) == 2;
+  T* s_kc = reinterpret_cast<T*>(castle_smem);   // [CK][LDK]
+  T* s_qu = s_kc + CK * LDK;                     // [CK][LDK]
+  T* s_ub0 = s_qu + CK * LDK;                    // [NBLK_Q][CK][LDK]
+  T* s_vct = s_ub0 + NBLK_Q * CK * LDK;          // fp32: [HDP][LDV] (transposed); 16-bit: [CK][LDK]
+  T* s_a = s_vct + (TRV ? CK * LDK : vtile_elems<T, HD>());   // [CK][LDA]
+  constexpr bool TL = attn_t_in_lds<T, HD>();
+  constexpr int LDT = lds_ld<T>(kNB);
+  T* s_t = s_a + CK * LDA;                                    // [QB][LDT], only if TL
 
   prio_by_band(blockIdx.x, a.s.cus);
   int rank, bh;
@@ -360,7 +372,10 @@ __global__ __launch_bounds__(kThreads, (sizeof(T) == 2 && HD <= 64) ? 2 : 1) voi
     fku[s] = ldg_nat_scaled<T, T>(ku, HD, i, 16 * s + 8 * g, true, -c1);
   }
 #pragma unroll
-  for (int s = 0; s < kNB / 16; ++s) ft[s] = ldg_nat<T>(tb, kNB, i, 16 * s + 8 * g, s < nintra);
+  for (int s = 0; s < kNB / 16; ++s) {
+    ft[s] = ldg_nat<T>(tb, kNB, i, 16 * s + 8 * g, s < nintra);
+    if (TL) *reinterpret_cast<frag<T>*>(s_t + (32 * wave + c) * LDT + 16 * s + 8 * g) = ft[s];
+  }
 
   acc_t o[NT];
 #pragma unroll
@@ -368,24 +383,26 @@ __global__ __launch_bounds__(kThreads, (sizeof(T) == 2 && HD <= 64) ? 2 : 1) voi
   float m = -INFINITY, l = 0.f;
   if (!TRV && HDP > HD) lds_zero(s_vct + HD * LDV, (HDP - HD) * LDV);
 
-  int nchunks = (qb * QB + QB) / kNB;
-  if (nchunks > a.s.nblk) nchunks = a.s.nblk;
+  int nchunks = (qb * QB + QB) / CK;
+  if (nchunks > a.s.nblk * (kNB / CK)) nchunks = a.s.nblk * (kNB / CK);
 
-  RowStage<T, T, kNB, HD> pkc, pqu, pvr;
-  ColStage<T, T, kNB, HD> pvc;
-  SnapStage<T, kNB, HD> pub[NBLK_Q];
-  auto load_chunk = [&](int Kb) __attribute__((always_inline)) {
-    pkc.load_flat(kc + (int64_t)Kb * kNB * HD);
-    if (TRV) pvr.load_flat(vc + (int64_t)Kb * kNB * HD);
-    else pvc.load(vc, HD, (int64_t)Kb * kNB, kNoRowLimit);
-    pqu.load_flat(qu + (int64_t)Kb * kNB * HD);
+  RowStage<T, T, CK, HD> pkc, pqu, pvr;
+  ColStage<T, T, CK, HD> pvc;
+  SnapStage<T, CK, HD> pub[NBLK_Q];
+  auto load_chunk = [&](int ck) __attribute__((always_inline)) {   // chunk ck = keys [ck*CK, ck*CK + CK)
+    const int Kb = ck * CK / kNB;
+    pkc.load_flat(kc + (int64_t)ck * CK * HD);
+    if (TRV) pvr.load_flat(vc + (int64_t)ck * CK * HD);
+    else pvc.load(vc, HD, (int64_t)ck * CK, kNoRowLimit);
+    pqu.load_flat(qu + (int64_t)ck * CK * HD);
 #pragma unroll
     for (int q = 0; q < NBLK_Q; ++q) {
       const int blk = Ifirst + q;
-      if (Kb < blk && blk < a.s.nblk) pub[q].load(snap + (usnap_off(blk) + (int64_t)Kb * kNB) * HD);
+      if (Kb < blk && blk < a.s.nblk) pub[q].load(snap + (usnap_off(blk) + (int64_t)ck * CK) * HD);
     }
   };
-  auto store_chunk = [&](int Kb) __attribute__((always_inline)) {
+  auto store_chunk = [&](int ck) __attribute__((always_inline)) {
+    const int Kb = ck * CK / kNB;
     pkc.store(s_kc, LDK);
     if (TRV) pvr.store(s_vct, LDK);
     else pvc.store(s_vct, LDV);
@@ -393,7 +410,7 @@ __global__ __launch_bounds__(kThreads, (sizeof(T) == 2 && HD <= 64) ? 2 : 1) voi
 #pragma unroll
     for (int q = 0; q < NBLK_Q; ++q) {
       const int blk = Ifirst + q;
-      if (Kb < blk && blk < a.s.nblk) pub[q].store(s_ub0 + q * kNB * LDK, LDK);
+      if (Kb < blk && blk < a.s.nblk) pub[q].store(s_ub0 + q * CK * LDK, LDK);
     }
   };
 
@@ -402,13 +419,15 @@ __global__ __launch_bounds__(kThreads, (sizeof(T) == 2 && HD <= 64) ? 2 : 1) voi
 #pragma unroll
   for (int s = 0; s < KS; ++s) { asm volatile("" : "+v"(fqc[s])); asm volatile("" : "+v"(fku[s])); }
 #pragma unroll
-  for (int s = 0; s < kNB / 16; ++s) asm volatile("" : "+v"(ft[s]));
+  for (int s = 0; s < kNB / 16; ++s)
+    if (!TL) asm volatile("" : "+v"(ft[s]));
   if (PF) load_chunk(0);
-  for (int Kb = 0; Kb < nchunks; ++Kb) {
+  for (int ck = 0; ck < nchunks; ++ck) {
+    const int Kb = ck * CK / kNB;
     __syncthreads();
-    if (!PF) load_chunk(Kb);
-    store_chunk(Kb);
-    if (PF && Kb + 1 < nchunks) load_chunk(Kb + 1);   // in flight while this chunk is processed
+    if (!PF) load_chunk(ck);
+    store_chunk(ck);
+    if (PF && ck + 1 < nchunks) load_chunk(ck + 1);   // in flight while this chunk is processed
     __syncthreads();
     const bool active = Kb <= Iw;
     if (active) {
@@ -422,7 +441,7 @@ __global__ __launch_bounds__(kThreads, (sizeof(T) == 2 && HD <= 64) ? 2 : 1) voi
 #pragma unroll
         for (int r = 0; r < 16; ++r) aT[r] = fast_rcp(1.f + fast_exp2(aT[r]));
         if (Kb == Iw) {
-          const int kk = Kb * kNB + 32 * kt + c;
+          const int kk = ck * CK + 32 * kt + c;
 #pragma unroll
           for (int r = 0; r < 16; ++r)
             if (i0w + acc_row(r, g) <= kk) aT[r] = 0.f;
@@ -435,7 +454,7 @@ __global__ __launch_bounds__(kThreads, (sizeof(T) == 2 && HD <= 64) ? 2 : 1) voi
     if (active) {
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt) {
-        const int k0 = Kb * kNB + 32 * kt;
+        const int k0 = ck * CK + 32 * kt;
         if (k0 > i0w + 31) continue;
         acc_t sc, su;
         zero(sc);
@@ -446,9 +465,10 @@ __global__ __launch_bounds__(kThreads, (sizeof(T) == 2 && HD <= 64) ? 2 : 1) voi
         // starts the accumulator is unconditional and takes the zero as a constant operand
 #pragma unroll
         for (int s = 0; s < kNB / 16; ++s)
-          if (s < 2 || s < nintra) mma(su, ld_nat<T>(s_a, LDA, 32 * kt + c, cb + 16 * s + 8 * g), ft[s]);
+          if (s < 2 || s < nintra)
+            mma(su, ld_nat<T>(s_a, LDA, 32 * kt + c, cb + 16 * s + 8 * g), TL ? ld_nat<T>(s_t, LDT, 32 * wave + c, 16 * s + 8 * g) : ft[s]);
         if (Kb < Iw) {
-          const T* ub = s_ub0 + (Iw - Ifirst) * kNB * LDK;
+          const T* ub = s_ub0 + (Iw - Ifirst) * CK * LDK;
 #pragma unroll
           for (int s = 0; s < KS; ++s) mma(su, ld_nat<T>(ub, LDK, 32 * kt + c, 16 * s + 8 * g), fqc[s]);
         }
