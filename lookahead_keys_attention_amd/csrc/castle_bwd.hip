@@ -55,14 +55,15 @@ constexpr int a16(int bytes) { return (bytes + 15) / 16 * 16; }
 // [n rows, lanes] accumulator tiles -> (row = lane index, 4 consecutive n) stores, scaled
 // Writes one gradient row held as accumulator tiles [n rows, this lane's row].  rope_pos >= 0: the
 // operand was rotated by that position before use, so its gradient is rotated back first.
+// The NT tiles are columns 32 nt0 .. 32 (nt0 + NT) - 1 of the row.
 template <typename T, int HD, int NT>   // T: element type of the destination tensor
-__device__ __forceinline__ void store_rows(T* dst_row, acc_t (&acc)[NT], float mul, int g, int rope_pos = -1) {
+__device__ __forceinline__ void store_rows(T* dst_row, acc_t (&acc)[NT], float mul, int g, int rope_pos = -1, int nt0 = 0) {
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
     if (rope_pos >= 0) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int n = 32 * nt + 8 * q + 4 * g;
+        const int n = 32 * (nt0 + nt) + 8 * q + 4 * g;
         if (n < HD) {
           CASTLE_ROPE_PAIR(acc[nt][4 * q], acc[nt][4 * q + 1], (float)rope_pos, n / 2, HD, true);
           CASTLE_ROPE_PAIR(acc[nt][4 * q + 2], acc[nt][4 * q + 3], (float)rope_pos, n / 2 + 1, HD, true);
@@ -73,7 +74,7 @@ __device__ __forceinline__ void store_rows(T* dst_row, acc_t (&acc)[NT], float m
     for (int r = 0; r < 16; ++r) acc[nt][r] *= mul;
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      const int n = 32 * nt + 8 * q + 4 * g;
+      const int n = 32 * (nt0 + nt) + 8 * q + 4 * g;
       if (n < HD) st4<T>(dst_row + n, pack4<T>(acc[nt], q));
     }
   }
@@ -788,14 +789,14 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_key2_kernel(BwdArgs a) {
 //                                               (snapshots), dA = G Vu^T + dSu^T T' -> LDS for the partner
 // Pair (w, w + 4) owns keys kb*128 + 32 w .. + 31, as in bwd_key2_kernel.
 template <typename T, int HD> constexpr int bwd_keyw1_lds_bytes() {
-  int b = 3 * a16((int)sizeof(T) * kNB * lds_ld<T>(HD));    // qc, do, ku
+  int b = 3 * a16((int)sizeof(T) * kNB * lds_ld_tr<T>(HD));    // qc, do, ku
   b += a16((int)sizeof(T) * kNB * lds_ld_chain<T>(kNB));    // T'
   b += 2 * a16(4 * kNB);                                    // lse, delta
   b += 4 * 3 * a16((int)sizeof(T) * 32 * lds_ld<T>(kNB));   // P, dS, dSu per wave pair
   return b;
 }
 template <typename T, int HD> constexpr int bwd_keyw2_lds_bytes() {
-  int b = 3 * a16((int)sizeof(T) * kNB * lds_ld<T>(HD));    // qc, ku (two blocks)
+  int b = 3 * a16((int)sizeof(T) * kNB * lds_ld_tr<T>(HD));    // qc, ku (two blocks)
   b += a16((int)sizeof(T) * kNB * lds_ld_chain<T>(HD));     // vu
   b += a16((int)sizeof(T) * kNB * lds_ld_chain<T>(kNB));    // T'
   b += 2 * 4 * a16((int)sizeof(T) * 32 * lds_ld<T>(kNB));   // dA per wave pair, two blocks
@@ -808,7 +809,7 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_keyw1_kernel(BwdArgs a) {
   constexpr int KS = HD / 16;
   constexpr int NT = HD / 32;
   constexpr int BT = kNB / 32;
-  constexpr int LDK = lds_ld<T>(HD), LDT = lds_ld_chain<T>(kNB), LDX = lds_ld<T>(kNB);
+  constexpr int LDK = lds_ld_tr<T>(HD), LDT = lds_ld_chain<T>(kNB), LDX = lds_ld<T>(kNB);
 
   Carver cv{castle_smem};
   T* s_qc = cv.take<T>(kNB * LDK);
@@ -1068,7 +1069,7 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_keyw2_kernel(BwdArgs a) {
   constexpr int KS = HD / 16;
   constexpr int NT = HD / 32;
   constexpr int BT = kNB / 32;
-  constexpr int LDK = lds_ld<T>(HD), LDU = lds_ld_chain<T>(HD), LDT = lds_ld_chain<T>(kNB), LDX = lds_ld<T>(kNB);
+  constexpr int LDK = lds_ld_tr<T>(HD), LDU = lds_ld_chain<T>(HD), LDT = lds_ld_chain<T>(kNB), LDX = lds_ld<T>(kNB);
   // dA crosses the LDS as a 16-bit value: a quarter of it, so that it needs no more range than
   // dZ = dA A (1 - A) <= dA / 4, which is a 16-bit MFMA operand in every variant of this kernel
   constexpr float kHand = 0.25f, kUnhand = 4.f;
@@ -1118,37 +1119,40 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_keyw2_kernel(BwdArgs a) {
       for (int q = 0; q < 4; ++q) w[jt][q] = vec<T, 4>{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
     RowStage<T, T, kNB, HD> pku, pqc, pvu;
     RowStage<T, T, kNB, kNB> ptb;
-#define CASTLE_BKW_LOAD(I_)                                  \
-  do {                                                       \
-    const int64_t r_ = (int64_t)(I_) * kNB;                  \
-    pku.load_flat(ku + r_ * HD);                             \
-    pqc.load_flat(qc + r_ * HD);                             \
-    pvu.load_flat(vu + r_ * HD);                             \
-    ptb.load_flat(tb + r_ * kNB);                            \
+    // The pieces of the next block are requested in four portions spread over the block: the CU takes
+    // one 1 KB wave load per 16 cycles, and a burst of all 56 of them held every wave of the workgroup
+    // up for more than a thousand cycles behind barrier 1.
+#define CASTLE_BKW_LOAD(I_, PORTION)                                        \
+  do {                                                                      \
+    const int64_t r_ = (int64_t)(I_) * kNB;                                 \
+    if ((PORTION) == 0 || (PORTION) < 0) pku.load_flat(ku + r_ * HD);       \
+    if ((PORTION) == 1 || (PORTION) < 0) pqc.load_flat(qc + r_ * HD);       \
+    if ((PORTION) == 2 || (PORTION) < 0) pvu.load_flat(vu + r_ * HD);       \
+    if ((PORTION) == 3 || (PORTION) < 0) ptb.load_flat(tb + r_ * kNB);      \
   } while (0)
     // dZ^T = dA^T * A (1 - A)  ->  dQu, for source block J: its Ku tile is still in its buffer
-#define CASTLE_BKW_DQU(J_)                                                                           \
+#define CASTLE_BKW_DQU(J_, JT_)                                                                      \
   do {                                                                                               \
     const T* ku_tile_ = CASTLE_BKW_KU(J_);                                                           \
     const T* da_tile_ = CASTLE_BKW_DA(J_);                                                           \
-    _Pragma("unroll") for (int jt = 0; jt < BT; ++jt) {                                              \
-      acc_t dz;                                                                                      \
-      _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                                \
-        const vec<T, 4> d4 = *reinterpret_cast<const vec4_mem<T>*>(da_tile_ + c * LDX + 32 * jt + 8 * q + 4 * g); \
-        _Pragma("unroll") for (int e = 0; e < 4; ++e) dz[4 * q + e] = (float)d4[e] * (float)w[jt][q][e]; \
-      }                                                                                              \
-      _Pragma("unroll") for (int s2 = 0; s2 < 2; ++s2) {                                             \
-        frag<T> okt[NT];                                                                             \
-        _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                            \
-          okt[nt] = ld_free<T, true>(ku_tile_, LDK, 32 * nt, HD, 32 * jt + 16 * s2, c, g);           \
-        __builtin_amdgcn_sched_barrier(0);                                                           \
-        const frag<T> fdz = chain<T>(dz, s2);                                                        \
-        _Pragma("unroll") for (int nt = 0; nt < NT; ++nt) mma(dqu[nt], okt[nt], fdz);                \
-      }                                                                                              \
+    constexpr int jt = (JT_);                                                                        \
+    acc_t dz;                                                                                        \
+    _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                                  \
+      const vec<T, 4> d4 = *reinterpret_cast<const vec4_mem<T>*>(da_tile_ + c * LDX + 32 * jt + 8 * q + 4 * g); \
+      _Pragma("unroll") for (int e = 0; e < 4; ++e) dz[4 * q + e] = (float)d4[e] * (float)w[jt][q][e]; \
+    }                                                                                                \
+    _Pragma("unroll") for (int s2 = 0; s2 < 2; ++s2) {                                               \
+      frag<T> okt[NT];                                                                               \
+      _Pragma("unroll") for (int nt = 0; nt < NT; ++nt)                                              \
+        okt[nt] = ld_free<T, true>(ku_tile_, LDK, 32 * nt, HD, 32 * jt + 16 * s2, c, g);             \
+      __builtin_amdgcn_sched_barrier(0);                                                             \
+      const frag<T> fdz = chain<T>(dz, s2);                                                          \
+      _Pragma("unroll") for (int nt = 0; nt < NT; ++nt) mma(dqu[nt], okt[nt], fdz);                  \
     }                                                                                                \
   } while (0)
 
-    CASTLE_BKW_LOAD(Ilast);
+    static_assert(BT == 2, "the portions below are placed around two gate tiles");
+    CASTLE_BKW_LOAD(Ilast, -1);
     for (int I = Ilast; I >= I0; --I) {
       // every wave has passed the end barrier of block I + 1: its tiles are free, and so is the Ku
       // buffer of block I + 2, which block I takes over
@@ -1157,12 +1161,17 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_keyw2_kernel(BwdArgs a) {
       ptb.store_halves(s_t, LDT);
       pku.store(CASTLE_BKW_KU(I), LDK);
       __syncthreads();   // 1: tiles staged
-      if (I > I0) CASTLE_BKW_LOAD(I - 1);   // in flight for the whole block
-      if (I < Ilast && I + 1 >= Iw) CASTLE_BKW_DQU(I + 1);   // finish the previous block
+      const bool more = I > I0, owed = I < Ilast && I + 1 >= Iw;
+      if (more) CASTLE_BKW_LOAD(I - 1, 0);
+      if (owed) CASTLE_BKW_DQU(I + 1, 0);   // finish the previous block
+      if (more) CASTLE_BKW_LOAD(I - 1, 1);
+      if (owed) CASTLE_BKW_DQU(I + 1, 1);
+      if (more) CASTLE_BKW_LOAD(I - 1, 2);
       if (I >= Iw) {   // gate of this block: 4 A (1 - A) stays in registers until its dA arrives
         const T* ku_tile = CASTLE_BKW_KU(I);
 #pragma unroll
         for (int jt = 0; jt < BT; ++jt) {
+          if (jt == 1 && more) CASTLE_BKW_LOAD(I - 1, 3);
           acc_t aT;
           zero(aT);
 #pragma unroll
@@ -1191,7 +1200,10 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_keyw2_kernel(BwdArgs a) {
       }
       __syncthreads();   // 2: block done, dA of block I written
     }
-    if (I0 >= Iw) CASTLE_BKW_DQU(I0);
+    if (I0 >= Iw) {
+      CASTLE_BKW_DQU(I0, 0);
+      CASTLE_BKW_DQU(I0, 1);
+    }
 #undef CASTLE_BKW_LOAD
 #undef CASTLE_BKW_DQU
     if (k < L) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqu, b, h) + (int64_t)k * a.dqu.sl, dqu, c0 * kLn2 * gun, g, a.s.rotary ? k : -1);
@@ -1230,7 +1242,7 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_keyw2_kernel(BwdArgs a) {
       // reverse state as of block I; the query-stationary kernel reads those behind a pair of blocks
       if (active && I <= a.s.nblk - 2 && (I & 1)) store_snap_tile<T, HD, NT>(gsnap + (gsnap_off(I) + kw0) * HD, G, c, g);
       __syncthreads();   // 1: tiles staged
-      if (I > I0) CASTLE_BKW_TILES(tnext, I - 1);
+      if (!active && I > I0) CASTLE_BKW_TILES(tnext, I - 1);
       if (active) {
         // dA^T[j rows, k lanes] of this block, second term first: G (before this block) times Vu^T
         acc_t dA[BT];
@@ -1247,6 +1259,7 @@ __global__ __launch_bounds__(2 * kThreads, 1) void bwd_keyw2_kernel(BwdArgs a) {
             for (int u = 0; u < 4; ++u) mma(dA[jt], ovu[u], chain<T>(G[(s0 + u) / 2], (s0 + u) % 2));
           }
         }
+        if (I > I0) CASTLE_BKW_TILES(tnext, I - 1);   // behind the partner's requests, which come right after barrier 1
 #pragma unroll
         for (int it = 0; it < BT; ++it) {
           const int i0 = I * kNB + 32 * it;
@@ -1628,20 +1641,19 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_query_kernel(BwdArgs a) {
 }
 
 // ---------------------------------------------------------------------------
-// Query-stationary backward that consumes the dS / dSu tiles written by bwd_key2_kernel
-// (16-bit compute types, d <= 64): no score recomputation, only the gate.
+// Query-stationary backward that consumes the dS / dSu tiles written by the key-stationary kernels
+// (16-bit compute types): no score recomputation, only the gate.
 //   row = query i:   dQc += dS Kc + dSu U_I,  dT^T += A^T dSu^T
 //   row = source j:  dA = dSu^T T' + G' Vu^T,  dZ = dA A (1 - A),  dKu += dZ^T Qu,  dVu += A^T G'
 template <typename T> constexpr int kLdD = 128 + 8;   // dS / dSu tiles [key][128 queries]
 template <typename T> constexpr int kLdA = kCK + 8;   // gate tile [128 sources][key]
 template <typename T> constexpr int kLdT2 = 128 + 4;  // dT of the row pair [128 queries][128 sources]
-template <typename T> constexpr int kLdTT = 128 + 8;  // T'^T rows of the pair [128 sources][128 queries] (d = 128 only)
+template <typename T> constexpr int kLdTT = 128 + 8;  // T'^T rows of the pair [128 sources][128 queries] (bwd_queryw_kernel)
 template <typename T, int HD> constexpr int bwd_query2_lds_bytes() {
-  int b = 4 * a16((int)sizeof(T) * kCK * lds_ld<T>(HD));          // kc, qu, ub, g
+  int b = 4 * a16((int)sizeof(T) * kCK * lds_ld_tr<T>(HD));       // kc, qu, ub, g
   b += a16((int)sizeof(T) * 128 * kLdA<T>);                       // A^T [j][k]
   b += 2 * a16((int)sizeof(T) * kCK * kLdD<T>);                   // dS, dSu [k][i]
-  if (HD > 64) b += a16((int)sizeof(T) * 128 * kLdTT<T>) + a16((int)sizeof(T) * 128 * lds_ld<T>(HD));   // T'^T and vu rows
-  int e = 2 * a16((int)sizeof(T) * 128 * lds_ld<T>(HD)) + a16((int)sizeof(T) * 128 * kLdT2<T>);
+  int e = 2 * a16((int)sizeof(T) * 128 * lds_ld_tr<T>(HD)) + a16((int)sizeof(T) * 128 * kLdT2<T>);
   return b > e ? b : e;
 }
 
@@ -1685,22 +1697,18 @@ struct TileStage {
 //   dA[k,j]  = sum_{i in pair, i >= j} dSu[i,k] T'[i,j] + G'[k] . vu_j
 //   dQc[i]  += sum_k dSu[i,k] U[k]  (keys before the pair)  + sum_{j in pair, j <= i} dT[i,j] vu_j
 //   dVu[j]  += sum_k A[k,j] G'[k] + sum_{i in pair, i >= j} dT[i,j] qc'_i,   dT[i,j] = sum_k dSu[i,k] A[k,j]
-// PART selects the outputs of a launch: 0 = all (d <= 64); at d = 128, where the accumulators of
-// all outputs do not fit the register file, 1 = dQc and 2 = dKu, dVu (gate and dT are formed in
-// both).  At d = 128 the T'^T and vu rows of the pair also sit in LDS instead of registers.
-template <typename T, typename TI, int HD, int PART>
+// Head dimensions up to 64: the accumulators of all outputs fit two waves per SIMD (bwd_queryw_kernel
+// below is the same kernel laid out for d = 128).
+template <typename T, typename TI, int HD>
 __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) {
-  static_assert(sizeof(T) == 2 && kCK == 32, "tile consumer: 16-bit operands");
-  static_assert((PART == 0) == (HD <= 64), "one launch up to d = 64, two at d = 128");
-  constexpr bool DO_Q = PART != 2, DO_S = PART != 1;
-  constexpr bool LDS_ROWS = HD > 64;   // T'^T / vu rows of the pair in LDS, not in registers
+  static_assert(sizeof(T) == 2 && kCK == 32 && HD <= 64, "tile consumer: 16-bit operands, d <= 64");
   constexpr int KS = HD / 16;
   constexpr int HDP = HD < 32 ? 32 : HD;
   constexpr int NT = HDP / 32;
   constexpr int QB = 128;
   constexpr int PT = QB / 32;    // 32-row tiles across the pair
   constexpr int PS = QB / 16;    // 16-deep steps across the pair
-  constexpr int LDK = lds_ld<T>(HD), LDT = kLdT2<T>, LDA = kLdA<T>, LDD = kLdD<T>, LDTT = kLdTT<T>;
+  constexpr int LDK = lds_ld_tr<T>(HD), LDT = kLdT2<T>, LDA = kLdA<T>, LDD = kLdD<T>;
 
   Carver cv{castle_smem};
   T* s_kc = cv.take<T>(kCK * LDK);
@@ -1710,8 +1718,6 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
   T* s_at = cv.take<T>(QB * LDA);    // gate, [source j][key k]
   T* s_ds = cv.take<T>(kCK * LDD);   // dS,  [key k][query i]
   T* s_dsu = cv.take<T>(kCK * LDD);  // dSu, [key k][query i]
-  T* s_tt = LDS_ROWS ? cv.take<T>(QB * LDTT) : nullptr;   // T'^T [source j][query i of the pair]
-  T* s_vu = LDS_ROWS ? cv.take<T>(QB * LDK) : nullptr;    // vu rows of the pair
   // the epilogue reuses the same memory
   Carver ce{castle_smem};
   T* e_vu = ce.take<T>(QB * LDK);
@@ -1734,7 +1740,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
   const int i = i0w + c;                      // this lane's row
   const int blk0 = 2 * qb, blk1 = 2 * qb + 1;
   const int sfirst = jw / 16;                 // first step covering queries i >= j
-  const bool has_g = DO_S && blk1 <= a.s.nblk - 2;    // a reverse state exists behind the pair (and is needed)
+  const bool has_g = blk1 <= a.s.nblk - 2;    // a reverse state exists behind the pair
 
   const T* qc = prep_ptr<T>(a.ws.qc_p, bh, a.s.Lp, HD);
   const T* vu = prep_ptr<T>(a.ws.vu_p, bh, a.s.Lp, HD);
@@ -1747,26 +1753,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
   const T* dsum = reinterpret_cast<const T*>(a.dsu_mat) + (int64_t)bh * a.s.Lp * a.s.Lp + (int64_t)qb * 4 * 1024;
   int kend = qb * QB + QB;
   if (kend > a.s.Lp) kend = a.s.Lp;
-  TileStage<T, (HD > 64)> pds, pdsu;   // every thread: one piece of each
-
-  if constexpr (LDS_ROWS && DO_S) {
-    // rows j of the pair: T'^T[j][i] over the pair's queries (own block from tt_blk; for the first
-    // block the second block's queries from the cross quarter), and vu_j.  Columns a row never
-    // uses (queries before its block) are left unwritten.
-    constexpr int VH = kNB / 8;   // 16-byte pieces per half row
-    for (int p = threadIdx.x; p < QB * 2 * VH; p += 2 * kThreads) {
-      const int j = p / (2 * VH), half = (p / VH) & 1, v = p % VH;
-      const bool first = j < kNB;
-      if (!first && half == 0) continue;
-      const T* src = (first && half == 1) ? ttx : ttb;
-      *reinterpret_cast<frag_mem<T>*>(s_tt + j * LDTT + half * kNB + v * 8) =
-          *reinterpret_cast<const frag_mem<T>*>(src + ((int64_t)qb * QB + j) * kNB + v * 8);
-    }
-    RowStage<T, T, QB, HD, 2 * kThreads> st;
-    st.load_flat(vu + (int64_t)qb * QB * HD);
-    st.store(s_vu, LDK);
-    // visible after the first barrier of the chunk loop; first used behind its third
-  }
+  TileStage<T, false> pds, pdsu;   // every thread: one piece of each
 
   if (source_role) {
     const T* kc = prep_ptr<T>(a.ws.kc_p, bh, a.s.Lp, HD);
@@ -1774,44 +1761,40 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
     const T* ku = prep_ptr<T>(a.ws.ku_p, bh, a.s.Lp, HD);
     // T'^T rows of this wave across the queries of the pair: its own block from tt_blk, and for a
     // wave of the first block the second block from the cross quarter
-    constexpr int NREG = (LDS_ROWS || !DO_S) ? 1 : PS;   // register copies only up to d = 64
-    constexpr int NVU = (LDS_ROWS || !DO_S) ? 1 : KS;
-    frag<T> fku[KS], fvu[NVU], ftt[NREG];
+    frag<T> fku[KS], fvu[KS], ftt[PS];
 #pragma unroll
     for (int s = 0; s < KS; ++s) fku[s] = ldg_nat_scaled<T, T>(ku, HD, i, 16 * s + 8 * g, true, -c1);
-    if constexpr (DO_S && !LDS_ROWS) {
 #pragma unroll
-      for (int s = 0; s < KS; ++s) fvu[s] = ldg_nat<T>(vu, HD, i, 16 * s + 8 * g, true);
+    for (int s = 0; s < KS; ++s) fvu[s] = ldg_nat<T>(vu, HD, i, 16 * s + 8 * g, true);
 #pragma unroll
-      for (int s = 0; s < PS; ++s) {
-        const bool own = (s < PS / 2) == (pw < 2);   // queries of step s lie in this wave's own block
-        const T* src = own ? ttb : ttx;
-        ftt[s] = ldg_nat<T>(src, kNB, i, 16 * (s % (PS / 2)) + 8 * g, s >= sfirst);
-      }
+    for (int s = 0; s < PS; ++s) {
+      const bool own = (s < PS / 2) == (pw < 2);   // queries of step s lie in this wave's own block
+      const T* src = own ? ttb : ttx;
+      ftt[s] = ldg_nat<T>(src, kNB, i, 16 * (s % (PS / 2)) + 8 * g, s >= sfirst);
     }
-    acc_t dku[DO_S ? NT : 1];   // [n rows, j lanes]
+    acc_t dku[NT];   // [n rows, j lanes]
 #pragma unroll
-    for (int nt = 0; nt < (DO_S ? NT : 1); ++nt) zero(dku[nt]);
+    for (int nt = 0; nt < NT; ++nt) zero(dku[nt]);
 
     // this role stages kc, qu and the lookahead state
     RowStage<T, T, kCK, HD> pkc, pqu;
     SnapStage<T, kCK, HD> pu;
 #define CASTLE_BQ2_LOAD_A(K0)                                                            \
   do {                                                                                   \
-    if (DO_Q) pkc.load_flat(kc + (int64_t)(K0) * HD, tid);                               \
+    pkc.load_flat(kc + (int64_t)(K0) * HD, tid);                                         \
     pqu.load_flat(qu + (int64_t)(K0) * HD, tid);                                         \
-    if (DO_Q && (K0) / kNB < blk0) pu.load(usnap + (usnap_off(blk0) + (K0)) * HD, tid);  \
-    if (DO_Q) pds.load(dsm + (int64_t)((K0) / 32) * tile_row);                           \
+    if ((K0) / kNB < blk0) pu.load(usnap + (usnap_off(blk0) + (K0)) * HD, tid);          \
+    pds.load(dsm + (int64_t)((K0) / 32) * tile_row);                                     \
     pdsu.load(dsum + (int64_t)((K0) / 32) * tile_row);                                   \
   } while (0)
     CASTLE_BQ2_LOAD_A(0);
     for (int k0 = 0; k0 < kend; k0 += kCK) {
       const int Kb = k0 / kNB;
       __syncthreads();   // 1: tiles free
-      if (DO_Q) pkc.store(s_kc, LDK, tid);
+      pkc.store(s_kc, LDK, tid);
       pqu.store(s_qu, LDK, tid);
-      if (DO_Q && Kb < blk0) pu.store(s_ub, LDK, tid);
-      if (DO_Q) pds.store(s_ds);   // only the dQc product reads dS
+      if (Kb < blk0) pu.store(s_ub, LDK, tid);
+      pds.store(s_ds);
       pdsu.store(s_dsu);
       if (k0 + kCK < kend) CASTLE_BQ2_LOAD_A(k0 + kCK);   // in flight while this chunk is processed
       __syncthreads();   // 2: tiles staged
@@ -1843,77 +1826,44 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
 #pragma unroll
       for (int q = 0; q < 4; ++q) st4<T>(s_at + (jw + c) * LDA + 8 * q + 4 * g, pack4<T>(aK, q));
       __syncthreads();   // 3: gate shared
-      if (!live || !DO_S) continue;
+      if (!live) continue;
       // dA in two accumulators (two dependent MFMA chains instead of one of up to twelve)
       acc_t dA, dA2;
       zero(dA);
       zero(dA2);
-      if constexpr (!LDS_ROWS) {
-        frag<T> og[KS];
+      frag<T> og[KS];
 #pragma unroll
-        for (int s = 0; s < KS; ++s) og[s] = has_g ? ld_nat<T>(s_g, LDK, c, 16 * s + 8 * g) : zero_frag<T>();
+      for (int s = 0; s < KS; ++s) og[s] = has_g ? ld_nat<T>(s_g, LDK, c, 16 * s + 8 * g) : zero_frag<T>();
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {   // two batches keep the operand fragments in registers
-          frag<T> ods[PS / 2];
+      for (int half = 0; half < 2; ++half) {   // two batches keep the operand fragments in registers
+        frag<T> ods[PS / 2];
 #pragma unroll
-          for (int u = 0; u < PS / 2; ++u) ods[u] = ld_nat<T>(s_dsu, LDD, c, 16 * (PS - 1 - (half * (PS / 2) + u)) + 8 * g);
-          __builtin_amdgcn_sched_barrier(0);
-          // steps from the last one down: the last two run for every wave, so the product that starts
-          // dA is unconditional and takes the zero as a constant operand
+        for (int u = 0; u < PS / 2; ++u) ods[u] = ld_nat<T>(s_dsu, LDD, c, 16 * (PS - 1 - (half * (PS / 2) + u)) + 8 * g);
+        __builtin_amdgcn_sched_barrier(0);
+        // steps from the last one down: the last two run for every wave, so the product that starts
+        // dA is unconditional and takes the zero as a constant operand
 #pragma unroll
-          for (int u = 0; u < PS / 2; ++u) {
-            const int step = PS - 1 - (half * (PS / 2) + u);
-            if (step >= PS - 2 || step >= sfirst) mma(dA, ods[u], ftt[NREG == 1 ? 0 : step]);
-            if (half == 0 && u < KS) mma(dA2, og[u], fvu[NVU == 1 ? 0 : u]);   // og is zero where no reverse state exists
-          }
-        }
-      } else {
-#pragma unroll
-        for (int half = 0; half < 2; ++half) {   // dSu^T T'
-          frag<T> ods[PS / 2], ott[PS / 2];
-#pragma unroll
-          for (int u = 0; u < PS / 2; ++u) {
-            ods[u] = ld_nat<T>(s_dsu, LDD, c, 16 * (half * (PS / 2) + u) + 8 * g);
-            ott[u] = ld_nat<T>(s_tt, LDTT, jw + c, 16 * (half * (PS / 2) + u) + 8 * g);
-          }
-          __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int u = 0; u < PS / 2; ++u)
-            if (half * (PS / 2) + u >= sfirst) mma(dA, ods[u], ott[u]);
-        }
-#pragma unroll
-        for (int s0 = 0; s0 < KS; s0 += 4) {   // G' Vu^T; og is zero where no reverse state exists
-          frag<T> og[4], ovu[4];
-#pragma unroll
-          for (int u = 0; u < 4; ++u) {
-            og[u] = has_g ? ld_nat<T>(s_g, LDK, c, 16 * (s0 + u) + 8 * g) : zero_frag<T>();
-            ovu[u] = ld_nat<T>(s_vu, LDK, jw + c, 16 * (s0 + u) + 8 * g);
-          }
-          __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int u = 0; u < 4; ++u)
-            if (s0 + u < KS) mma(dA2, og[u], ovu[u]);
+        for (int u = 0; u < PS / 2; ++u) {
+          const int step = PS - 1 - (half * (PS / 2) + u);
+          if (step >= PS - 2 || step >= sfirst) mma(dA, ods[u], ftt[step]);
+          if (half == 0 && u < KS) mma(dA2, og[u], fvu[u]);   // og is zero where no reverse state exists
         }
       }
       acc_t dz;
 #pragma unroll
       for (int r = 0; r < 16; ++r) dz[r] = (dA[r] + dA2[r]) * __builtin_fmaf(-aK[r], aK[r], aK[r]);   // A (1 - A) in one instruction
       {
-        constexpr int SB = LDS_ROWS ? 1 : 2;
+        frag<T> oqt[2][NT];
 #pragma unroll
-        for (int s0 = 0; s0 < 2; s0 += SB) {
-          frag<T> oqt[SB][NT];
+        for (int u = 0; u < 2; ++u)
 #pragma unroll
-          for (int u = 0; u < SB; ++u)
+          for (int nt = 0; nt < NT; ++nt) oqt[u][nt] = ld_free<T, true>(s_qu, LDK, 32 * nt, HD, 16 * u, c, g);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) oqt[u][nt] = ld_free<T, true>(s_qu, LDK, 32 * nt, HD, 16 * (s0 + u), c, g);
-          __builtin_amdgcn_sched_barrier(0);
+        for (int u = 0; u < 2; ++u) {
+          const frag<T> fdz = chain<T>(dz, u);
 #pragma unroll
-          for (int u = 0; u < SB; ++u) {
-            const frag<T> fdz = chain<T>(dz, s0 + u);
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) mma(dku[DO_S ? nt : 0], oqt[u][nt], fdz);
-          }
+          for (int nt = 0; nt < NT; ++nt) mma(dku[nt], oqt[u][nt], fdz);
         }
       }
     }
@@ -1922,21 +1872,19 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
     __syncthreads();   // e1: chunk tiles dead
     {
       RowStage<T, T, QB, HD, 2 * kThreads> st;
-      if (DO_Q) { st.load_flat(vu + (int64_t)qb * QB * HD); st.store(e_vu, LDK); }
-      if (DO_S) { st.load_flat(qc + (int64_t)qb * QB * HD); st.store(e_qc, LDK); }
+      st.load_flat(vu + (int64_t)qb * QB * HD); st.store(e_vu, LDK);
+      st.load_flat(qc + (int64_t)qb * QB * HD); st.store(e_qc, LDK);
     }
     __syncthreads();   // e2: epilogue tiles and dT shared
-    if constexpr (DO_S) {
-      if (i < L) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dku, b, h) + (int64_t)i * a.dku.sl, dku, c0 * kLn2 * gun, g, a.s.rotary ? i : -1);
-    }
+    if (i < L) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dku, b, h) + (int64_t)i * a.dku.sl, dku, c0 * kLn2 * gun, g, a.s.rotary ? i : -1);
   } else {
-    acc_t dqc[DO_Q ? NT : 1];   // [n rows, i lanes]
-    acc_t dvu[DO_S ? NT : 1];   // [n rows, j lanes]: this role's rows taken as lookahead sources
+    acc_t dqc[NT];   // [n rows, i lanes]
+    acc_t dvu[NT];   // [n rows, j lanes]: this role's rows taken as lookahead sources
     acc_t dtacc[PT];            // [j rows (pair local), i lanes]
 #pragma unroll
-    for (int nt = 0; nt < (DO_Q ? NT : 1); ++nt) zero(dqc[nt]);
+    for (int nt = 0; nt < NT; ++nt) zero(dqc[nt]);
 #pragma unroll
-    for (int nt = 0; nt < (DO_S ? NT : 1); ++nt) zero(dvu[nt]);
+    for (int nt = 0; nt < NT; ++nt) zero(dvu[nt]);
 #pragma unroll
     for (int jt = 0; jt < PT; ++jt) zero(dtacc[jt]);
     // this role stages the reverse state
@@ -1944,7 +1892,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
 #define CASTLE_BQ2_LOAD_B(K0)                                                                             \
   do {                                                                                                    \
     if (has_g) pg.load(gsnap + (gsnap_off(blk1) + (K0)) * HD, tid);                                       \
-    if (DO_Q) pds.load(dsm + (int64_t)((K0) / 32) * tile_row);                                            \
+    pds.load(dsm + (int64_t)((K0) / 32) * tile_row);                                                      \
     pdsu.load(dsum + (int64_t)((K0) / 32) * tile_row);                                                    \
   } while (0)
     CASTLE_BQ2_LOAD_B(0);
@@ -1952,41 +1900,32 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
       const int Kb = k0 / kNB;
       __syncthreads();   // 1
       if (has_g) pg.store(s_g, LDK, tid);
-      if (DO_Q) pds.store(s_ds);   // only the dQc product reads dS
+      pds.store(s_ds);
       pdsu.store(s_dsu);
       if (k0 + kCK < kend) CASTLE_BQ2_LOAD_B(k0 + kCK);
       __syncthreads();   // 2
       const bool live = k0 <= i0w;
       frag<T> bdsu[2];
       if (live) {
-        constexpr int SB = LDS_ROWS ? 1 : 2;   // 16-key steps whose operand fragments are requested together
+        frag<T> bds[2], okt[2][NT], out[2][NT];   // the operand fragments of both 16-key steps are requested together
 #pragma unroll
-        for (int s0 = 0; s0 < 2; s0 += SB) {
-          frag<T> bds[SB], okt[SB][NT], out[SB][NT];
+        for (int s2 = 0; s2 < 2; ++s2) {
+          bdsu[s2] = ld_free<T, false>(s_dsu, LDD, jw, 1 << 30, 16 * s2, c, g);
+          bds[s2] = ld_free<T, false>(s_ds, LDD, jw, 1 << 30, 16 * s2, c, g);
 #pragma unroll
-          for (int u = 0; u < SB; ++u) {
-            const int s2 = s0 + u;
-            bdsu[s2] = ld_free<T, false>(s_dsu, LDD, jw, 1 << 30, 16 * s2, c, g);
-            if constexpr (DO_Q) {
-              bds[u] = ld_free<T, false>(s_ds, LDD, jw, 1 << 30, 16 * s2, c, g);
-#pragma unroll
-              for (int nt = 0; nt < NT; ++nt) {
-                okt[u][nt] = ld_free<T, false>(s_kc, LDK, 32 * nt, HD, 16 * s2, c, g);
-                out[u][nt] = ld_free<T, false>(s_ub, LDK, 32 * nt, HD, 16 * s2, c, g);
-              }
-            }
-          }
-          if constexpr (DO_Q) {
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int u = 0; u < SB; ++u)
-#pragma unroll
-              for (int nt = 0; nt < NT; ++nt) {
-                mma(dqc[nt], okt[u][nt], bds[u]);
-                if (Kb < blk0) mma(dqc[nt], out[u][nt], bdsu[s0 + u]);
-              }
+          for (int nt = 0; nt < NT; ++nt) {
+            okt[s2][nt] = ld_free<T, false>(s_kc, LDK, 32 * nt, HD, 16 * s2, c, g);
+            out[s2][nt] = ld_free<T, false>(s_ub, LDK, 32 * nt, HD, 16 * s2, c, g);
           }
         }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) {
+            mma(dqc[nt], okt[s2][nt], bds[s2]);
+            if (Kb < blk0) mma(dqc[nt], out[s2][nt], bdsu[s2]);
+          }
       }
       __syncthreads();   // 3
       if (!live) continue;
@@ -1998,19 +1937,15 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
           if (jt <= pw) oat[jt] = ld_nat<T>(s_at, LDA, 32 * jt + c, 16 * s2 + 8 * g);
         // dVu += G'^T A for the rows taken as sources: A^T[j][k] of this wave's own rows
         const frag<T> fa = ld_nat<T>(s_at, LDA, jw + c, 16 * s2 + 8 * g);
-        if constexpr (DO_S) {
 #pragma unroll
-          for (int nt = 0; nt < NT; ++nt)
-            ogt[nt] = has_g ? ld_free<T, false>(s_g, LDK, 32 * nt, HD, 16 * s2, c, g) : zero_frag<T>();
-        }
+        for (int nt = 0; nt < NT; ++nt)
+          ogt[nt] = has_g ? ld_free<T, false>(s_g, LDK, 32 * nt, HD, 16 * s2, c, g) : zero_frag<T>();
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int jt = 0; jt < PT; ++jt)
           if (jt <= pw) mma(dtacc[jt], oat[jt], bdsu[s2]);
-        if constexpr (DO_S) {
 #pragma unroll
-          for (int nt = 0; nt < NT; ++nt) mma(dvu[nt], ogt[nt], fa);   // ogt is zero where no reverse state exists
-        }
+        for (int nt = 0; nt < NT; ++nt) mma(dvu[nt], ogt[nt], fa);   // ogt is zero where no reverse state exists
       }
     }
 #undef CASTLE_BQ2_LOAD_B
@@ -2018,8 +1953,8 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
     __syncthreads();   // e1
     {
       RowStage<T, T, QB, HD, 2 * kThreads> st;
-      if (DO_Q) { st.load_flat(vu + (int64_t)qb * QB * HD); st.store(e_vu, LDK); }
-      if (DO_S) { st.load_flat(qc + (int64_t)qb * QB * HD); st.store(e_qc, LDK); }
+      st.load_flat(vu + (int64_t)qb * QB * HD); st.store(e_vu, LDK);
+      st.load_flat(qc + (int64_t)qb * QB * HD); st.store(e_qc, LDK);
     }
     // dT^T[j rows, i lanes] masked to j <= i, shared as dT[i][j] for the source-side product
 #pragma unroll
@@ -2027,39 +1962,379 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
 #pragma unroll
       for (int r = 0; r < 16; ++r)
         if (32 * jt + acc_row(r, g) > jw + c) dtacc[jt][r] = 0.f;
-      if constexpr (DO_S) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) st4<T>(e_dt + (jw + c) * LDT + 32 * jt + 8 * q + 4 * g, pack4<T>(dtacc[jt], q));
-      }
+      for (int q = 0; q < 4; ++q) st4<T>(e_dt + (jw + c) * LDT + 32 * jt + 8 * q + 4 * g, pack4<T>(dtacc[jt], q));
     }
     __syncthreads();   // e2
-    if constexpr (DO_Q) {
 #pragma unroll
-      for (int jt = 0; jt < PT; ++jt) {
-        if (jt > pw) continue;
+    for (int jt = 0; jt < PT; ++jt) {
+      if (jt > pw) continue;
 #pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2) {
-          const frag<T> fdt = chain<T>(dtacc[jt], s2);
+      for (int s2 = 0; s2 < 2; ++s2) {
+        const frag<T> fdt = chain<T>(dtacc[jt], s2);
 #pragma unroll
-          for (int nt = 0; nt < NT; ++nt)
-            mma(dqc[nt], ld_free<T, true>(e_vu, LDK, 32 * nt, HD, 32 * jt + 16 * s2, c, g), fdt);
+        for (int nt = 0; nt < NT; ++nt)
+          mma(dqc[nt], ld_free<T, true>(e_vu, LDK, 32 * nt, HD, 32 * jt + 16 * s2, c, g), fdt);
+      }
+    }
+#pragma unroll
+    for (int s = 0; s < PS; ++s) {
+      if (s < sfirst) continue;
+      // B operand: source j = jw + c on lanes, queries i = 16 s .. in natural order, from dT[i][j]
+      const frag<T> fdt = ld_free<T, false>(e_dt, LDT, jw, QB, 16 * s, c, g);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+        mma(dvu[nt], ld_free<T, false>(e_qc, LDK, 32 * nt, HD, 16 * s, c, g), fdt);
+    }
+    if (i < L) {
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqc, b, h) + (int64_t)i * a.dqc.sl, dqc, c0 * gun, g, a.s.rotary ? i : -1);
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvu, b, h) + (int64_t)i * a.dvu.sl, dvu, kLn2 * gun * vu_scale, g, a.s.rotary ? i : -1);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// The tile-consuming query-stationary backward for head dimensions above 64, in ONE launch.  Same
+// 128 rows per workgroup, same chunks of 32 keys and the same three barriers per chunk as
+// bwd_query2_kernel, but the outputs are dealt to the two waves of a pair so that neither holds
+// more than half a SIMD's registers:
+//   waves 0-3 (source rows j):  gate A, dA, dZ, dKu (all columns), dVu columns 0 .. 31 (the gate
+//                               operand of  dVu += G'^T A  comes straight from their registers)
+//   waves 4-7 (query rows i):   dQc (all columns), dT, dVu columns 32 .. d - 1
+// Every tile, snapshot and gate is read or formed once (two launches with half of the outputs each
+// read the dSu tiles, and formed the gate and dT, twice).
+template <typename T, int HD> constexpr int bwd_queryw_lds_bytes() {
+  int b = 4 * a16((int)sizeof(T) * kCK * lds_ld_tr<T>(HD));       // kc, qu, ub, g
+  b += a16((int)sizeof(T) * 128 * kLdA<T>);                       // A^T [j][k]
+  b += 2 * a16((int)sizeof(T) * kCK * kLdD<T>);                   // dS, dSu [k][i]
+  b += a16((int)sizeof(T) * 128 * kLdTT<T>) + a16((int)sizeof(T) * 128 * lds_ld_tr<T>(HD));   // T'^T and vu rows
+  int e = 2 * a16((int)sizeof(T) * 128 * lds_ld_tr<T>(HD)) + a16((int)sizeof(T) * 128 * kLdT2<T>);
+  return b > e ? b : e;
+}
+
+template <typename T, typename TI, int HD>
+__global__ __launch_bounds__(2 * kThreads, 2) void bwd_queryw_kernel(BwdArgs a) {
+  static_assert(sizeof(T) == 2 && kCK == 32 && HD > 64, "tile consumer for wide heads: 16-bit operands");
+  constexpr int KS = HD / 16;
+  constexpr int NT = HD / 32;
+  constexpr int NHA = 1, NHB = NT - NHA;   // dVu tiles of the source-row / query-row waves (what the registers of each allow)
+  constexpr int QB = 128;
+  constexpr int PT = QB / 32;    // 32-row tiles across the pair
+  constexpr int PS = QB / 16;    // 16-deep steps across the pair
+  constexpr int LDK = lds_ld_tr<T>(HD), LDT = kLdT2<T>, LDA = kLdA<T>, LDD = kLdD<T>, LDTT = kLdTT<T>;
+
+  Carver cv{castle_smem};
+  T* s_kc = cv.take<T>(kCK * LDK);
+  T* s_qu = cv.take<T>(kCK * LDK);
+  T* s_ub = cv.take<T>(kCK * LDK);   // lookahead state at the start of the pair
+  T* s_g = cv.take<T>(kCK * LDK);    // reverse state behind the pair
+  T* s_at = cv.take<T>(QB * LDA);    // gate, [source j][key k]
+  T* s_ds = cv.take<T>(kCK * LDD);   // dS,  [key k][query i]
+  T* s_dsu = cv.take<T>(kCK * LDD);  // dSu, [key k][query i]
+  T* s_tt = cv.take<T>(QB * LDTT);   // T'^T [source j][query i of the pair]
+  T* s_vu = cv.take<T>(QB * LDK);    // vu rows of the pair
+  // the epilogue reuses the same memory
+  Carver ce{castle_smem};
+  T* e_vu = ce.take<T>(QB * LDK);
+  T* e_qc = ce.take<T>(QB * LDK);
+  T* e_dt = ce.take<T>(QB * LDT);    // dT, [query i][source j] (pair local)
+
+  int rank, bh;
+  work_item(a.s.B * a.s.H, rank, bh);
+  const int qb = a.s.Lp / 128 - 1 - rank;   // the last row block meets the most keys
+  const int b = bh / a.s.H, h = bh % a.s.H;
+  const int lane = lane_id(), wave = wave_id(), c = lane & 31, g = lane >> 5;
+  const bool source_role = wave < 4;
+  const int pw = wave & 3;
+  const int tid = threadIdx.x & (kThreads - 1);   // thread index inside the role
+  const int L = a.s.L;
+  const float c0 = a.s.scale, c1 = a.s.scale * kLog2e;
+  const float gun = a.bhdr->grad_unscale, vu_scale = a.ws.hdr->vu_scale;
+  const int jw = 32 * pw;                     // rows of this wave pair inside the 128-row exchange tiles
+  const int i0w = qb * QB + jw;
+  const int i = i0w + c;                      // this lane's row
+  const int blk0 = 2 * qb, blk1 = 2 * qb + 1;
+  const int sfirst = jw / 16;                 // first step covering queries i >= j
+  const bool has_g = blk1 <= a.s.nblk - 2;    // a reverse state exists behind the pair
+
+  const T* qc = prep_ptr<T>(a.ws.qc_p, bh, a.s.Lp, HD);
+  const T* vu = prep_ptr<T>(a.ws.vu_p, bh, a.s.Lp, HD);
+  const T* usnap = reinterpret_cast<const T*>(a.ws.usnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
+  const T* gsnap = reinterpret_cast<const T*>(a.gsnap) + (int64_t)bh * snap_rows(a.s.nblk) * HD;
+  const T* ttb = reinterpret_cast<const T*>(a.ws.tt_blk) + (int64_t)bh * a.s.Lp * kNB;
+  const T* ttx = reinterpret_cast<const T*>(a.ws.ttx_blk) + (int64_t)bh * a.s.Lp * kNB;
+  const int64_t tile_row = (int64_t)(a.s.Lp / 32) * 1024;   // elements between the tiles of consecutive key groups
+  const T* dsm = reinterpret_cast<const T*>(a.ds_mat) + (int64_t)bh * a.s.Lp * a.s.Lp + (int64_t)qb * 4 * 1024;
+  const T* dsum = reinterpret_cast<const T*>(a.dsu_mat) + (int64_t)bh * a.s.Lp * a.s.Lp + (int64_t)qb * 4 * 1024;
+  int kend = qb * QB + QB;
+  if (kend > a.s.Lp) kend = a.s.Lp;
+  TileStage<T, true> pds, pdsu;   // every thread: one piece of each
+
+  {
+    // rows j of the pair: T'^T[j][i] over the pair's queries (own block from tt_blk; for the first
+    // block the second block's queries from the cross quarter), and vu_j.  Columns a row never
+    // uses (queries before its block) are left unwritten.
+    constexpr int VH = kNB / 8;   // 16-byte pieces per half row
+    for (int p = threadIdx.x; p < QB * 2 * VH; p += 2 * kThreads) {
+      const int j = p / (2 * VH), half = (p / VH) & 1, v = p % VH;
+      const bool first = j < kNB;
+      if (!first && half == 0) continue;
+      const T* src = (first && half == 1) ? ttx : ttb;
+      *reinterpret_cast<frag_mem<T>*>(s_tt + j * LDTT + half * kNB + v * 8) =
+          *reinterpret_cast<const frag_mem<T>*>(src + ((int64_t)qb * QB + j) * kNB + v * 8);
+    }
+    RowStage<T, T, QB, HD, 2 * kThreads> st;
+    st.load_flat(vu + (int64_t)qb * QB * HD);
+    st.store(s_vu, LDK);
+    // visible after the first barrier of the chunk loop; first used behind its third
+  }
+
+  if (source_role) {
+    const T* kc = prep_ptr<T>(a.ws.kc_p, bh, a.s.Lp, HD);
+    const T* qu = prep_ptr<T>(a.ws.qu_p, bh, a.s.Lp, HD);
+    const T* ku = prep_ptr<T>(a.ws.ku_p, bh, a.s.Lp, HD);
+    frag<T> fku[KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) fku[s] = ldg_nat_scaled<T, T>(ku, HD, i, 16 * s + 8 * g, true, -c1);
+    acc_t dku[NT];   // [n rows, j lanes]
+    acc_t dvu[NHA];   // [n rows, j lanes], columns 0 .. 31
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) zero(dku[nt]);
+#pragma unroll
+    for (int nt = 0; nt < NHA; ++nt) zero(dvu[nt]);
+
+    // this role stages kc, qu and its half of the dS / dSu tiles
+    RowStage<T, T, kCK, HD> pkc, pqu;
+#define CASTLE_BQW_LOAD_A(K0)                                     \
+  do {                                                            \
+    pkc.load_flat(kc + (int64_t)(K0) * HD, tid);                  \
+    pqu.load_flat(qu + (int64_t)(K0) * HD, tid);                  \
+    pds.load(dsm + (int64_t)((K0) / 32) * tile_row);              \
+    pdsu.load(dsum + (int64_t)((K0) / 32) * tile_row);            \
+  } while (0)
+    CASTLE_BQW_LOAD_A(0);
+    for (int k0 = 0; k0 < kend; k0 += kCK) {
+      __syncthreads();   // 1: tiles free
+      pkc.store(s_kc, LDK, tid);
+      pqu.store(s_qu, LDK, tid);
+      pds.store(s_ds);
+      pdsu.store(s_dsu);
+      if (k0 + kCK < kend) CASTLE_BQW_LOAD_A(k0 + kCK);   // in flight while this chunk is processed
+      __syncthreads();   // 2: tiles staged
+      const bool live = k0 <= i0w;   // the chunk's keys do not lie beyond this wave's rows
+      // gate tile A[k rows, j lanes] for this wave's 32 source rows, shared as A^T[j][k]
+      acc_t aK;
+      zero(aK);   // a constant operand of the first product where the chunk is live, registers of zeros where it is not
+      if (live) {
+        zero(aK);
+#pragma unroll
+        for (int s0 = 0; s0 < KS; s0 += 4) {   // operand fragments in batches of four
+          frag<T> oqu[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) oqu[u] = ld_nat<T>(s_qu, LDK, c, 16 * (s0 + u) + 8 * g);
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int u = 0; u < 4; ++u) mma(aK, oqu[u], fku[s0 + u]);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) aK[r] = fast_rcp(1.f + fast_exp2(aK[r]));
+        if (k0 + 31 >= i0w) {   // the tile reaches the diagonal: keep j > k only
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            if (i <= k0 + acc_row(r, g)) aK[r] = 0.f;
+        }
+      }
+      // a wave the chunk has passed still owes zeros: the later rows of the pair read its rows
+#pragma unroll
+      for (int q = 0; q < 4; ++q) st4<T>(s_at + (jw + c) * LDA + 8 * q + 4 * g, pack4<T>(aK, q));
+      __syncthreads();   // 3: gate shared
+      if (!live) continue;
+      // dA in two accumulators (two dependent MFMA chains instead of one)
+      acc_t dA, dA2;
+      zero(dA);
+      zero(dA2);
+#pragma unroll
+      for (int s0 = 0; s0 < PS; s0 += 2) {   // dSu^T T' and G' Vu^T, two steps of each at a time
+        frag<T> ods[2], ott[2], og[2], ovu[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          ods[u] = ld_nat<T>(s_dsu, LDD, c, 16 * (s0 + u) + 8 * g);
+          ott[u] = ld_nat<T>(s_tt, LDTT, jw + c, 16 * (s0 + u) + 8 * g);
+          og[u] = has_g ? ld_nat<T>(s_g, LDK, c, 16 * (s0 + u) + 8 * g) : zero_frag<T>();   // zero where no reverse state exists
+          ovu[u] = ld_nat<T>(s_vu, LDK, jw + c, 16 * (s0 + u) + 8 * g);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          if (s0 + u >= sfirst) mma(dA, ods[u], ott[u]);
+          mma(dA2, og[u], ovu[u]);
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dA[r] = (dA[r] + dA2[r]) * __builtin_fmaf(-aK[r], aK[r], aK[r]);   // dZ; A (1 - A) in one instruction
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {   // small batches of operand fragments: this role is at the register limit
+        const frag<T> fdz = chain<T>(dA, s2), fa = chain<T>(aK, s2);
+#pragma unroll
+        for (int n0 = 0; n0 < NT; n0 += 2) {
+          frag<T> oqt[2];
+#pragma unroll
+          for (int u = 0; u < 2; ++u) oqt[u] = ld_free<T, true>(s_qu, LDK, 32 * (n0 + u), HD, 16 * s2, c, g);
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int u = 0; u < 2; ++u) mma(dku[n0 + u], oqt[u], fdz);
+        }
+        frag<T> ogt[NHA];
+#pragma unroll
+        for (int nt = 0; nt < NHA; ++nt) ogt[nt] = has_g ? ld_free<T, true>(s_g, LDK, 32 * nt, HD, 16 * s2, c, g) : zero_frag<T>();
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int nt = 0; nt < NHA; ++nt) mma(dvu[nt], ogt[nt], fa);   // dVu += G'^T A; ogt is zero where no reverse state exists
+      }
+    }
+#undef CASTLE_BQW_LOAD_A
+    // ---- epilogue: dvu += dT^T Qc' for this role's columns ------------------------------------
+    __syncthreads();   // e1: chunk tiles dead
+    {
+      RowStage<T, T, QB, HD, 2 * kThreads> st;
+      st.load_flat(vu + (int64_t)qb * QB * HD); st.store(e_vu, LDK);
+      st.load_flat(qc + (int64_t)qb * QB * HD); st.store(e_qc, LDK);
+    }
+    __syncthreads();   // e2: epilogue tiles and dT shared
+#pragma unroll
+    for (int s = 0; s < PS; ++s) {
+      if (s < sfirst) continue;
+      // B operand: source j = jw + c on lanes, queries i = 16 s .. in natural order, from dT[i][j]
+      const frag<T> fdt = ld_free<T, false>(e_dt, LDT, jw, QB, 16 * s, c, g);
+#pragma unroll
+      for (int nt = 0; nt < NHA; ++nt)
+        mma(dvu[nt], ld_free<T, false>(e_qc, LDK, 32 * nt, HD, 16 * s, c, g), fdt);
+    }
+    if (i < L) {
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dku, b, h) + (int64_t)i * a.dku.sl, dku, c0 * kLn2 * gun, g, a.s.rotary ? i : -1);
+      store_rows<TI, HD, NHA>(head_ptr_mut<TI>(a.dvu, b, h) + (int64_t)i * a.dvu.sl, dvu, kLn2 * gun * vu_scale, g, a.s.rotary ? i : -1, 0);
+    }
+  } else {
+    acc_t dqc[NT];      // [n rows, i lanes]
+    acc_t dvu[NHB];      // [n rows, j lanes], columns 32 .. HD - 1: this role's rows taken as lookahead sources
+    acc_t dtacc[PT];    // [j rows (pair local), i lanes]
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) zero(dqc[nt]);
+#pragma unroll
+    for (int nt = 0; nt < NHB; ++nt) zero(dvu[nt]);
+#pragma unroll
+    for (int jt = 0; jt < PT; ++jt) zero(dtacc[jt]);
+    // this role stages the two states and its half of the dS / dSu tiles
+    SnapStage<T, kCK, HD> pu, pg;
+#define CASTLE_BQW_LOAD_B(K0)                                                          \
+  do {                                                                                 \
+    if ((K0) / kNB < blk0) pu.load(usnap + (usnap_off(blk0) + (K0)) * HD, tid);        \
+    if (has_g) pg.load(gsnap + (gsnap_off(blk1) + (K0)) * HD, tid);                    \
+    pds.load(dsm + (int64_t)((K0) / 32) * tile_row);                                   \
+    pdsu.load(dsum + (int64_t)((K0) / 32) * tile_row);                                 \
+  } while (0)
+    CASTLE_BQW_LOAD_B(0);
+    for (int k0 = 0; k0 < kend; k0 += kCK) {
+      const int Kb = k0 / kNB;
+      __syncthreads();   // 1
+      if (Kb < blk0) pu.store(s_ub, LDK, tid);
+      if (has_g) pg.store(s_g, LDK, tid);
+      pds.store(s_ds);
+      pdsu.store(s_dsu);
+      if (k0 + kCK < kend) CASTLE_BQW_LOAD_B(k0 + kCK);
+      __syncthreads();   // 2
+      const bool live = k0 <= i0w;
+      frag<T> bdsu[2];
+      if (live) {
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {   // one 16-key step at a time keeps the operand registers few
+          bdsu[s2] = ld_free<T, false>(s_dsu, LDD, jw, 1 << 30, 16 * s2, c, g);
+          const frag<T> bds = ld_free<T, false>(s_ds, LDD, jw, 1 << 30, 16 * s2, c, g);
+#pragma unroll
+          for (int n0 = 0; n0 < NT; n0 += 2) {
+            frag<T> okt[2], out[2];
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+              okt[u] = ld_free<T, false>(s_kc, LDK, 32 * (n0 + u), HD, 16 * s2, c, g);
+              out[u] = ld_free<T, false>(s_ub, LDK, 32 * (n0 + u), HD, 16 * s2, c, g);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+              mma(dqc[n0 + u], okt[u], bds);
+              if (Kb < blk0) mma(dqc[n0 + u], out[u], bdsu[s2]);
+            }
+          }
+        }
+      }
+      __syncthreads();   // 3
+      if (!live) continue;
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {   // two small batches of operand fragments: this role is at the register limit
+        {
+          frag<T> oat[PT];
+#pragma unroll
+          for (int jt = 0; jt < PT; ++jt)
+            if (jt <= pw) oat[jt] = ld_nat<T>(s_at, LDA, 32 * jt + c, 16 * s2 + 8 * g);
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int jt = 0; jt < PT; ++jt)
+            if (jt <= pw) mma(dtacc[jt], oat[jt], bdsu[s2]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        {
+          // dVu += G'^T A for the rows taken as sources: A^T[j][k] of this wave's own rows
+          frag<T> ogt[NHB];
+          const frag<T> fa = ld_nat<T>(s_at, LDA, jw + c, 16 * s2 + 8 * g);
+#pragma unroll
+          for (int nt = 0; nt < NHB; ++nt)
+            ogt[nt] = has_g ? ld_free<T, false>(s_g, LDK, 32 * (NHA + nt), HD, 16 * s2, c, g) : zero_frag<T>();
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int nt = 0; nt < NHB; ++nt) mma(dvu[nt], ogt[nt], fa);   // ogt is zero where no reverse state exists
         }
       }
     }
-    if constexpr (DO_S) {
+#undef CASTLE_BQW_LOAD_B
+    // ---- epilogue: dT = tril(dTacc) over the pair:  dqc += dT Vu,  dvu += dT^T Qc' ------------
+    __syncthreads();   // e1
+    {
+      RowStage<T, T, QB, HD, 2 * kThreads> st;
+      st.load_flat(vu + (int64_t)qb * QB * HD); st.store(e_vu, LDK);
+      st.load_flat(qc + (int64_t)qb * QB * HD); st.store(e_qc, LDK);
+    }
+    // dT^T[j rows, i lanes] masked to j <= i, shared as dT[i][j] for the source-side product
 #pragma unroll
-      for (int s = 0; s < PS; ++s) {
-        if (s < sfirst) continue;
-        // B operand: source j = jw + c on lanes, queries i = 16 s .. in natural order, from dT[i][j]
-        const frag<T> fdt = ld_free<T, false>(e_dt, LDT, jw, QB, 16 * s, c, g);
+    for (int jt = 0; jt < PT; ++jt) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        if (32 * jt + acc_row(r, g) > jw + c) dtacc[jt][r] = 0.f;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) st4<T>(e_dt + (jw + c) * LDT + 32 * jt + 8 * q + 4 * g, pack4<T>(dtacc[jt], q));
+    }
+    __syncthreads();   // e2
+#pragma unroll
+    for (int jt = 0; jt < PT; ++jt) {
+      if (jt > pw) continue;
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        const frag<T> fdt = chain<T>(dtacc[jt], s2);
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
-          mma(dvu[nt], ld_free<T, false>(e_qc, LDK, 32 * nt, HD, 16 * s, c, g), fdt);
+          mma(dqc[nt], ld_free<T, true>(e_vu, LDK, 32 * nt, HD, 32 * jt + 16 * s2, c, g), fdt);
       }
     }
+#pragma unroll
+    for (int s = 0; s < PS; ++s) {
+      if (s < sfirst) continue;
+      const frag<T> fdt = ld_free<T, false>(e_dt, LDT, jw, QB, 16 * s, c, g);
+#pragma unroll
+      for (int nt = 0; nt < NHB; ++nt)
+        mma(dvu[nt], ld_free<T, false>(e_qc, LDK, 32 * (NHA + nt), HD, 16 * s, c, g), fdt);
+    }
     if (i < L) {
-      if constexpr (DO_Q) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqc, b, h) + (int64_t)i * a.dqc.sl, dqc, c0 * gun, g, a.s.rotary ? i : -1);
-      if constexpr (DO_S) store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dvu, b, h) + (int64_t)i * a.dvu.sl, dvu, kLn2 * gun * vu_scale, g, a.s.rotary ? i : -1);
+      store_rows<TI, HD, NT>(head_ptr_mut<TI>(a.dqc, b, h) + (int64_t)i * a.dqc.sl, dqc, c0 * gun, g, a.s.rotary ? i : -1);
+      store_rows<TI, HD, NHB>(head_ptr_mut<TI>(a.dvu, b, h) + (int64_t)i * a.dvu.sl, dvu, kLn2 * gun * vu_scale, g, a.s.rotary ? i : -1, NHA);
     }
   }
 }
@@ -2090,21 +2365,18 @@ template <typename T, typename TI, int HD> static int launch_bwd_t(const BwdArgs
     bool& configured2 = once2.flag();
     if (!configured2) {
       if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_key2_kernel<T, TI, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_key2_lds_bytes<T, HD>()) != hipSuccess) return -3;
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_query2_kernel<T, TI, HD, 0>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_query2_lds_bytes<T, HD>()) != hipSuccess) return -3;
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_query2_kernel<T, TI, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_query2_lds_bytes<T, HD>()) != hipSuccess) return -3;
       configured2 = true;
     }
-  } else if constexpr (TILES) {
-    static_assert(bwd_query2_lds_bytes<T, HD>() <= kMaxLds, "tile consumer does not fit the LDS");
+  } else if constexpr (TILES) {   // 16-bit tensors at d = 128: the two-role kernels for wide heads
+    static_assert(bwd_queryw_lds_bytes<T, HD>() <= kMaxLds, "wide-head query kernel does not fit the LDS");
+    static_assert(bwd_keyw1_lds_bytes<T, HD>() <= kMaxLds && bwd_keyw2_lds_bytes<T, HD>() <= kMaxLds, "wide-head key kernels do not fit the LDS");
     static PerDeviceOnce once3;
     bool& configured3 = once3.flag();
     if (!configured3) {
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_query2_kernel<T, TI, HD, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_query2_lds_bytes<T, HD>()) != hipSuccess) return -3;
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_query2_kernel<T, TI, HD, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_query2_lds_bytes<T, HD>()) != hipSuccess) return -3;
-      if constexpr (SPLIT) {
-        static_assert(bwd_keyw1_lds_bytes<T, HD>() <= kMaxLds && bwd_keyw2_lds_bytes<T, HD>() <= kMaxLds, "wide-head key kernels do not fit the LDS");
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_keyw1_kernel<T, TI, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_keyw1_lds_bytes<T, HD>()) != hipSuccess) return -3;
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_keyw2_kernel<T, TI, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_keyw2_lds_bytes<T, HD>()) != hipSuccess) return -3;
-      }
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_queryw_kernel<T, TI, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_queryw_lds_bytes<T, HD>()) != hipSuccess) return -3;
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_keyw1_kernel<T, TI, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_keyw1_lds_bytes<T, HD>()) != hipSuccess) return -3;
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_keyw2_kernel<T, TI, HD>), hipFuncAttributeMaxDynamicSharedMemorySize, bwd_keyw2_lds_bytes<T, HD>()) != hipSuccess) return -3;
       configured3 = true;
     }
   }
@@ -2153,12 +2425,12 @@ template <typename T, typename TI, int HD> static int launch_bwd_t(const BwdArgs
     bool done = false;
     if constexpr (TILES) {
       if (a.ds_mat != nullptr) {   // the key kernel left the dS / dSu tiles
-        constexpr int query2_lds = bwd_query2_lds_bytes<T, HD>();
         if constexpr (SPLIT) {
-          hipLaunchKernelGGL((bwd_query2_kernel<T, TI, HD, 1>), grid, dim3(2 * kThreads), query2_lds, stream, a);
-          hipLaunchKernelGGL((bwd_query2_kernel<T, TI, HD, 2>), grid, dim3(2 * kThreads), query2_lds, stream, a);
+          constexpr int queryw_lds = bwd_queryw_lds_bytes<T, HD>();
+          hipLaunchKernelGGL((bwd_queryw_kernel<T, TI, HD>), grid, dim3(2 * kThreads), queryw_lds, stream, a);
         } else {
-          hipLaunchKernelGGL((bwd_query2_kernel<T, TI, HD, 0>), grid, dim3(2 * kThreads), query2_lds, stream, a);
+          constexpr int query2_lds = bwd_query2_lds_bytes<T, HD>();
+          hipLaunchKernelGGL((bwd_query2_kernel<T, TI, HD>), grid, dim3(2 * kThreads), query2_lds, stream, a);
         }
         done = true;
       }

@@ -33,10 +33,10 @@ extern __shared__ __attribute__((aligned(16))) unsigned char castle_smem[];
 // value tile of the scan / attention kernels: 16-bit operands keep it row-major and read it with
 // transpose loads, fp32 stores it transposed
 template <typename T, int HD> constexpr int vtile_elems() {
-  return sizeof(T) == 2 ? kNB * lds_ld<T>(HD) : (HD < 32 ? 32 : HD) * lds_ld_chain<T>(kNB);
+  return sizeof(T) == 2 ? kNB * lds_ld_tr<T>(HD) : (HD < 32 ? 32 : HD) * lds_ld_chain<T>(kNB);
 }
 template <typename T, int HD> constexpr int scan_lds_bytes() {
-  return (int)sizeof(T) * (kNB * lds_ld<T>(HD) + vtile_elems<T, HD>());
+  return (int)sizeof(T) * (kNB * lds_ld_tr<T>(HD) + vtile_elems<T, HD>());
 }
 // keys per chunk of the attention kernel: 32 for 16-bit operands from d = 64 up.  At d = 128 the smaller
 // tiles and staging registers are what lets two workgroups share a CU (two waves per SIMD instead of
@@ -46,7 +46,7 @@ template <typename T, int HD> constexpr int attn_chunk() { return sizeof(T) == 2
 template <typename T, int HD> constexpr bool attn_t_in_lds() { return sizeof(T) == 2 && HD == 128; }
 template <typename T, int HD> constexpr int attn_lds_bytes() {
   constexpr int CK = attn_chunk<T, HD>();
-  return (int)sizeof(T) * (4 * CK * lds_ld<T>(HD) + (sizeof(T) == 2 ? CK * lds_ld<T>(HD) : vtile_elems<T, HD>()) + CK * lds_ld<T>(128) +
+  return (int)sizeof(T) * (4 * CK * lds_ld_tr<T>(HD) + (sizeof(T) == 2 ? CK * lds_ld_tr<T>(HD) : vtile_elems<T, HD>()) + CK * lds_ld<T>(128) +
                            (attn_t_in_lds<T, HD>() ? 128 * lds_ld<T>(kNB) : 0));
 }
 // register prefetch of the next tile is affordable for 16-bit operands up to d = 64
@@ -204,7 +204,7 @@ __global__ __launch_bounds__(kThreads, (scan_waves_per_simd<T, HD>())) void scan
   constexpr int HDP = HD < 32 ? 32 : HD;
   constexpr int NT = HDP / 32;
   constexpr int JT = kNB / 32;
-  constexpr int LDK = lds_ld<T>(HD), LDV = lds_ld_chain<T>(kNB);
+  constexpr int LDK = lds_ld_tr<T>(HD), LDV = lds_ld_chain<T>(kNB);
   constexpr bool PF = use_prefetch<T, HD>();
   T* s_ku = reinterpret_cast<T*>(castle_smem);   // [kNB][LDK]
   T* s_vut = s_ku + kNB * LDK;                   // fp32: [HDP][LDV] (transposed); 16-bit: [kNB][LDK]
@@ -327,7 +327,7 @@ __global__ __launch_bounds__(kThreads, sizeof(T) == 2 ? 2 : 1) void attn_kernel(
   constexpr int KT = CK / 32;
   constexpr int QB = 128;
   constexpr int NBLK_Q = QB / kNB;   // snapshot blocks per workgroup
-  constexpr int LDK = lds_ld<T>(HD), LDV = lds_ld_chain<T>(kNB), LDA = lds_ld<T>(QB);
+  constexpr int LDK = lds_ld_tr<T>(HD), LDV = lds_ld_chain<T>(kNB), LDA = lds_ld<T>(QB);
   constexpr bool PF = use_prefetch<T, HD>();
   constexpr bool TRV = sizeof(T) == 2;
   T* s_kc = reinterpret_cast<T*>(castle_smem);   // [CK][LDK]

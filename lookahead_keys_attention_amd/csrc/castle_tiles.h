@@ -53,6 +53,12 @@ template <> struct elem_traits<float> { static constexpr int vec16 = 4; };
 
 // padded leading dimension of an LDS tile with `cols` payload columns (16 bytes of pad)
 template <typename T> __host__ __device__ constexpr int lds_ld(int cols) { return cols + elem_traits<T>::vec16; }
+// The same for a 16-bit tile that is also read with transpose reads (ds_read_b64_tr_b16): on rows 132 or 136
+// elements apart such a read takes 48 cycles instead of 26 (measured; 40 ... 152 otherwise all take 26, and
+// 16-byte reads are slow only at 48, 80 and 144), so a 128-column tile gets rows of 152.
+template <typename T> __host__ __device__ constexpr int lds_ld_tr(int cols) {
+  return sizeof(T) == 2 && cols == 128 ? 152 : lds_ld<T>(cols);
+}
 
 __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
 // The wave index is read through readfirstlane so that the compiler knows it is uniform:
