@@ -67,6 +67,7 @@ BWD_CASES = [
     (1, 2, 300, 32, torch.bfloat16), (1, 2, 256, 16, torch.bfloat16), (1, 2, 256, 64, torch.float16),
     (1, 2, 300, 128, torch.bfloat16), (1, 1, 130, 128, torch.float16),
     (1, 3, 129, 16, torch.bfloat16), (3, 1, 448, 64, torch.float16), (1, 9, 640, 64, torch.bfloat16),
+    (2, 3, 709, 128, torch.bfloat16),
 ]
 
 
@@ -136,16 +137,18 @@ def test_rope_entry_point_matches_formula():
         assert (out.double().cpu() - want).abs().max() <= tol
 
 
-def test_backward_without_score_tiles(monkeypatch):
+@pytest.mark.parametrize("d", [64, 128])
+def test_backward_without_score_tiles(d, monkeypatch):
     """Long sequences do not get the dS / dSu tile buffers (they grow with L^2); the second backward
-    kernel then recomputes the score chain.  Forced here through FLAG_RECOMPUTE_SCORES."""
+    kernel then recomputes the score chain (at d = 128 both single-role kernels run, in two passes
+    each).  Forced here through FLAG_RECOMPUTE_SCORES."""
     from lookahead_keys_attention_amd import _native
 
-    small = _native.lib().castle_bwd_workspace_bytes(2, 2, 300, 64, 1, _native.FLAG_RECOMPUTE_SCORES)
-    assert small < _native.lib().castle_bwd_workspace_bytes(2, 2, 300, 64, 1, 0)
+    small = _native.lib().castle_bwd_workspace_bytes(2, 2, 300, d, 1, _native.FLAG_RECOMPUTE_SCORES)
+    assert small < _native.lib().castle_bwd_workspace_bytes(2, 2, 300, d, 1, 0)
     monkeypatch.setattr(H(), "DEFAULT_FLAGS", _native.FLAG_RECOMPUTE_SCORES)
-    ops, dout = rand_ops(2, 2, 300, 64, torch.bfloat16, seed=77)
-    s = 64 ** -0.5
+    ops, dout = rand_ops(2, 2, 300, d, torch.bfloat16, seed=77)
+    s = d ** -0.5
     leaves = [t.to(DEV).requires_grad_() for t in ops]
     H().castle_attention_hip(*leaves, s).backward(dout.to(DEV))
     ref = O.closed_form_grads(*[t.double() for t in ops], s, dout.double())
