@@ -1995,8 +1995,8 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
 
 // ---------------------------------------------------------------------------
 // The tile-consuming query-stationary backward for head dimensions above 64, in ONE launch.  Same
-// 128 rows per workgroup, same chunks of 32 keys and the same three barriers per chunk as
-// bwd_query2_kernel, but the outputs are dealt to the two waves of a pair so that neither holds
+// 128 rows per workgroup and same chunks of 32 keys as bwd_query2_kernel, but two barriers per chunk
+// (the gate is computed ahead of the second), and the outputs are dealt to the two waves of a pair so that neither holds
 // more than half a SIMD's registers:
 //   waves 0-3 (source rows j):  gate A, dA, dZ, dKu (all columns), dVu columns 0 .. 31 (the gate
 //                               operand of  dVu += G'^T A  comes straight from their registers)
@@ -2004,7 +2004,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_query2_kernel(BwdArgs a) 
 // Every tile, snapshot and gate is read or formed once (two launches with half of the outputs each
 // read the dSu tiles, and formed the gate and dT, twice).
 template <typename T, int HD> constexpr int bwd_queryw_lds_bytes() {
-  int b = 4 * a16((int)sizeof(T) * kCK * lds_ld_tr<T>(HD));       // kc, qu, ub, g
+  int b = 5 * a16((int)sizeof(T) * kCK * lds_ld_tr<T>(HD));       // kc, qu (two chunks), ub, g
   b += a16((int)sizeof(T) * 128 * kLdA<T>);                       // A^T [j][k]
   b += 2 * a16((int)sizeof(T) * kCK * kLdD<T>);                   // dS, dSu [k][i]
   b += a16((int)sizeof(T) * 128 * kLdTT<T>) + a16((int)sizeof(T) * 128 * lds_ld_tr<T>(HD));   // T'^T and vu rows
@@ -2025,7 +2025,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_queryw_kernel(BwdArgs a) 
 
   Carver cv{castle_smem};
   T* s_kc = cv.take<T>(kCK * LDK);
-  T* s_qu = cv.take<T>(kCK * LDK);
+  T* s_qu2 = cv.take<T>(2 * kCK * LDK);   // qu rows of a chunk, chunk n in buffer n & 1: staged one chunk ahead (see the source-row waves)
   T* s_ub = cv.take<T>(kCK * LDK);   // lookahead state at the start of the pair
   T* s_g = cv.take<T>(kCK * LDK);    // reverse state behind the pair
   T* s_at = cv.take<T>(QB * LDA);    // gate, [source j][key k]
@@ -2103,24 +2103,29 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_queryw_kernel(BwdArgs a) 
 #pragma unroll
     for (int nt = 0; nt < NHA; ++nt) zero(dvu[nt]);
 
-    // this role stages kc, qu and its half of the dS / dSu tiles
+    // This role stages kc, qu and its half of the dS / dSu tiles.  The qu rows run one chunk ahead of the
+    // rest (two LDS buffers): the gate of a chunk then needs nothing that is staged in that chunk, and
+    // is computed between barriers 1 and 2, while the partner waves are still held up requesting their
+    // snapshot rows - two barriers per chunk instead of three, and no wave idles behind barrier 1.
     RowStage<T, T, kCK, HD> pkc, pqu;
-#define CASTLE_BQW_LOAD_A(K0)                                     \
-  do {                                                            \
-    pkc.load_flat(kc + (int64_t)(K0) * HD, tid);                  \
-    pqu.load_flat(qu + (int64_t)(K0) * HD, tid);                  \
-    pds.load(dsm + (int64_t)((K0) / 32) * tile_row);              \
-    pdsu.load(dsum + (int64_t)((K0) / 32) * tile_row);            \
+#define CASTLE_BQW_LOAD_A(K0)                                                       \
+  do {                                                                              \
+    pkc.load_flat(kc + (int64_t)(K0) * HD, tid);                                    \
+    if ((K0) + kCK < kend) pqu.load_flat(qu + (int64_t)((K0) + kCK) * HD, tid);     \
+    pds.load(dsm + (int64_t)((K0) / 32) * tile_row);                                \
+    pdsu.load(dsum + (int64_t)((K0) / 32) * tile_row);                              \
   } while (0)
+    pqu.load_flat(qu, tid);
+    pqu.store(s_qu2, LDK, tid);   // chunk 0: visible behind the first barrier
     CASTLE_BQW_LOAD_A(0);
     for (int k0 = 0; k0 < kend; k0 += kCK) {
+      const T* s_qu = s_qu2 + ((k0 / kCK) & 1) * kCK * LDK;
       __syncthreads();   // 1: tiles free
       pkc.store(s_kc, LDK, tid);
-      pqu.store(s_qu, LDK, tid);
+      if (k0 + kCK < kend) pqu.store(s_qu2 + (((k0 / kCK) & 1) ^ 1) * kCK * LDK, LDK, tid);
       pds.store(s_ds);
       pdsu.store(s_dsu);
       if (k0 + kCK < kend) CASTLE_BQW_LOAD_A(k0 + kCK);   // in flight while this chunk is processed
-      __syncthreads();   // 2: tiles staged
       const bool live = k0 <= i0w;   // the chunk's keys do not lie beyond this wave's rows
       // gate tile A[k rows, j lanes] for this wave's 32 source rows, shared as A^T[j][k]
       acc_t aK;
@@ -2147,7 +2152,7 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_queryw_kernel(BwdArgs a) 
       // a wave the chunk has passed still owes zeros: the later rows of the pair read its rows
 #pragma unroll
       for (int q = 0; q < 4; ++q) st4<T>(s_at + (jw + c) * LDA + 8 * q + 4 * g, pack4<T>(aK, q));
-      __syncthreads();   // 3: gate shared
+      __syncthreads();   // 2: tiles staged, gate shared
       if (!live) continue;
       // dA in two accumulators (two dependent MFMA chains instead of one)
       acc_t dA, dA2;
@@ -2267,7 +2272,6 @@ __global__ __launch_bounds__(2 * kThreads, 2) void bwd_queryw_kernel(BwdArgs a) 
           }
         }
       }
-      __syncthreads();   // 3
       if (!live) continue;
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {   // two small batches of operand fragments: this role is at the register limit
